@@ -1,0 +1,183 @@
+"""The engine against the plain implementation, in 32-bit and in bfloat16, under
+every way of cutting the work: whole requests; most of a request in one step and
+the last 32 tokens one by one; portions of changing size; and mixed steps of up
+to four live requests on so few pages that they are used again.
+
+Tolerances, fixed beforehand (relative to the largest logit magnitude of the
+request): 32-bit 1e-4 (accumulation order over a few layers); bfloat16 2.5e-2
+(about 40 roundings of 2^-9 along the path, worst entry of thousands).
+"""
+
+import math
+
+import pytest
+import torch
+
+import engine_util as eu
+import plain_lfm2 as plain
+from tiny_configs import TINY_A, TINY_B, TINY_C
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"float32": 1e-4, "bfloat16": 2.5e-2}
+CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
+LENGTHS = {"A": [5, 17, 33, 70], "B": [1, 8, 31, 64, 100], "C": [40, 3, 77]}
+
+_cache = {}
+
+
+def setup(name: str, dtype: str):
+    """(runner factory, plain logits per request, prompts)."""
+    key = (name, dtype)
+    if key not in _cache:
+        from zig_ai_amd.engine import DecoderModel
+        cfg, seed = CONFIGS[name]
+        store = torch.float32 if dtype == "float32" else torch.bfloat16
+        folder = eu.model_folder(cfg, seed, store, **eu.sharp_kwargs())
+        model = DecoderModel.from_folder(folder, dtype)
+        oracle = plain.PlainLfm2(folder)
+        prompts = [eu.random_tokens(n, cfg["vocab_size"], 100 + i) for i, n in enumerate(LENGTHS[name])]
+        expect = [oracle.logits(p) for p in prompts]
+        _cache[key] = (model, expect, prompts)
+    return _cache[key]
+
+
+def runner_for(model, page_size, num_pages, num_slots=4):
+    from zig_ai_amd.engine import ModelRunner
+    return ModelRunner(model, page_size=page_size, num_pages=num_pages, num_slots=num_slots)
+
+
+def check(got, expect, dtype, what):
+    for i, (g, e) in enumerate(zip(got, expect)):
+        err = eu.rel_err(g, e)
+        assert err < TOL[dtype], f"{what}: request {i} off by {err:.3e} (allowed {TOL[dtype]:.1e})"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_whole_requests(name, dtype):
+    model, expect, prompts = setup(name, dtype)
+    runner = runner_for(model, 16, 16)
+    got = eu.run_schedule(runner, prompts, eu.whole(LENGTHS[name]))
+    check(got, expect, dtype, "whole")
+    assert runner.cache.stats()["requests"] == 0
+    assert all(g["pages_free"] == g["pages"] for g in runner.cache.stats()["groups"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_bulk_then_last_32_one_by_one(name, dtype):
+    model, expect, prompts = setup(name, dtype)
+    runner = runner_for(model, 4 if name == "A" else 8, 64)
+    got = eu.run_schedule(runner, prompts, eu.bulk_then_single(LENGTHS[name], 32))
+    check(got, expect, dtype, "bulk+tail")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_portions_of_changing_size(name, dtype):
+    model, expect, prompts = setup(name, dtype)
+    for seed in (0, 3):
+        runner = runner_for(model, 8 if name == "B" else 4, 64)
+        got = eu.run_schedule(runner, prompts, eu.changing_portions(LENGTHS[name], seed))
+        check(got, expect, dtype, f"portions seed {seed}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_mixed_steps_with_page_reuse(name, dtype):
+    model, expect, prompts = setup(name, dtype)
+    # the same requests twice over, so that late ones land on pages early ones used
+    lengths = LENGTHS[name] * 2
+    prompts2, expect2 = prompts * 2, expect * 2
+    page = 4
+    for seed in (1, 2):
+        schedule = eu.mixed(lengths, seed=seed, max_live=4 if seed == 1 else 3)
+        pages = eu.peak_tokens(lengths, schedule, round_to=page) // page
+        runner = runner_for(model, page, pages, num_slots=4)
+        got = eu.run_schedule(runner, prompts2, schedule)
+        check(got, expect2, dtype, f"mixed seed {seed}")
+        stats = runner.cache.stats()
+        assert stats["pages_reused"] > 0, "the pool was too large to reuse a page"
+        assert stats["slots_high_water"] <= 4
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_cuts_agree_with_each_other(dtype):
+    """The engine against itself: a different cut changes rounding only."""
+    model, _, prompts = setup("B", dtype)
+    a = eu.run_schedule(runner_for(model, 8, 64), prompts, eu.whole(LENGTHS["B"]))
+    b = eu.run_schedule(runner_for(model, 8, 64), prompts, eu.changing_portions(LENGTHS["B"], 5))
+    tol = 2e-5 if dtype == "float32" else TOL["bfloat16"]
+    for x, y in zip(a, b):
+        assert eu.rel_err(y, x.double()) < tol
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(dtype):
+    """300 tokens one by one after a short prompt: positions far beyond a page,
+    a tile and a split of the attention kernel."""
+    from zig_ai_amd.engine import StepEntry
+    model, _, _ = setup("A", dtype)
+    cfg, seed = CONFIGS["A"]
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    oracle = plain.PlainLfm2(eu.model_folder(cfg, seed, store, **eu.sharp_kwargs()))
+    tokens = eu.random_tokens(7 + 300, cfg["vocab_size"], 55)
+    expect = oracle.logits(tokens)
+    runner = runner_for(model, 16, 32)
+    runner.admit("r")
+    got = [runner.step([StepEntry("r", tokens[:7], list(range(7)))]).cpu()]
+    for p in range(7, len(tokens)):
+        got.append(runner.step([StepEntry("r", tokens[p:p + 1], [0])]).cpu())
+    assert eu.rel_err(torch.cat(got), expect) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens(dtype):
+    """The very first positions: one token alone, two, three (shorter than the
+    convolution), each as its own request."""
+    model, _, _ = setup("B", dtype)
+    cfg, seed = CONFIGS["B"]
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    oracle = plain.PlainLfm2(eu.model_folder(cfg, seed, store, **eu.sharp_kwargs()))
+    prompts = [[7], [7, 300], [9, 9, 9], [511, 0, 1, 2]]
+    lengths = [len(p) for p in prompts]
+    expect = [oracle.logits(p) for p in prompts]
+    got = eu.run_schedule(runner_for(model, 8, 8), prompts, eu.whole(lengths))
+    check(got, expect, dtype, "first tokens")
+    got = eu.run_schedule(runner_for(model, 8, 8), prompts,
+                          eu.changing_portions(lengths, 0, sizes=(1,)))
+    check(got, expect, dtype, "first tokens one by one")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_wanted_rows_only(dtype):
+    """Logits come back only for the wanted places, in the order asked."""
+    from zig_ai_amd.engine import StepEntry
+    model, expect, prompts = setup("A", dtype)
+    runner = runner_for(model, 4, 64)
+    for i in (1, 2):
+        runner.admit(i)
+    out = runner.step([StepEntry(1, prompts[1], [16, 0]), StepEntry(2, prompts[2], []),
+                       ]).cpu()
+    assert out.shape == (2, TINY_A["vocab_size"])
+    assert eu.rel_err(out, expect[1][[16, 0]]) < TOL[dtype]
+    none = runner.step([StepEntry(1, [3], [])])
+    assert none.shape == (0, TINY_A["vocab_size"])
+
+
+def test_step_errors():
+    from zig_ai_amd.cache import OutOfPages
+    from zig_ai_amd.engine import StepEntry, StepError
+    model, _, prompts = setup("A", "float32")
+    runner = runner_for(model, 4, 4)
+    runner.admit("a")
+    with pytest.raises(StepError, match="vocabulary"):
+        runner.step([StepEntry("a", [256], [0])])
+    with pytest.raises(StepError, match="not admitted"):
+        runner.step([StepEntry("b", [1], [0])])
+    with pytest.raises(StepError, match="twice"):
+        runner.step([StepEntry("a", [1], [0]), StepEntry("a", [2], [0])])
+    with pytest.raises(OutOfPages):
+        runner.step([StepEntry("a", list(range(17)), [0])])
+    runner.cache.check()

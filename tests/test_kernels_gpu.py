@@ -1,0 +1,518 @@
+"""Each HIP kernel alone against the plain formulas of tests/plain_lfm2.py, at
+sizes other than the engine's (odd widths, tails in every dimension, head sizes
+from 16 to 256, any group size).
+
+Tolerances, fixed beforehand: a kernel computing in 32-bit must agree with the
+float64 formula to 2e-5 of the result's largest magnitude (accumulation order);
+a kernel that stores bfloat16 adds one rounding of the stored value, 2^-8
+relative, so 6e-3 of the largest magnitude.
+"""
+
+import math
+
+import pytest
+import torch
+
+import plain_lfm2 as plain
+
+pytestmark = pytest.mark.gpu
+
+F32_TOL = 2e-5
+BF16_TOL = 6e-3
+
+
+def dev():
+    return torch.device("cuda", 0)
+
+
+def ops():
+    from zig_ai_amd.kernels import ops as _ops
+    return _ops
+
+
+def rel_err(actual: torch.Tensor, expected: torch.Tensor) -> float:
+    a = actual.detach().double().cpu()
+    e = expected.detach().double().cpu()
+    assert a.shape == e.shape, (a.shape, e.shape)
+    assert torch.isfinite(a).all()
+    return float((a - e).abs().max() / e.abs().max().clamp_min(1e-30))
+
+
+def tol_of(dtype):
+    return F32_TOL if dtype == torch.float32 else BF16_TOL
+
+
+def rand(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+# ----------------------------------------------------------------------- norm
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,width", [(1, 64), (7, 96), (33, 100), (5, 2048), (3, 4099)])
+def test_add_rmsnorm(dtype, rows, width):
+    x = rand((rows, width), torch.float32, 1, 3.0)
+    delta = rand((rows, width), dtype, 2)
+    w = rand((width,), torch.float32, 3) + 1.0
+    eps = 1e-5
+    res = x.clone().to(dev())
+    out = ops().add_rmsnorm(res, delta.to(dev()), w.to(dev()), eps, dtype)
+    h = x.double() + delta.double()
+    expect = plain.rms_norm(h, w.double(), eps)
+    assert rel_err(res, h) < F32_TOL                      # the stream took the sum, in 32-bit
+    assert rel_err(out, expect) < tol_of(dtype)
+    # norm of the stream alone leaves it untouched
+    res2 = x.clone().to(dev())
+    out2 = ops().add_rmsnorm(res2, None, w.to(dev()), eps, dtype)
+    assert torch.equal(res2.cpu(), x)
+    assert rel_err(out2, plain.rms_norm(x.double(), w.double(), eps)) < tol_of(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_add_rmsnorm_selected_rows(dtype):
+    x = rand((20, 72), torch.float32, 4)
+    delta = rand((20, 72), dtype, 5)
+    w = rand((72,), torch.float32, 6)
+    rows = torch.tensor([19, 0, 7], dtype=torch.int32)
+    res = x.clone().to(dev())
+    out = ops().add_rmsnorm(res, delta.to(dev()), w.to(dev()), 1e-6, dtype, rows=rows.to(dev()))
+    assert torch.equal(res.cpu(), x)                      # nothing stored back
+    expect = plain.rms_norm((x.double() + delta.double())[rows.long()], w.double(), 1e-6)
+    assert rel_err(out, expect) < tol_of(dtype)
+
+
+def test_rmsnorm_reference_vectors():
+    """The inputs of /root/reference/src/transformer/norm.zig:83-103 ([1,2,3,4] and
+    [1,1,1,1], weight 1): the values follow from the formula; ones stay ones."""
+    x = torch.tensor([[1.0, 2.0, 3.0, 4.0], [1.0, 1.0, 1.0, 1.0]])
+    out = ops().add_rmsnorm(x.to(dev()), None, torch.ones(4, device=dev()), 0.0, torch.float32,
+                            write_residual=False).cpu()
+    assert torch.allclose(out[0], x[0] / math.sqrt(7.5), atol=1e-6)
+    assert torch.allclose(out[1], torch.ones(4), atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed_gather(dtype):
+    table = rand((37, 50), dtype, 7)
+    tokens = torch.tensor([0, 5, 10, 20, 30, 36, 5], dtype=torch.int32)
+    out = ops().embed_gather(tokens.to(dev()), table.to(dev())).cpu()
+    assert out.dtype == torch.float32
+    assert torch.equal(out, table.float()[tokens.long()])
+
+
+# ----------------------------------------------------------------------- gemm
+@pytest.mark.parametrize("M,N,K", [(1, 7, 5), (33, 65, 17), (130, 200, 96), (64, 64, 64), (2, 301, 80)])
+def test_gemm_f32(M, N, K):
+    x, w, b = rand((M, K), torch.float32, 8), rand((N, K), torch.float32, 9), rand((N,), torch.float32, 10)
+    out = ops().linear(x.to(dev()), w.to(dev()), b.to(dev()))
+    expect = x.double() @ w.double().T + b.double()
+    assert out.dtype == torch.float32
+    assert rel_err(out, expect) < F32_TOL
+    out_nb = ops().linear(x.to(dev()), w.to(dev()))
+    assert rel_err(out_nb, x.double() @ w.double().T) < F32_TOL
+
+
+def test_gemm_f32_weight_with_bf16_activations():
+    """A weight stored in 32-bit stays 32-bit in a bfloat16 run."""
+    x, w = rand((9, 40), torch.bfloat16, 11), rand((23, 40), torch.float32, 12)
+    out = ops().linear(x.to(dev()), w.to(dev()))
+    assert out.dtype == torch.bfloat16
+    assert rel_err(out, x.double() @ w.double().T) < BF16_TOL
+
+
+@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 64, 65, 130, 300])
+@pytest.mark.parametrize("N,K", [(50, 96), (130, 264), (16, 8), (257, 1024)])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_gemm_bf16(M, N, K, out_dtype):
+    x, w, b = rand((M, K), torch.bfloat16, 13), rand((N, K), torch.bfloat16, 14), rand((N,), torch.float32, 15)
+    out = ops().linear(x.to(dev()), w.to(dev()), b.to(dev()), out_dtype=out_dtype)
+    expect = x.double() @ w.double().T + b.double()
+    assert out.dtype == out_dtype
+    assert rel_err(out, expect) < tol_of(out_dtype)
+
+
+@pytest.mark.parametrize("M", [1, 16, 40, 64])
+def test_gemm_bf16_skinny_and_tiled_agree(M):
+    """The two bfloat16 kernels may differ in rounding only."""
+    x, w = rand((M, 512), torch.bfloat16, 16), rand((96, 512), torch.bfloat16, 17)
+    a = ops().linear(x.to(dev()), w.to(dev()), out_dtype=torch.float32)
+    b = ops().linear(x.to(dev()), w.to(dev()), out_dtype=torch.float32, force_tiled=True)
+    assert rel_err(a, b.double()) < F32_TOL
+
+
+def test_gemm_rows_do_not_depend_on_batch():
+    """A token's projection is the same whatever else is in the step (bitwise,
+    within one kernel)."""
+    x, w = rand((64, 256), torch.bfloat16, 18), rand((80, 256), torch.bfloat16, 19)
+    full = ops().linear(x.to(dev()), w.to(dev()), out_dtype=torch.float32).cpu()
+    for m in (1, 5, 16, 33):
+        part = ops().linear(x[:m].contiguous().to(dev()), w.to(dev()), out_dtype=torch.float32).cpu()
+        assert torch.equal(part, full[:m])
+    x32, w32 = x.float(), w.float()
+    full32 = ops().linear(x32.to(dev()), w32.to(dev())).cpu()
+    part32 = ops().linear(x32[:3].contiguous().to(dev()), w32.to(dev())).cpu()
+    assert torch.equal(part32, full32[:3])
+
+
+def test_gemm_bf16_refuses_odd_k():
+    from zig_ai_amd.kernels import KernelError
+    x, w = rand((4, 12), torch.bfloat16, 20), rand((8, 12), torch.bfloat16, 21)
+    with pytest.raises(KernelError, match="multiple of 8"):
+        ops().linear(x.to(dev()), w.to(dev()))
+
+
+# ---------------------------------------------------------------- rope + cache
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,d,rot,pairing", [
+    (4, 2, 16, 16, "half"), (3, 1, 32, 32, "half"), (5, 5, 48, 48, "adjacent"),
+    (8, 2, 64, 32, "half"), (2, 2, 256, 256, "half"), (6, 3, 128, 64, "adjacent")])
+def test_qk_norm_rope_kv_write(dtype, nh, nkv, d, rot, pairing):
+    T, page_size, pages = 11, 4, 9
+    theta, eps = 10000.0, 1e-5
+    qkv = rand((T, (nh + 2 * nkv) * d), dtype, 22)
+    qw, kw = rand((d,), torch.float32, 23) + 1.0, rand((d,), torch.float32, 24) + 1.0
+    positions = torch.tensor([0, 1, 2, 3, 100, 101, 7, 8, 9, 10, 11], dtype=torch.int32)
+    perm = torch.randperm(pages * page_size, generator=torch.Generator().manual_seed(25))[:T]
+    slots = perm.to(torch.int32)
+    inv = (1.0 / torch.pow(torch.tensor(theta, dtype=torch.float64),
+                           2.0 * torch.arange(0, rot // 2, dtype=torch.float64) / rot)).float()
+    cache = torch.zeros((pages, 2, nkv, page_size, d), dtype=dtype, device=dev())
+    q = ops().qk_norm_rope_kv_write(qkv.to(dev()), positions.to(dev()), slots.to(dev()),
+                                    qw.to(dev()), kw.to(dev()), inv.to(dev()), cache, nh, nkv, d,
+                                    rot, pairing == "adjacent", eps)
+    heads = qkv.double().view(T, nh + 2 * nkv, d)
+    qe = plain.apply_rope(plain.rms_norm(heads[:, :nh], qw.double(), eps), positions, theta, rot, pairing)
+    ke = plain.apply_rope(plain.rms_norm(heads[:, nh:nh + nkv], kw.double(), eps), positions, theta,
+                          rot, pairing)
+    ve = heads[:, nh + nkv:]
+    # angles are computed in 32-bit: position 101 * 2^-24 relative error in the angle
+    tol = tol_of(dtype) + 101 * 1.2e-7
+    assert rel_err(q, qe) < tol
+    c = cache.cpu()
+    got_k = torch.stack([c[s // page_size, 0, :, s % page_size, :] for s in slots.tolist()])
+    got_v = torch.stack([c[s // page_size, 1, :, s % page_size, :] for s in slots.tolist()])
+    assert rel_err(got_k, ke) < tol
+    assert torch.equal(got_v.double(), ve)                 # values are stored as they are
+    written = torch.zeros(pages * page_size, dtype=torch.bool)
+    written[slots.long()] = True
+    untouched = c.permute(0, 3, 1, 2, 4).reshape(pages * page_size, -1)[~written]
+    assert (untouched == 0).all()                          # and nothing else was touched
+
+
+def test_rope_position_zero_is_identity_and_norm_is_kept():
+    """rope.zig:226-253 holds the rotation to preserving the norm; position 0 rotates
+    by nothing."""
+    nh, nkv, d = 2, 1, 64
+    T = 6
+    qkv = rand((T, (nh + 2 * nkv) * d), torch.float32, 26)
+    positions = torch.tensor([0, 1, 5, 50, 500, 4000], dtype=torch.int32)
+    inv = (1.0 / torch.pow(torch.tensor(10000.0, dtype=torch.float64),
+                           2.0 * torch.arange(0, d // 2, dtype=torch.float64) / d)).float()
+    q = ops().qk_norm_rope_kv_write(qkv.to(dev()), positions.to(dev()), None, None, None,
+                                    inv.to(dev()), None, nh, nkv, d, d, False, 0.0,
+                                    write_kv=False).cpu()
+    src = qkv.view(T, nh + 2 * nkv, d)[:, :nh]
+    assert torch.equal(q[0], src[0])
+    assert torch.allclose(q.norm(dim=-1), src.norm(dim=-1), rtol=1e-5)
+
+
+# ------------------------------------------------------------------ attention
+def paged_from_dense(k, v, page_size, dtype, extra_pages=3, seed=0):
+    """Scatter dense per-request K/V ``[len, nkv, d]`` into a shuffled paged cache.
+    Returns cache, block table [S, max_pages]."""
+    nkv, d = k[0].shape[1], k[0].shape[2]
+    need = [(x.shape[0] + page_size - 1) // page_size for x in k]
+    total = sum(need) + extra_pages
+    order = torch.randperm(total, generator=torch.Generator().manual_seed(seed)).tolist()
+    cache = torch.zeros((total, 2, nkv, page_size, d), dtype=dtype)
+    # poison pages nobody owns so that a stray read shows
+    table = torch.full((len(k), max(need)), -1, dtype=torch.int32)
+    nxt = 0
+    for s, (ks, vs) in enumerate(zip(k, v)):
+        for p in range(need[s]):
+            page = order[nxt]
+            nxt += 1
+            table[s, p] = page
+            lo, hi = p * page_size, min((p + 1) * page_size, ks.shape[0])
+            cache[page, 0, :, : hi - lo] = ks[lo:hi].transpose(0, 1).to(dtype)
+            cache[page, 1, :, : hi - lo] = vs[lo:hi].transpose(0, 1).to(dtype)
+    for page in order[nxt:]:
+        cache[page] = 1e4
+    return cache, table
+
+
+def items_for(seq_lens, rows_per_item):
+    from zig_ai_amd.engine.batch import _make_items
+    seq, row0, cnt = _make_items(seq_lens, rows_per_item)
+    mk = lambda x: torch.tensor(x, dtype=torch.int32, device=dev())
+    return mk(seq), mk(row0), mk(cnt), len(seq)
+
+
+def run_attention(dtype, nh, nkv, d, page_size, ctx, new, window=0, keys_per_split=0, nsplit=1,
+                  seed=30, sharpen=False):
+    """ctx[s] cached tokens and new[s] query tokens per request."""
+    G = nh // nkv
+    ks, vs, qs, pos = [], [], [], []
+    for s, (c, n) in enumerate(zip(ctx, new)):
+        k = rand((c + n, nkv, d), dtype, seed + 3 * s)
+        v = rand((c + n, nkv, d), dtype, seed + 3 * s + 1)
+        q = rand((n, nh, d), dtype, seed + 3 * s + 2)
+        if sharpen and c > 3:
+            # one far key matches the last query strongly: its value must dominate
+            k[1] = 0
+            k[1, :, 0] = 8.0
+            q[-1] = 0
+            q[-1, :, 0] = 8.0
+        ks.append(k); vs.append(v); qs.append(q)
+        pos += list(range(c, c + n))
+    cache, table = paged_from_dense(ks, vs, page_size, dtype, seed=seed)
+    q_all = torch.cat(qs).to(dev())
+    positions = torch.tensor(pos, dtype=torch.int32, device=dev())
+    rows = max(1, 32 // G)
+    out = ops().paged_attention(q_all, cache.to(dev()), table.to(dev()), positions,
+                                *items_for(new, rows), 1.0 / math.sqrt(d), window,
+                                keys_per_split, nsplit)
+    expect = []
+    for s, (c, n) in enumerate(zip(ctx, new)):
+        full_q = torch.zeros((c + n, nh, d), dtype=torch.float64)
+        full_q[c:] = qs[s].double()
+        o = plain.causal_attention(full_q, ks[s].double(), vs[s].double(), window=window)
+        expect.append(o[c:])
+    return out, torch.cat(expect)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,d,page_size", [
+    (4, 2, 16, 4), (3, 1, 32, 8), (5, 5, 48, 16), (32, 8, 64, 16), (8, 1, 128, 16),
+    (2, 2, 256, 8), (16, 1, 64, 32)])
+def test_paged_attention_mixed_batch(dtype, nh, nkv, d, page_size):
+    """Portions of prompts beside single decoded tokens, in one launch."""
+    ctx = [0, 37, 129, 5, 64]
+    new = [33, 1, 1, 70, 2]
+    out, expect = run_attention(dtype, nh, nkv, d, page_size, ctx, new)
+    assert rel_err(out, expect) < tol_of(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_paged_attention_reference_shapes(dtype):
+    """The shapes of the reference's own attention tests
+    (/root/reference/tests/test_paged_attention_gpu.zig:40-131, 284-327): 9 decoded
+    tokens at block size 4 with 8 query / 2 key heads of size 8; a 6-token prompt;
+    40 tokens at block size 16 with head size 128.  Their tolerance is 5e-3 to 1e-2."""
+    for nh, nkv, d, ps, ctx, new in [(8, 2, 8, 4, [8], [1]), (8, 2, 8, 4, [0], [6]),
+                                     (32, 8, 128, 16, [39], [1])]:
+        out, expect = run_attention(dtype, nh, nkv, d, ps, ctx, new)
+        assert rel_err(out, expect) < tol_of(dtype)
+
+
+def test_single_token_attention_returns_value():
+    """One key: the softmax is 1 and the output is V (derived, but only checked for
+    finiteness, in /root/reference/src/transformer/hybrid_attn.zig:1207-1212)."""
+    nh, nkv, d = 4, 2, 16
+    k, v, q = rand((1, nkv, d), torch.float32, 40), rand((1, nkv, d), torch.float32, 41), rand((1, nh, d), torch.float32, 42)
+    cache, table = paged_from_dense([k], [v], 4, torch.float32)
+    out = ops().paged_attention(q.to(dev()), cache.to(dev()), table.to(dev()),
+                                torch.zeros(1, dtype=torch.int32, device=dev()),
+                                *items_for([1], 16), 0.25).cpu()
+    for h in range(nh):
+        assert torch.allclose(out[0, h], v[0, h // 2], atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_paged_attention_far_key_dominates(dtype):
+    """One early key among hundreds carries the weight: a kernel that loses far
+    keys (a page's edge, a tile's edge) cannot pass."""
+    out, expect = run_attention(dtype, 8, 2, 64, 16, [700, 300], [1, 5], sharpen=True)
+    assert rel_err(out, expect) < tol_of(dtype)
+    assert float(expect.abs().max()) > 0.5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("keys,nsplit", [(64, 12), (256, 3), (128, 8)])
+def test_paged_attention_split_context(dtype, keys, nsplit):
+    ctx, new = [700, 1, 255, 64], [1, 1, 1, 1]
+    whole, expect = run_attention(dtype, 8, 2, 64, 16, ctx, new, sharpen=True)
+    cut, _ = run_attention(dtype, 8, 2, 64, 16, ctx, new, keys_per_split=keys, nsplit=nsplit,
+                           sharpen=True)
+    assert rel_err(cut, expect) < tol_of(dtype)
+    assert rel_err(cut, whole.double()) < tol_of(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [1, 5, 16, 100])
+def test_paged_attention_window(dtype, window):
+    out, expect = run_attention(dtype, 6, 2, 32, 8, [0, 90, 41], [50, 1, 9], window=window)
+    assert rel_err(out, expect) < tol_of(dtype)
+
+
+def test_paged_attention_window_skips_freed_pages():
+    """Pages behind the window may be gone from the table (-1): never read."""
+    nh, nkv, d, ps, window = 4, 2, 16, 4, 6
+    c, n = 40, 3
+    k, v, q = rand((c + n, nkv, d), torch.float32, 50), rand((c + n, nkv, d), torch.float32, 51), rand((n, nh, d), torch.float32, 52)
+    cache, table = paged_from_dense([k], [v], ps, torch.float32)
+    first_needed = c - window + 1
+    for p in range(first_needed // ps):
+        cache[table[0, p]] = float("nan")
+        table[0, p] = -1
+    pos = torch.arange(c, c + n, dtype=torch.int32, device=dev())
+    out = ops().paged_attention(q.to(dev()), cache.to(dev()), table.to(dev()), pos,
+                                *items_for([n], 16), 0.25, window)
+    full_q = torch.zeros((c + n, nh, d), dtype=torch.float64)
+    full_q[c:] = q.double()
+    expect = plain.causal_attention(full_q, k.double(), v.double(), window=window)[c:]
+    assert rel_err(out, expect) < F32_TOL
+
+
+# ------------------------------------------------------------------ short conv
+def conv_reference(z, w, b, H):
+    B, C, x = z[:, :H], z[:, H:2 * H], z[:, 2 * H:]
+    return C * plain.causal_depthwise_conv(B * x, w, b)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,L,bias", [(64, 3, False), (96, 4, True), (80, 2, True), (300, 1, False),
+                                      (2048, 3, False), (40, 8, True)])
+def test_short_conv_whole_and_in_portions(dtype, H, L, bias):
+    """Three requests packed in one launch; then the same tokens in portions of
+    changing size (down to one token) with the carried state: same result."""
+    lens = [23, 1, 9]
+    zs = [rand((n, 3 * H), dtype, 60 + i) for i, n in enumerate(lens)]
+    w = rand((H, L), torch.float32, 70)
+    b = rand((H,), torch.float32, 71) if bias else None
+    expect = [conv_reference(z.double(), w.double(), b.double() if bias else None, H) for z in zs]
+
+    def launch(parts, state, slot_ids):
+        z = torch.cat(parts).to(dev())
+        n = [p.shape[0] for p in parts]
+        token_seq = torch.cat([torch.full((m,), i, dtype=torch.int32) for i, m in enumerate(n)])
+        seq_start = torch.tensor([0] + list(torch.tensor(n).cumsum(0)), dtype=torch.int32)
+        return ops().short_conv(z, w.to(dev()), b.to(dev()) if bias else None, state,
+                                token_seq.to(dev()), seq_start.to(dev()),
+                                torch.tensor(slot_ids, dtype=torch.int32, device=dev()))
+
+    # slots live in a wider row, as the cache manager lays them out
+    memory = torch.zeros((5, H * L + 7), dtype=torch.float32, device=dev())
+    state = memory[:, 3:3 + H * L].unflatten(1, (H, L))
+    y = launch(zs, state, [4, 0, 2])
+    assert rel_err(y, torch.cat(expect)) < tol_of(dtype)
+    # the state holds the last L gated inputs, oldest first, zeros before the start
+    for z, slot in zip(zs, [4, 0, 2]):
+        u = (z.double()[:, :H] * z.double()[:, 2 * H:])
+        padded = torch.cat([torch.zeros(L, H, dtype=torch.float64), u])[-L:]
+        assert rel_err(state[slot].cpu().T, padded) < F32_TOL if padded.abs().max() > 0 else True
+    assert (memory[[1, 3]] == 0).all() and (memory[:, :3] == 0).all() and (memory[:, 3 + H * L:] == 0).all()
+
+    memory.zero_()
+    cuts = [[5, 1, 2, 7, 1, 1, 6], [1], [2, 2, 1, 4]]
+    cursor = [0, 0, 0]
+    got = [[] for _ in lens]
+    for step in range(max(len(c) for c in cuts)):
+        parts, slots, who = [], [], []
+        for i in range(3):
+            if step < len(cuts[i]):
+                n = cuts[i][step]
+                parts.append(zs[i][cursor[i]:cursor[i] + n])
+                cursor[i] += n
+                slots.append([4, 0, 2][i])
+                who.append(i)
+        y = launch(parts, state, slots).cpu()
+        row = 0
+        for i, p in zip(who, parts):
+            got[i].append(y[row:row + p.shape[0]])
+            row += p.shape[0]
+    for i in range(3):
+        assert rel_err(torch.cat(got[i]), expect[i]) < tol_of(dtype)
+
+
+def test_short_conv_identity_filter():
+    """Filter e_{L-1} with B = C = 1 passes x through."""
+    H, L, T = 32, 3, 10
+    x = rand((T, H), torch.float32, 80)
+    z = torch.cat([torch.ones(T, H), torch.ones(T, H), x], dim=1)
+    w = torch.zeros(H, L)
+    w[:, L - 1] = 1.0
+    state = torch.zeros((1, H, L), device=dev())
+    y = ops().short_conv(z.to(dev()), w.to(dev()), None, state,
+                         torch.zeros(T, dtype=torch.int32, device=dev()),
+                         torch.tensor([0, T], dtype=torch.int32, device=dev()),
+                         torch.zeros(1, dtype=torch.int32, device=dev())).cpu()
+    assert torch.equal(y, x)
+
+
+# ------------------------------------------------------------------ activation
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,I", [(1, 8), (5, 176), (3, 13), (4, 128), (2, 8192)])
+def test_swiglu(dtype, T, I):
+    gu = rand((T, 2 * I), dtype, 90, 2.0)
+    out = ops().swiglu(gu.to(dev()))
+    g, u = gu.double()[:, :I], gu.double()[:, I:]
+    assert out.shape == (T, I)
+    assert rel_err(out, torch.nn.functional.silu(g) * u) < tol_of(dtype)
+
+
+def test_cast_round_trip():
+    x = rand((1000,), torch.float32, 91)
+    b = ops().cast(x.to(dev()), torch.bfloat16)
+    assert torch.equal(b.cpu(), x.to(torch.bfloat16))       # round to nearest even, as torch
+    assert torch.equal(ops().cast(b, torch.float32).cpu(), x.to(torch.bfloat16).float())
+
+
+# -------------------------------------------------------------------- sampling
+def test_argmax_first_occurrence():
+    logits = rand((6, 1000), torch.float32, 100)
+    logits[0, 17] = logits[0, 900] = 50.0       # a tie: the first index wins
+    logits[1, 999] = 60.0
+    logits[2, 0] = 60.0
+    logits[3] = 0.0                             # all equal
+    out = ops().argmax(logits.to(dev())).cpu().tolist()
+    assert out == [plain.argmax_first(r) for r in logits]
+    assert out[0] == 17 and out[1] == 999 and out[2] == 0 and out[3] == 0
+
+
+@pytest.mark.parametrize("vocab", [50, 1000, 65536])
+def test_sample_matches_plain(vocab):
+    R = 12
+    logits = rand((R, vocab), torch.float32, 101, 3.0)
+    temps = torch.tensor([0.0, 0.7, 1.0, 1.5, 0.7, 0.7, 1.0, 0.2, 1.0, 1.0, 0.7, 0.0])
+    top_k = torch.tensor([0, 0, 0, 0, 5, 0, 40, 0, 1, 0, 10, 3], dtype=torch.int32)
+    top_p = torch.tensor([1.0, 1.0, 1.0, 1.0, 1.0, 0.9, 0.5, 1.0, 1.0, 0.01, 0.8, 0.9])
+    u = torch.tensor([0.3, 0.0, 0.999999, 0.5, 0.25, 0.75, 0.6, 0.1, 0.9, 0.4, 0.33, 0.5])
+    out = ops().sample(logits.to(dev()), temps.to(dev()), top_k.to(dev()), top_p.to(dev()),
+                       u.to(dev())).cpu().tolist()
+    for r in range(R):
+        want = plain.sample_token(logits[r].double(), float(temps[r]), float(u[r]),
+                                  int(top_k[r]), float(top_p[r]))
+        if out[r] != want:
+            # the draw may fall within rounding of a boundary between two tokens:
+            # accept the neighbour only if u sits on that boundary
+            v = logits[r].double() / float(temps[r])
+            keep = plain.kept_after_top_k_top_p(v, int(top_k[r]), float(top_p[r]))
+            assert bool(keep[out[r]]), (r, out[r], want)
+            e = torch.where(keep, torch.exp(v - v[keep].max()), torch.zeros_like(v))
+            cdf = torch.cumsum(e, 0) / e.sum()
+            lo = float(cdf[out[r] - 1]) if out[r] > 0 else 0.0
+            assert lo - 1e-5 <= float(u[r]) <= float(cdf[out[r]]) + 1e-5, (r, out[r], want)
+
+
+def test_sample_distribution():
+    """Frequencies over many uniforms follow softmax(logits / T)."""
+    vocab, n = 8, 4000
+    row = torch.tensor([2.0, 1.0, 0.5, 0.0, -1.0, 3.0, 1.5, -2.0])
+    logits = row.repeat(n, 1)
+    u = (torch.arange(n, dtype=torch.float32) + 0.5) / n
+    out = ops().sample(logits.to(dev()), torch.full((n,), 0.7, device=dev()),
+                       torch.zeros(n, dtype=torch.int32, device=dev()),
+                       torch.ones(n, device=dev()), u.to(dev())).cpu()
+    freq = torch.bincount(out.long(), minlength=vocab).double() / n
+    assert (freq - torch.softmax(row.double() / 0.7, 0)).abs().max() < 2.0 / n + 1e-3
+
+
+def test_repetition_penalty():
+    logits = torch.tensor([[2.0, -2.0, 0.0, 4.0], [1.0, 1.0, -1.0, -1.0]])
+    rows = torch.tensor([0, 0, 1, 1], dtype=torch.int32)
+    toks = torch.tensor([0, 1, 3, 0], dtype=torch.int32)
+    fac = torch.tensor([2.0, 2.0, 4.0, 1.5])
+    work = logits.clone().to(dev())
+    ops().repetition_penalty_(work, rows.to(dev()), toks.to(dev()), fac.to(dev()))
+    assert torch.allclose(work.cpu(), torch.tensor([[1.0, -4.0, 0.0, 4.0], [1.0 / 1.5, 1.0, -1.0, -4.0]]))

@@ -1,0 +1,34 @@
+"""Small LFM2 configurations for tests.  A and B are the two that differ in
+every size and option; C adds sizes that are multiples of neither 16 nor a
+power of two where the kernels allow it."""
+
+TINY_A = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 64, "num_hidden_layers": 4, "num_attention_heads": 4,
+    "num_key_value_heads": 2, "vocab_size": 256,
+    "layer_types": ["conv", "conv", "full_attention", "conv"],
+    "block_ff_dim": 192, "block_auto_adjust_ff_dim": False,
+    "rope_theta": 10000.0, "norm_eps": 1e-5, "conv_L_cache": 3, "conv_bias": False,
+    "tie_embedding": True, "max_position_embeddings": 4096,
+}
+
+TINY_B = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 96, "num_hidden_layers": 6, "num_attention_heads": 3,
+    "num_key_value_heads": 1, "head_dim": 32, "vocab_size": 512,
+    "layer_types": ["full_attention", "conv", "conv", "full_attention", "conv", "full_attention"],
+    "block_ff_dim": 384, "block_auto_adjust_ff_dim": True, "block_multiple_of": 128,
+    "rope_theta": 1000000.0, "norm_eps": 1e-6, "conv_L_cache": 4, "conv_bias": True,
+    "tie_embedding": False, "max_position_embeddings": 4096,
+}
+
+TINY_C = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 80, "num_hidden_layers": 3, "num_attention_heads": 5,
+    "num_key_value_heads": 5, "head_dim": 48, "vocab_size": 301,
+    "layer_types": ["full_attention", "conv", "full_attention"],
+    "block_ff_dim": 200, "block_auto_adjust_ff_dim": True, "block_multiple_of": 8,
+    "block_ffn_dim_multiplier": 1.3,
+    "rope_theta": 50000.0, "norm_eps": 3e-6, "conv_L_cache": 2, "conv_bias": True,
+    "tie_embedding": True, "max_position_embeddings": 4096,
+}

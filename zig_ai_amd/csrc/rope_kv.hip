@@ -1,0 +1,111 @@
+// Per-head RMSNorm of queries and keys, rotary position encoding, and the
+// scatter of keys and values into their cache pages: one pass over the fused
+// q|k|v projection.
+//
+// Per (token, head), in 32-bit:
+//   q, k:  x <- x * (1/sqrt(mean(x^2) + eps)) * w[head_dim]      (if norm weights are given;
+//          before the rotation, never on v: /root/reference/src/transformer/hybrid_attn.zig:371-382)
+//   q, k:  for pair p < rotary_dim/2 with angle = position * inv_freq[p]:
+//            (a, b) <- (a cos - b sin, a sin + b cos)
+//          (/root/reference/src/transformer/rope.zig:40-56); the pair is (p, p + rotary_dim/2)
+//          for "half" pairing (the reference's device kernel,
+//          /root/reference/src/cuda/layer_kernels.cu:353-365) or (2p, 2p+1) for "adjacent"
+//          pairing (rope.zig:46-53).  Elements beyond rotary_dim pass through.
+//   k, v -> cache[page][0 or 1][kv_head][offset][head_dim],  slot = page * page_size + offset
+//   q    -> q_out[token][head][head_dim]
+#include "common.h"
+
+#define RK_MAX_D 256
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+qk_norm_rope_kv_write_kernel(const T* __restrict__ qkv, const int* __restrict__ positions,
+                             const int* __restrict__ slots, const float* __restrict__ q_norm_w,
+                             const float* __restrict__ k_norm_w, const float* __restrict__ inv_freq,
+                             T* __restrict__ q_out, T* __restrict__ kv_cache, int nh, int nkv, int d,
+                             int rot, int adjacent, float eps, int page_size, int write_kv) {
+  __shared__ float vec[4][RK_MAX_D];
+  const int t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int head = blockIdx.y * 4 + wave;  // 0..nh-1: q; then nkv k heads; then nkv v heads
+  const int total = nh + 2 * nkv;
+  const bool active = head < total;
+  const bool is_q = head < nh;
+  const bool is_k = !is_q && head < nh + nkv;
+  float* s = vec[wave];
+
+  float ss = 0.f;
+  if (active) {
+    const T* src = qkv + ((size_t)t * total + head) * d;
+    for (int i = lane; i < d; i += 64) {
+      const float v = to_f32<T>(src[i]);
+      s[i] = v;
+      ss += v * v;
+    }
+  }
+  ss = wave_sum(ss);
+  __syncthreads();
+  const float* nw = is_q ? q_norm_w : (is_k ? k_norm_w : nullptr);
+  if (active && nw) {
+    const float scale = 1.0f / sqrtf(ss / (float)d + eps);
+    for (int i = lane; i < d; i += 64) s[i] = s[i] * scale * nw[i];
+  }
+  __syncthreads();
+  if (active && (is_q || is_k) && rot > 0) {
+    const float pos = (float)positions[t];
+    const int half = rot / 2;
+    for (int p = lane; p < half; p += 64) {
+      const int i0 = adjacent ? 2 * p : p;
+      const int i1 = adjacent ? 2 * p + 1 : p + half;
+      const float angle = pos * inv_freq[p];
+      float sn, cs;
+      sincosf(angle, &sn, &cs);
+      const float a = s[i0], b = s[i1];
+      s[i0] = a * cs - b * sn;
+      s[i1] = a * sn + b * cs;
+    }
+  }
+  __syncthreads();
+  if (!active) return;
+  if (is_q) {
+    T* dst = q_out + ((size_t)t * nh + head) * d;
+    for (int i = lane; i < d; i += 64) dst[i] = from_f32<T>(s[i]);
+  } else if (write_kv) {
+    const int slot = slots[t];
+    if (slot < 0) return;
+    const int page = slot / page_size, off = slot % page_size;
+    const int kvh = is_k ? head - nh : head - nh - nkv;
+    const int which = is_k ? 0 : 1;
+    T* dst = kv_cache + ((((size_t)page * 2 + which) * nkv + kvh) * page_size + off) * d;
+    for (int i = lane; i < d; i += 64) dst[i] = from_f32<T>(s[i]);
+  }
+}
+
+extern "C" int za_qk_norm_rope_kv_write(const void* qkv, const int* positions, const int* slots,
+                                        const float* q_norm_w, const float* k_norm_w,
+                                        const float* inv_freq, void* q_out, void* kv_cache,
+                                        int dtype, int n_tokens, int nh, int nkv, int d, int rot,
+                                        int adjacent, float eps, int page_size, int write_kv,
+                                        hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  if (n_tokens < 0 || nh <= 0 || nkv <= 0 || d <= 0 || !qkv || !positions || !q_out)
+    return ZA_ERR_ARG;
+  if (d > RK_MAX_D || rot < 0 || rot > d || (rot % 2) != 0) return ZA_ERR_UNSUPPORTED;
+  if (rot > 0 && !inv_freq) return ZA_ERR_ARG;
+  if (write_kv && (!kv_cache || !slots || page_size <= 0)) return ZA_ERR_ARG;
+  dim3 grid(n_tokens, (nh + 2 * nkv + 3) / 4), block(256);
+  if (dtype == 0) {
+    hipLaunchKernelGGL((qk_norm_rope_kv_write_kernel<float>), grid, block, 0, stream,
+                       (const float*)qkv, positions, slots, q_norm_w, k_norm_w, inv_freq,
+                       (float*)q_out, (float*)kv_cache, nh, nkv, d, rot, adjacent, eps, page_size,
+                       write_kv);
+  } else if (dtype == 1) {
+    hipLaunchKernelGGL((qk_norm_rope_kv_write_kernel<bf16_t>), grid, block, 0, stream,
+                       (const bf16_t*)qkv, positions, slots, q_norm_w, k_norm_w, inv_freq,
+                       (bf16_t*)q_out, (bf16_t*)kv_cache, nh, nkv, d, rot, adjacent, eps,
+                       page_size, write_kv);
+  } else {
+    return ZA_ERR_UNSUPPORTED;
+  }
+  return za_launch_status();
+}

@@ -1,0 +1,5 @@
+"""The step function, the scheduler above it, and generation."""
+
+from .batch import StepContext, StepEntry, StepError, build_step  # noqa: F401
+from .model import DecoderModel, require_gpu, run_dtype  # noqa: F401
+from .runner import ModelRunner  # noqa: F401

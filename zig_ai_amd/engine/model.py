@@ -1,0 +1,130 @@
+"""The decoder assembled from a ``ModelSpec``: embedding, blocks in run order,
+final norm, output head.  Nothing here is specific to one architecture; the
+spec decides which parts make up which layer and in which order layers run.
+"""
+
+from __future__ import annotations
+
+from typing import Any, Dict, List, Mapping, Optional, Sequence
+
+import torch
+
+from ..cache.manager import CacheManager, CacheView
+from ..config import load_config
+from ..config.spec import LayerCall, ModelSpec, PartSpec
+from ..kernels import build as kernel_build
+from ..parts import base as parts
+from ..weights.loader import load_tensors
+from .batch import StepContext
+
+_RUN_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
+               "float32": torch.float32, "fp32": torch.float32, "f32": torch.float32}
+
+
+def run_dtype(name) -> torch.dtype:
+    if isinstance(name, torch.dtype):
+        if name not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"the engine runs in bfloat16 or float32, not {name}")
+        return name
+    if name not in _RUN_DTYPES:
+        raise ValueError(f"dtype must be bfloat16 or float32, got {name!r}")
+    return _RUN_DTYPES[name]
+
+
+def require_gpu() -> torch.device:
+    if not torch.cuda.is_available():
+        raise RuntimeError("no GPU is visible: this engine has no CPU path")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec, tensors: Mapping[Any, Mapping[str, torch.Tensor]],
+                 runtime: parts.Runtime):
+        self.spec = spec
+        self.runtime = runtime
+
+        def make(family: str, part: PartSpec, owner):
+            cls = parts.lookup(family, part.kind)
+            return cls(part.params, dict(tensors.get(owner, {})), runtime)
+
+        sources = set()
+
+        def note(cls_or_obj) -> None:
+            sources.update(getattr(cls_or_obj, "kernel_sources", ()))
+
+        self.embedding = make("embedding", spec.embedding, ("embedding",))
+        note(self.embedding)
+        self.blocks = []
+        self.mixer_classes = []
+        for i, layer in enumerate(spec.layers):
+            mixer_norm = make("norm", layer.mixer_norm, ("layer", i, "mixer_norm"))
+            mixer = make("mixer", layer.mixer, ("layer", i, "mixer"))
+            ffn_norm = make("norm", layer.feed_forward_norm, ("layer", i, "feed_forward_norm"))
+            ffn = make("feed_forward", layer.feed_forward, ("layer", i, "feed_forward"))
+            for p in (mixer_norm, mixer, ffn_norm, ffn):
+                note(p)
+            arrangement = parts.lookup("arrangement", layer.arrangement)
+            self.blocks.append(arrangement(mixer_norm, mixer, ffn_norm, ffn))
+        self.final_norm = make("norm", spec.final_norm, ("final_norm",))
+        self.head = make("head", spec.lm_head, ("lm_head",))
+        note(self.final_norm)
+        note(self.head)
+        if getattr(self.head, "tied", False):
+            self.head.weight = self.embedding.weight     # the same memory, not a copy
+        if getattr(self.head, "weight", None) is None:
+            raise ValueError("the output head has no weight")
+
+        self.schedule: Sequence[LayerCall] = spec.resolved_schedule()
+        self.cache_needs: Dict[int, object] = {}
+        for call in self.schedule:
+            layer = spec.layers[call.layer]
+            need = parts.lookup("mixer", layer.mixer.kind).cache_need(layer.mixer.params)
+            if call.cache in self.cache_needs and self.cache_needs[call.cache] != need:
+                raise ValueError(
+                    f"run-order entries sharing cache {call.cache} need different caches: "
+                    f"{self.cache_needs[call.cache]} and {need}")
+            self.cache_needs[call.cache] = need
+        writers = {c.cache for c in self.schedule if c.writes_cache}
+        for call in self.schedule:
+            if self.cache_needs[call.cache] is not None and call.cache not in writers:
+                raise ValueError(f"cache {call.cache} is read but no run-order entry writes it")
+        self.item_granularities = sorted({
+            b.mixer.rows_per_item for b in self.blocks if hasattr(b.mixer, "rows_per_item")})
+        self.kernel_sources = sorted(sources)
+        # Compile what this model's parts use, together, before the first step.
+        if self.kernel_sources:
+            kernel_build.build_all(self.kernel_sources, jobs=len(self.kernel_sources))
+
+    # ------------------------------------------------------------- construction
+    @classmethod
+    def from_folder(cls, model_dir: str, dtype="bfloat16", device: Optional[torch.device] = None):
+        device = device or require_gpu()
+        config = load_config(model_dir)
+        spec = config.to_spec()
+        rt = parts.Runtime(device=device, dtype=run_dtype(dtype))
+        tensors = load_tensors(model_dir, spec, rt.dtype, device)
+        model = cls(spec, tensors, rt)
+        model.config = config
+        return model
+
+    def make_cache(self, page_size: int, num_pages, num_slots: int) -> CacheManager:
+        return CacheManager(self.cache_needs, page_size, num_pages, num_slots,
+                            device=self.runtime.device, dtype=self.runtime.dtype)
+
+    def cache_views(self, cache: CacheManager) -> List[CacheView]:
+        """One view per run-order entry."""
+        return [cache.view(call.cache, call.writes_cache) for call in self.schedule]
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, step: StepContext, views: Sequence[CacheView]) -> torch.Tensor:
+        """Run the step's tokens through every run-order entry and return 32-bit
+        logits ``[R, vocab]`` for ``step.logit_rows``."""
+        residual = self.embedding.forward(step.token_ids)
+        pending = None
+        for call, view in zip(self.schedule, views):
+            residual, pending = self.blocks[call.layer].forward(residual, pending, step, view)
+        if step.n_logit_rows == 0:
+            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32,
+                               device=self.runtime.device)
+        normed = self.final_norm.add_forward(residual, pending, rows=step.logit_rows)
+        return self.head.forward(normed)

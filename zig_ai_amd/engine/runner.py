@@ -1,0 +1,73 @@
+"""The step function: a model, its cache, and ``step(entries) -> logits``.
+
+One call runs exactly the tokens it is given, as one batch, from the cache that
+earlier calls left, and returns the logits at the wanted places.  Generation
+(through the scheduler) and trace replay both go through this class; there is
+no second forward path.
+
+The reference has no such function: its driver calls every layer for one
+sequence, in chunks of ``--ubatch-size`` tokens and then token by token
+(/root/reference/src/main.zig:795-865, 1138-1217), although its kernels are
+written for several sequences (``num_seqs``, ``block_tables[seq]``:
+/root/reference/src/cuda/paged_attention.cu:121-137).
+"""
+
+from __future__ import annotations
+
+from typing import Hashable, List, Optional, Sequence
+
+import torch
+
+from ..cache.manager import CacheManager
+from ..cache.pages import OutOfPages
+from .batch import StepContext, StepEntry, StepError, build_step
+from .model import DecoderModel
+
+
+class ModelRunner:
+    def __init__(self, model: DecoderModel, page_size: int = 16, num_pages: int = 1024,
+                 num_slots: int = 64):
+        self.model = model
+        self.device = model.runtime.device
+        self.cache = model.make_cache(page_size, num_pages, num_slots)
+        self.views = model.cache_views(self.cache)
+        self.steps_run = 0
+
+    # ----------------------------------------------------------------- requests
+    def admit(self, request: Hashable) -> None:
+        self.cache.admit(request)
+
+    def release(self, request: Hashable) -> None:
+        self.cache.release(request)
+
+    def is_live(self, request: Hashable) -> bool:
+        return request in self.cache.requests
+
+    # --------------------------------------------------------------------- step
+    def prepare(self, entries: Sequence[StepEntry]) -> StepContext:
+        """Reserve pages for the entries (all of them or none) and lay out the step."""
+        wanted = {}
+        for e in entries:
+            if e.request not in self.cache.requests:
+                raise StepError(f"request {e.request!r} was not admitted")
+            for gi, n in self.cache.pages_needed(e.request, len(e.tokens)).items():
+                wanted[gi] = wanted.get(gi, 0) + n
+        for gi, n in wanted.items():
+            pool = self.cache.groups[gi].pool
+            if n > pool.free_count:
+                raise OutOfPages(f"the step needs {n} pages of group {gi}, "
+                                 f"{pool.free_count} of {pool.size} are free")
+        for e in entries:
+            self.cache.reserve(e.request, len(e.tokens))
+        return build_step(entries, self.cache, self.device, self.model.spec.vocab_size,
+                          self.model.item_granularities, self.model.spec.max_position)
+
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Logits ``[R, vocab]`` (32-bit) at the wanted places, in the order of the
+        entries and of each entry's ``want``."""
+        ctx = self.prepare(entries)
+        logits = self.model.forward(ctx, self.views)
+        for e in entries:
+            self.cache.commit(e.request, len(e.tokens))
+        self.steps_run += 1
+        return logits

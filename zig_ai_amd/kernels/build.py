@@ -1,0 +1,186 @@
+"""Compiling the HIP sources under ``csrc/`` for gfx950 and loading the result.
+
+Every ``<name>.hip`` becomes ``lib<name>.so`` in ``zig_ai_amd/_lib`` (or, when
+the package folder cannot be written, in a per-user folder under the system's
+temporary directory).  A library is compiled the first time something needs it
+and it is not there, or when its sources have changed since it was built;
+``build_all(force=True)`` compiles everything regardless.  While compiling, a
+line is printed now and then so that a first call does not look hung.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import threading
+import time
+from concurrent.futures import ThreadPoolExecutor
+from typing import Dict, Iterable, List, Optional
+
+PACKAGE_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC_DIR = os.path.join(PACKAGE_DIR, "csrc")
+ARCH = "gfx950"
+SOURCES = ("norm", "gemm", "rope_kv", "attention", "shortconv", "activation", "sampling")
+HIPCC_FLAGS = [
+    f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+_loaded: Dict[str, ctypes.CDLL] = {}
+_lock = threading.Lock()
+
+
+class KernelBuildError(RuntimeError):
+    pass
+
+
+def _say(msg: str) -> None:
+    print(f"[zig_ai_amd] {msg}", file=sys.stderr, flush=True)
+
+
+def find_hipcc() -> Optional[str]:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.isfile(cand) and os.access(cand, os.X_OK):
+            return cand
+    return None
+
+
+def _lib_dirs() -> List[str]:
+    """Folders that may hold built libraries, in order of preference."""
+    dirs = [os.path.join(PACKAGE_DIR, "_lib")]
+    uid = os.getuid() if hasattr(os, "getuid") else 0
+    dirs.append(os.path.join(tempfile.gettempdir(), f"zig_ai_amd-{uid}", "_lib"))
+    return dirs
+
+
+def _writable_lib_dir() -> str:
+    for d in _lib_dirs():
+        try:
+            os.makedirs(d, exist_ok=True)
+            probe = os.path.join(d, f".probe-{os.getpid()}-{threading.get_ident()}")
+            with open(probe, "w"):
+                pass
+            os.remove(probe)
+            return d
+        except OSError:
+            continue
+    raise KernelBuildError("no writable folder for compiled kernels: tried " + ", ".join(_lib_dirs()))
+
+
+def source_digest(name: str) -> str:
+    h = hashlib.sha256()
+    for path in (os.path.join(CSRC_DIR, "common.h"), os.path.join(CSRC_DIR, name + ".hip")):
+        with open(path, "rb") as f:
+            h.update(f.read())
+    h.update(" ".join(HIPCC_FLAGS).encode())
+    return h.hexdigest()
+
+
+def _find_built(name: str) -> Optional[str]:
+    """Path of an up-to-date library, or None."""
+    want = source_digest(name)
+    for d in _lib_dirs():
+        so = os.path.join(d, f"lib{name}.so")
+        tag = so + ".digest"
+        if os.path.isfile(so) and os.path.isfile(tag):
+            try:
+                with open(tag, "r") as f:
+                    if f.read().strip() == want:
+                        return so
+            except OSError:
+                pass
+    return None
+
+
+def _find_stale(name: str) -> Optional[str]:
+    for d in _lib_dirs():
+        so = os.path.join(d, f"lib{name}.so")
+        if os.path.isfile(so):
+            return so
+    return None
+
+
+def compile_one(name: str) -> str:
+    hipcc = find_hipcc()
+    if hipcc is None:
+        raise KernelBuildError(
+            f"kernel library lib{name}.so is not built and hipcc was not found "
+            "(looked at $HIPCC, PATH and /opt/rocm/bin/hipcc)")
+    src = os.path.join(CSRC_DIR, name + ".hip")
+    if not os.path.isfile(src):
+        raise KernelBuildError(f"{src} does not exist")
+    out_dir = _writable_lib_dir()
+    so = os.path.join(out_dir, f"lib{name}.so")
+    tmp = os.path.join(out_dir, f".lib{name}.{os.getpid()}.{threading.get_ident()}.so")
+    cmd = [hipcc] + HIPCC_FLAGS + ["-I", CSRC_DIR, "-o", tmp, src]
+    env = dict(os.environ)
+    home = env.get("HOME", "")
+    if not home or not os.path.isdir(home) or not os.access(home, os.W_OK):
+        env["HOME"] = tempfile.gettempdir()   # the compiler wants a writable HOME
+    start = time.time()
+    proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, env=env, text=True)
+    output: List[str] = []
+
+    def drain() -> None:
+        assert proc.stdout is not None
+        for line in proc.stdout:
+            output.append(line)
+
+    reader = threading.Thread(target=drain, daemon=True)
+    reader.start()
+    while True:
+        try:
+            proc.wait(timeout=15)
+            break
+        except subprocess.TimeoutExpired:
+            _say(f"still compiling {name}.hip for {ARCH} ({time.time() - start:.0f} s)")
+    reader.join()
+    if proc.returncode != 0:
+        if os.path.exists(tmp):
+            os.remove(tmp)
+        text = "".join(l for l in output if "packed-fp32-ops" not in l)
+        raise KernelBuildError(f"hipcc failed on {name}.hip (exit {proc.returncode}):\n{text}")
+    os.replace(tmp, so)
+    with open(so + ".digest.tmp", "w") as f:
+        f.write(source_digest(name))
+    os.replace(so + ".digest.tmp", so + ".digest")
+    _say(f"compiled {name}.hip in {time.time() - start:.1f} s -> {so}")
+    return so
+
+
+def build_all(names: Iterable[str] = SOURCES, force: bool = False, jobs: int = 4) -> Dict[str, str]:
+    """Compile the named sources (all by default); with ``force`` also those
+    that are up to date.  Returns ``{name: path}``."""
+    names = list(names)
+    todo = [n for n in names if force or _find_built(n) is None]
+    paths = {n: _find_built(n) for n in names if n not in todo}
+    if todo:
+        _say(f"compiling {len(todo)} kernel source(s) for {ARCH}: {', '.join(todo)}")
+        with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(todo)))) as pool:
+            for n, p in zip(todo, pool.map(compile_one, todo)):
+                paths[n] = p
+    return paths
+
+
+def load(name: str) -> ctypes.CDLL:
+    """The library of ``csrc/<name>.hip``, compiled first if need be."""
+    with _lock:
+        if name in _loaded:
+            return _loaded[name]
+        path = _find_built(name)
+        if path is None:
+            stale = _find_stale(name)
+            if stale is not None and find_hipcc() is None:
+                raise KernelBuildError(
+                    f"{stale} was built from other sources than the ones present and hipcc "
+                    "is not available to rebuild it")
+            path = compile_one(name)
+        lib = ctypes.CDLL(path)
+        _loaded[name] = lib
+        return lib

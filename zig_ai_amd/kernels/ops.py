@@ -1,0 +1,390 @@
+"""Python bindings of the HIP kernels: argument checks on the host, then one
+launch on torch's current stream.  Nothing here computes on the CPU and nothing
+falls back to a library: if a kernel library cannot be built or loaded the call
+raises.
+
+Shapes and dtypes are verified before every launch so that a kernel never sees
+operands other than the ones its indexing assumes.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Tuple
+
+import torch
+
+from . import build
+
+c_int, c_float, c_void_p, c_longlong = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_longlong
+
+_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+
+_SIGNATURES = {
+    ("norm", "za_add_rmsnorm"): [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p,
+                                 c_int, c_int, c_float, c_int, c_void_p],
+    ("norm", "za_embed_gather"): [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
+    ("gemm", "za_gemm_f32"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                              c_int, c_void_p],
+    ("gemm", "za_gemm_bf16"): [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                               c_int, c_void_p],
+    ("rope_kv", "za_qk_norm_rope_kv_write"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                              c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                              c_int, c_int, c_int, c_int, c_float, c_int, c_int,
+                                              c_void_p],
+    ("attention", "za_paged_attention"): [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                          c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p,
+                                          c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
+                                          c_int, c_int, c_int, c_void_p],
+    ("shortconv", "za_short_conv"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                     c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_longlong,
+                                     c_void_p],
+    ("activation", "za_swiglu"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    ("activation", "za_cast"): [c_void_p, c_int, c_void_p, c_int, c_longlong, c_void_p],
+    ("sampling", "za_argmax"): [c_void_p, c_int, c_int, c_void_p, c_void_p],
+    ("sampling", "za_sample"): [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                c_void_p, c_void_p],
+    ("sampling", "za_repetition_penalty"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                                            c_void_p],
+}
+_functions = {}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _fn(lib: str, name: str):
+    key = (lib, name)
+    f = _functions.get(key)
+    if f is None:
+        f = getattr(build.load(lib), name)
+        f.argtypes = _SIGNATURES[key]
+        f.restype = c_int
+        _functions[key] = f
+    return f
+
+
+def _check(rc: int, name: str, detail: str = "") -> None:
+    if rc == 0:
+        return
+    if rc == -1:
+        why = "bad argument"
+    elif rc == -2:
+        why = "size or dtype the kernel does not support"
+    else:
+        why = f"HIP error {rc}"
+    raise KernelError(f"{name}: {why}" + (f" ({detail})" if detail else ""))
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else c_void_p(t.data_ptr())
+
+
+def _stream():
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _code(dtype: torch.dtype) -> int:
+    if dtype not in _DTYPE_CODE:
+        raise KernelError(f"kernels take float32 or bfloat16, not {dtype}")
+    return _DTYPE_CODE[dtype]
+
+
+def _need(t: torch.Tensor, name: str, dtype=None, shape: Optional[Tuple[int, ...]] = None) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise KernelError(f"{name} is not a tensor")
+    if not t.is_cuda:
+        raise KernelError(f"{name} is on {t.device}; the kernels run on the GPU only")
+    if not t.is_contiguous():
+        raise KernelError(f"{name} is not contiguous")
+    if dtype is not None:
+        ok = t.dtype in dtype if isinstance(dtype, (tuple, list)) else t.dtype == dtype
+        if not ok:
+            raise KernelError(f"{name} has dtype {t.dtype}, expected {dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise KernelError(f"{name} has shape {tuple(t.shape)}, expected {tuple(shape)}")
+
+
+# --------------------------------------------------------------------- norms
+def add_rmsnorm(residual: Optional[torch.Tensor], delta: Optional[torch.Tensor],
+                weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+                rows: Optional[torch.Tensor] = None, write_residual: bool = True) -> torch.Tensor:
+    """``out = rmsnorm(residual + delta) * weight``; see csrc/norm.hip."""
+    if residual is None and delta is None:
+        raise KernelError("add_rmsnorm needs residual or delta")
+    ref = residual if residual is not None else delta
+    if ref.dim() != 2:
+        raise KernelError(f"add_rmsnorm takes [rows, width], got {tuple(ref.shape)}")
+    n, width = ref.shape
+    if residual is not None:
+        _need(residual, "residual", torch.float32, (n, width))
+    if delta is not None:
+        _need(delta, "delta", (torch.float32, torch.bfloat16), (n, width))
+    _need(weight, "weight", torch.float32, (width,))
+    n_out = n
+    if rows is not None:
+        _need(rows, "rows", torch.int32)
+        n_out = rows.numel()
+    out = torch.empty((n_out, width), dtype=out_dtype, device=ref.device)
+    rc = _fn("norm", "za_add_rmsnorm")(
+        _ptr(residual), _ptr(delta), _code(delta.dtype) if delta is not None else 0, _ptr(weight),
+        _ptr(out), _code(out_dtype), _ptr(rows), n_out, width, float(eps),
+        1 if (write_residual and residual is not None and delta is not None and rows is None) else 0,
+        _stream())
+    _check(rc, "add_rmsnorm")
+    return out
+
+
+def embed_gather(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """Rows of ``table`` as 32-bit floats: the start of the residual stream."""
+    _need(tokens, "tokens", torch.int32)
+    _need(table, "table", (torch.float32, torch.bfloat16))
+    if tokens.dim() != 1 or table.dim() != 2:
+        raise KernelError("embed_gather takes tokens [T] and table [vocab, width]")
+    vocab, width = table.shape
+    out = torch.empty((tokens.numel(), width), dtype=torch.float32, device=table.device)
+    rc = _fn("norm", "za_embed_gather")(_ptr(tokens), _ptr(table), _code(table.dtype), _ptr(out),
+                                        tokens.numel(), width, vocab, _stream())
+    _check(rc, "embed_gather")
+    return out
+
+
+# --------------------------------------------------------------------- gemm
+def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+           out_dtype: Optional[torch.dtype] = None, force_tiled: bool = False) -> torch.Tensor:
+    """``x [M, K] @ weight[N, K]^T + bias`` with 32-bit accumulation.
+
+    bfloat16 weights use the matrix-core kernels (``x`` must be bfloat16); 32-bit
+    weights use the all-32-bit kernel (``x`` may be either type and is widened)."""
+    if x.dim() != 2 or weight.dim() != 2:
+        raise KernelError(f"linear takes x [M, K] and weight [N, K], got {tuple(x.shape)} and "
+                          f"{tuple(weight.shape)}")
+    M, K = x.shape
+    N = weight.shape[0]
+    _need(x, "x", (torch.float32, torch.bfloat16))
+    _need(weight, "weight", (torch.float32, torch.bfloat16), (N, K))
+    if bias is not None:
+        _need(bias, "bias", torch.float32, (N,))
+    out_dtype = out_dtype or x.dtype
+    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    if weight.dtype == torch.float32:
+        rc = _fn("gemm", "za_gemm_f32")(_ptr(x), _code(x.dtype), _ptr(weight), _ptr(bias), _ptr(out),
+                                        _code(out_dtype), M, N, K, _stream())
+        _check(rc, "gemm_f32", f"M={M} N={N} K={K}")
+    else:
+        if x.dtype != torch.bfloat16:
+            raise KernelError("a bfloat16 weight needs bfloat16 activations")
+        if K % 8:
+            raise KernelError(f"the bfloat16 GEMM needs K to be a multiple of 8, got K={K}")
+        rc = _fn("gemm", "za_gemm_bf16")(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out),
+                                         _code(out_dtype), M, N, K, 1 if force_tiled else 0,
+                                         _stream())
+        _check(rc, "gemm_bf16", f"M={M} N={N} K={K}")
+    return out
+
+
+# ------------------------------------------------------------ rope + kv write
+def qk_norm_rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor,
+                          slots: Optional[torch.Tensor], q_norm_w: Optional[torch.Tensor],
+                          k_norm_w: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor],
+                          kv_cache: Optional[torch.Tensor], num_heads: int, num_kv_heads: int,
+                          head_dim: int, rotary_dim: int, adjacent_pairs: bool, eps: float,
+                          write_kv: bool = True) -> torch.Tensor:
+    """Returns the normalised, rotated queries ``[T, num_heads, head_dim]`` and
+    scatters keys/values into ``kv_cache [pages, 2, kv_heads, page_size, head_dim]``."""
+    T = qkv.shape[0]
+    total = num_heads + 2 * num_kv_heads
+    _need(qkv, "qkv", (torch.float32, torch.bfloat16), (T, total * head_dim))
+    _need(positions, "positions", torch.int32, (T,))
+    if head_dim > 256:
+        raise KernelError(f"head_dim {head_dim} exceeds the kernel's limit of 256")
+    if rotary_dim % 2 or not 0 <= rotary_dim <= head_dim:
+        raise KernelError(f"rotary_dim {rotary_dim} must be even and at most head_dim {head_dim}")
+    for name, w in (("q_norm_w", q_norm_w), ("k_norm_w", k_norm_w)):
+        if w is not None:
+            _need(w, name, torch.float32, (head_dim,))
+    if rotary_dim:
+        _need(inv_freq, "inv_freq", torch.float32, (rotary_dim // 2,))
+    page_size = 0
+    if write_kv:
+        if kv_cache is None or slots is None:
+            raise KernelError("write_kv needs kv_cache and slots")
+        _need(slots, "slots", torch.int32, (T,))
+        _need(kv_cache, "kv_cache", qkv.dtype)
+        if kv_cache.dim() != 5 or kv_cache.shape[1] != 2 or kv_cache.shape[2] != num_kv_heads \
+                or kv_cache.shape[4] != head_dim:
+            raise KernelError(f"kv_cache has shape {tuple(kv_cache.shape)}, expected "
+                              f"[pages, 2, {num_kv_heads}, page_size, {head_dim}]")
+        page_size = kv_cache.shape[3]
+    q_out = torch.empty((T, num_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
+    rc = _fn("rope_kv", "za_qk_norm_rope_kv_write")(
+        _ptr(qkv), _ptr(positions), _ptr(slots) if write_kv else None, _ptr(q_norm_w),
+        _ptr(k_norm_w), _ptr(inv_freq) if rotary_dim else None, _ptr(q_out),
+        _ptr(kv_cache) if write_kv else None, _code(qkv.dtype), T, num_heads, num_kv_heads,
+        head_dim, rotary_dim, 1 if adjacent_pairs else 0, float(eps), page_size,
+        1 if write_kv else 0, _stream())
+    _check(rc, "qk_norm_rope_kv_write")
+    return q_out
+
+
+# ----------------------------------------------------------------- attention
+ATTENTION_MAX_ROWS = 32
+
+
+def paged_attention(q: torch.Tensor, kv_cache: torch.Tensor, block_table: torch.Tensor,
+                    positions: torch.Tensor, item_seq: torch.Tensor, item_row0: torch.Tensor,
+                    item_count: torch.Tensor, n_items: int, scale: float, window: int = 0,
+                    keys_per_split: int = 0, nsplit: int = 1,
+                    workspace: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> torch.Tensor:
+    """Causal attention of ``q [T, heads, head_dim]`` over the cache; see
+    csrc/attention.hip.  ``item_*`` list the work items: the request (row of
+    ``block_table``), the first query row and the number of consecutive query
+    rows, at most ``ATTENTION_MAX_ROWS // (heads // kv_heads)`` each."""
+    if q.dim() != 3:
+        raise KernelError(f"q must be [T, heads, head_dim], got {tuple(q.shape)}")
+    T, nh, d = q.shape
+    _need(q, "q", (torch.float32, torch.bfloat16))
+    _need(kv_cache, "kv_cache", q.dtype)
+    if kv_cache.dim() != 5 or kv_cache.shape[1] != 2 or kv_cache.shape[4] != d:
+        raise KernelError(f"kv_cache has shape {tuple(kv_cache.shape)}, expected "
+                          f"[pages, 2, kv_heads, page_size, {d}]")
+    nkv, page_size = kv_cache.shape[2], kv_cache.shape[3]
+    if nh % nkv:
+        raise KernelError(f"{nh} heads do not divide into {nkv} key/value heads")
+    if nh // nkv > ATTENTION_MAX_ROWS:
+        raise KernelError(f"{nh // nkv} query heads per key/value head exceed the kernel's "
+                          f"limit of {ATTENTION_MAX_ROWS}")
+    if d % 8 or d > 256:
+        raise KernelError(f"head_dim {d} must be a multiple of 8 and at most 256")
+    _need(block_table, "block_table", torch.int32)
+    if block_table.dim() != 2:
+        raise KernelError("block_table must be [requests, max_pages]")
+    _need(positions, "positions", torch.int32, (T,))
+    for name, t in (("item_seq", item_seq), ("item_row0", item_row0), ("item_count", item_count)):
+        _need(t, name, torch.int32)
+        if t.numel() < n_items:
+            raise KernelError(f"{name} holds {t.numel()} entries, fewer than {n_items} items")
+    out = torch.empty_like(q)
+    part_acc = part_ml = None
+    if nsplit > 1:
+        if keys_per_split <= 0 or keys_per_split % 64:
+            raise KernelError("keys_per_split must be a positive multiple of 64")
+        if workspace is not None:
+            part_acc, part_ml = workspace
+            _need(part_acc, "part_acc", torch.float32)
+            _need(part_ml, "part_ml", torch.float32)
+            if part_acc.numel() < T * nh * nsplit * d or part_ml.numel() < T * nh * nsplit * 2:
+                raise KernelError("attention workspace is too small")
+        else:
+            part_acc = torch.empty((T, nh, nsplit, d), dtype=torch.float32, device=q.device)
+            part_ml = torch.empty((T, nh, nsplit, 2), dtype=torch.float32, device=q.device)
+    rc = _fn("attention", "za_paged_attention")(
+        _ptr(q), _ptr(out), _ptr(kv_cache), _ptr(block_table), block_table.shape[1],
+        _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
+        _ptr(part_acc), _ptr(part_ml), _code(q.dtype), nh, nkv, d, page_size, float(scale),
+        int(window), int(keys_per_split), int(nsplit), _stream())
+    _check(rc, "paged_attention")
+    return out
+
+
+# ---------------------------------------------------------------- short conv
+def short_conv(z: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+               state: torch.Tensor, token_seq: torch.Tensor, seq_start: torch.Tensor,
+               slot_id: torch.Tensor) -> torch.Tensor:
+    """Gated causal depth-wise convolution with carried state; see
+    csrc/shortconv.hip.  ``z [T, 3*width]``, ``weight [width, L]``,
+    ``state [slots, width, L]`` (updated in place; slots may be spaced
+    further apart than ``width * L`` floats)."""
+    T = z.shape[0]
+    width, L = weight.shape
+    _need(z, "z", (torch.float32, torch.bfloat16), (T, 3 * width))
+    _need(weight, "weight", torch.float32)
+    if L > 8:
+        raise KernelError(f"convolution length {L} exceeds the kernel's limit of 8")
+    if bias is not None:
+        _need(bias, "bias", torch.float32, (width,))
+    if not (isinstance(state, torch.Tensor) and state.is_cuda and state.dtype == torch.float32):
+        raise KernelError("state must be a float32 tensor on the GPU")
+    if state.dim() != 3 or tuple(state.shape[1:]) != (width, L):
+        raise KernelError(f"state has shape {tuple(state.shape)}, expected [slots, {width}, {L}]")
+    if state.stride(2) != 1 or state.stride(1) != L or state.stride(0) < width * L:
+        raise KernelError(f"state has strides {state.stride()}; a slot must be laid out "
+                          f"[{width}, {L}] contiguously")
+    _need(token_seq, "token_seq", torch.int32, (T,))
+    _need(seq_start, "seq_start", torch.int32)
+    _need(slot_id, "slot_id", torch.int32)
+    y = torch.empty((T, width), dtype=z.dtype, device=z.device)
+    rc = _fn("shortconv", "za_short_conv")(_ptr(z), _ptr(weight), _ptr(bias), _ptr(state),
+                                           _ptr(token_seq), _ptr(seq_start), _ptr(slot_id), _ptr(y),
+                                           _code(z.dtype), T, width, L, state.stride(0), _stream())
+    _check(rc, "short_conv")
+    return y
+
+
+# ---------------------------------------------------------------- activation
+def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
+    """``silu(gate) * up`` for ``gate_up = [gate | up]`` of shape ``[T, 2*I]``."""
+    _need(gate_up, "gate_up", (torch.float32, torch.bfloat16))
+    if gate_up.dim() != 2 or gate_up.shape[1] % 2:
+        raise KernelError(f"swiglu takes [T, 2*I], got {tuple(gate_up.shape)}")
+    T, two_i = gate_up.shape
+    out = torch.empty((T, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
+    rc = _fn("activation", "za_swiglu")(_ptr(gate_up), _ptr(out), _code(gate_up.dtype), T,
+                                        two_i // 2, _stream())
+    _check(rc, "swiglu")
+    return out
+
+
+def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """Element-wise conversion between float32 and bfloat16 (round to nearest even)."""
+    _need(x, "x", (torch.float32, torch.bfloat16))
+    if x.dtype == dtype:
+        return x
+    out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    rc = _fn("activation", "za_cast")(_ptr(x), _code(x.dtype), _ptr(out), _code(dtype), x.numel(),
+                                      _stream())
+    _check(rc, "cast")
+    return out
+
+
+# ------------------------------------------------------------------ sampling
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    _need(logits, "logits", torch.float32)
+    if logits.dim() != 2:
+        raise KernelError("argmax takes [rows, vocab]")
+    out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
+    rc = _fn("sampling", "za_argmax")(_ptr(logits), logits.shape[0], logits.shape[1], _ptr(out),
+                                      _stream())
+    _check(rc, "argmax")
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
+           top_p: torch.Tensor, uniform: torch.Tensor) -> torch.Tensor:
+    _need(logits, "logits", torch.float32)
+    if logits.dim() != 2:
+        raise KernelError("sample takes [rows, vocab]")
+    R = logits.shape[0]
+    _need(temperature, "temperature", torch.float32, (R,))
+    _need(top_k, "top_k", torch.int32, (R,))
+    _need(top_p, "top_p", torch.float32, (R,))
+    _need(uniform, "uniform", torch.float32, (R,))
+    out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    rc = _fn("sampling", "za_sample")(_ptr(logits), R, logits.shape[1], _ptr(temperature),
+                                      _ptr(top_k), _ptr(top_p), _ptr(uniform), _ptr(out), _stream())
+    _check(rc, "sample")
+    return out
+
+
+def repetition_penalty_(logits: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor,
+                        factors: torch.Tensor) -> None:
+    """In place; each (row, token) pair may be listed once."""
+    _need(logits, "logits", torch.float32)
+    n = rows.numel()
+    _need(rows, "rows", torch.int32, (n,))
+    _need(tokens, "tokens", torch.int32, (n,))
+    _need(factors, "factors", torch.float32, (n,))
+    rc = _fn("sampling", "za_repetition_penalty")(_ptr(logits), logits.shape[1], _ptr(rows),
+                                                  _ptr(tokens), _ptr(factors), n, _stream())
+    _check(rc, "repetition_penalty")

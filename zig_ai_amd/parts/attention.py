@@ -1,0 +1,143 @@
+"""Grouped-query attention over a paged cache, as a part.
+
+Per token (/root/reference/src/transformer/hybrid_attn.zig:286-640):
+  q, k, v = x Wq^T, x Wk^T, x Wv^T           (one fused projection, optional bias)
+  q, k    = per-head RMSNorm(q), RMSNorm(k)  if ``qk_norm``   (371-382)
+  q, k    = position encoding(q, k)          (rotary: fused into the same kernel)
+  k, v   -> the request's pages
+  o       = softmax(q k^T * scale, causal [, window]) v       (553-608)
+  y       = o Wo^T
+
+All sizes come from ``params``: ``hidden_size, num_heads, num_kv_heads,
+head_dim, qk_norm, norm_eps, window`` (0 = all keys), ``softmax_scale`` (None =
+1/sqrt(head_dim)), ``bias`` and ``position`` (a nested position-encoding spec or
+None).
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Any, Dict, Mapping
+
+import torch
+
+from ..kernels import ops
+from .base import (Mixer, PagedNeed, Runtime, TensorRule, lookup, register_mixer)
+from .feed_forward import fuse_rows
+
+# Contexts shorter than this are never cut; longer ones are cut into ranges of
+# this many keys (doubled while that would make more than SPLIT_MAX ranges).
+SPLIT_KEYS = 256
+SPLIT_MAX = 64
+# Enough workgroups to occupy the machine without cutting contexts.
+BUSY_WORKGROUPS = 1024
+
+
+def plan_split(n_items: int, num_kv_heads: int, max_keys: int):
+    """(keys per range, number of ranges) for one launch.  Cutting pays only when
+    the launch would otherwise leave most of the machine idle (decoding)."""
+    if n_items * num_kv_heads >= BUSY_WORKGROUPS or max_keys <= 2 * SPLIT_KEYS:
+        return 0, 1
+    keys = SPLIT_KEYS
+    while (max_keys + keys - 1) // keys > SPLIT_MAX:
+        keys *= 2
+    return keys, (max_keys + keys - 1) // keys
+
+
+class GroupedQueryAttention(Mixer):
+    kind = "gqa_attention"
+    kernel_sources = ("gemm", "rope_kv", "attention", "norm")
+
+    @classmethod
+    def tensor_rules(cls, params: Mapping[str, Any]) -> Dict[str, TensorRule]:
+        H, nh, nkv, d = (int(params[k]) for k in
+                         ("hidden_size", "num_heads", "num_kv_heads", "head_dim"))
+        rules = {"q_proj.weight": TensorRule(((nh * d, H),)),
+                 "k_proj.weight": TensorRule(((nkv * d, H),)),
+                 "v_proj.weight": TensorRule(((nkv * d, H),)),
+                 "out_proj.weight": TensorRule(((H, nh * d),))}
+        if params.get("qk_norm"):
+            rules["q_norm.weight"] = TensorRule(((d,),), role="norm")
+            rules["k_norm.weight"] = TensorRule(((d,),), role="norm")
+        if params.get("bias"):
+            rules["q_proj.bias"] = TensorRule(((nh * d,),), role="bias")
+            rules["k_proj.bias"] = TensorRule(((nkv * d,),), role="bias")
+            rules["v_proj.bias"] = TensorRule(((nkv * d,),), role="bias")
+            rules["out_proj.bias"] = TensorRule(((H,),), role="bias")
+        return rules
+
+    @classmethod
+    def cache_need(cls, params: Mapping[str, Any]):
+        return PagedNeed(int(params["num_kv_heads"]), int(params["head_dim"]),
+                         int(params.get("window") or 0))
+
+    def __init__(self, params, tensors, runtime: Runtime):
+        super().__init__(params, tensors, runtime)
+        self.num_heads = int(params["num_heads"])
+        self.num_kv_heads = int(params["num_kv_heads"])
+        self.head_dim = int(params["head_dim"])
+        if self.num_heads % self.num_kv_heads:
+            raise ValueError(f"{self.num_heads} heads do not divide into {self.num_kv_heads} groups")
+        self.group = self.num_heads // self.num_kv_heads
+        if self.group > ops.ATTENTION_MAX_ROWS:
+            raise ValueError(f"{self.group} query heads per key/value head exceed the attention "
+                             f"kernel's limit of {ops.ATTENTION_MAX_ROWS}")
+        if self.head_dim % 16 or self.head_dim > 256:
+            raise ValueError(f"head_dim {self.head_dim} must be a multiple of 16, at most 256")
+        self.rows_per_item = max(1, ops.ATTENTION_MAX_ROWS // self.group)
+        self.window = int(params.get("window") or 0)
+        scale = params.get("softmax_scale")
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
+        self.eps = float(params.get("norm_eps", 0.0))
+        self.w_qkv = fuse_rows(tensors["q_proj.weight"], tensors["k_proj.weight"],
+                               tensors["v_proj.weight"])
+        self.w_out = tensors["out_proj.weight"]
+        self.b_qkv = self.b_out = None
+        if params.get("bias"):
+            self.b_qkv = torch.cat([tensors["q_proj.bias"], tensors["k_proj.bias"],
+                                    tensors["v_proj.bias"]]).contiguous()
+            self.b_out = tensors["out_proj.bias"]
+        self.q_norm = tensors.get("q_norm.weight") if params.get("qk_norm") else None
+        self.k_norm = tensors.get("k_norm.weight") if params.get("qk_norm") else None
+        pos = params.get("position")
+        self.position = None
+        if pos is not None:
+            self.position = lookup("position", pos.kind)(pos.params, {}, runtime)
+        self.fused_rotation = bool(getattr(self.position, "fused_rotation", False))
+
+    def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
+        nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
+        T = x.shape[0]
+        qkv = ops.linear(x, self.w_qkv, self.b_qkv)
+        slots = step.slot_mapping[cache.group]
+        if self.position is None or self.fused_rotation:
+            rot = self.position.rotary_dim if self.position is not None else 0
+            q = ops.qk_norm_rope_kv_write(
+                qkv, step.positions, slots, self.q_norm, self.k_norm,
+                self.position.inv_freq if rot else None, cache.kv, nh, nkv, d, rot,
+                bool(rot) and self.position.pairing == "adjacent", self.eps,
+                write_kv=cache.writes)
+        else:
+            # Any other encoding: norm with the norm kernel, encode through the
+            # part's own ``apply``, then let the fused kernel store what it is given.
+            heads = qkv.view(T, nh + 2 * nkv, d)
+            qh, kh, vh = heads[:, :nh], heads[:, nh:nh + nkv], heads[:, nh + nkv:]
+            if self.q_norm is not None:
+                qh = ops.add_rmsnorm(None, qh.reshape(-1, d).contiguous(), self.q_norm, self.eps,
+                                     qkv.dtype).view(T, nh, d)
+                kh = ops.add_rmsnorm(None, kh.reshape(-1, d).contiguous(), self.k_norm, self.eps,
+                                     qkv.dtype).view(T, nkv, d)
+            qh, kh = self.position.apply(qh, kh, step.positions)
+            packed = torch.cat([qh.to(qkv.dtype), kh.to(qkv.dtype), vh], dim=1).reshape(T, -1)
+            q = ops.qk_norm_rope_kv_write(packed.contiguous(), step.positions, slots, None, None,
+                                          None, cache.kv, nh, nkv, d, 0, False, self.eps,
+                                          write_kv=cache.writes)
+        item_seq, item_row0, item_count, n_items = step.attention_items(self.rows_per_item)
+        keys, nsplit = plan_split(n_items, nkv, step.max_keys)
+        o = ops.paged_attention(q, cache.kv, step.block_tables[cache.group], step.positions,
+                                item_seq, item_row0, item_count, n_items, self.scale, self.window,
+                                keys, nsplit)
+        return ops.linear(o.view(T, nh * d), self.w_out, self.b_out)
+
+
+register_mixer(GroupedQueryAttention.kind, GroupedQueryAttention)

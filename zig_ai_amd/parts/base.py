@@ -1,0 +1,176 @@
+"""Interfaces every part obeys, and the registries that map a ``PartSpec.kind``
+to its class.
+
+A part knows its own sizes and constants (``params``) and its own tensors; it
+never learns which model it is in.  Five families exist:
+
+  mixer              ``forward(x, step, cache) -> y``; declares a cache need
+  feed-forward       ``forward(x, step) -> y``
+  norm               ``forward(x) -> y`` and ``add_forward(residual, delta) -> y``
+  position encoding  used by mixers: a rotation table, or ``apply(q, k, positions)``
+  arrangement        wires two norms, a mixer and a feed-forward into a block
+
+plus the embedding and the output head.  All ``forward`` functions take packed
+token rows ``[T, width]``: the tokens of every request in the step, one after
+the other; ``step`` says where each request's rows begin and what it has cached.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Callable, Dict, Mapping, Optional, Tuple
+
+import torch
+
+
+# --------------------------------------------------------------- tensor rules
+@dataclass(frozen=True)
+class TensorRule:
+    """What a part expects of one of its tensors.
+
+    ``shapes``: accepted stored shapes; the part receives the tensor reshaped
+    to the first.  ``stored_shape``: the shape the random model writer stores
+    (the first accepted shape if not given).  ``role`` picks the initialiser and the precision the tensor
+    is kept in: ``matrix`` and ``table`` stay in their stored dtype (bfloat16
+    stays bfloat16, 32-bit stays 32-bit); ``norm``, ``bias`` and ``filter`` are
+    small vectors that are always held in 32-bit.
+    """
+
+    shapes: Tuple[Tuple[int, ...], ...]
+    role: str = "matrix"
+    required: bool = True
+    stored_shape: Optional[Tuple[int, ...]] = None
+
+
+# ---------------------------------------------------------------- cache needs
+@dataclass(frozen=True)
+class PagedNeed:
+    """Keys and values per token: ``num_kv_heads * head_dim`` of each.  With
+    ``window > 0`` only the last ``window`` positions are ever read, so older
+    pages can be given back."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: int = 0
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """Per-request state of fixed size (32-bit floats), zero for a new request."""
+
+    shape: Tuple[int, ...]
+
+
+# ------------------------------------------------------------------- runtime
+@dataclass
+class Runtime:
+    """Where and how parts compute: the device, and the storage dtype of
+    activations (``torch.bfloat16`` for serving, ``torch.float32`` for the
+    all-32-bit path)."""
+
+    device: torch.device
+    dtype: torch.dtype
+
+
+class Part:
+    """Base of all parts.  Subclasses set ``kind`` and implement
+    ``tensor_rules``; their constructor receives tensors already placed on the
+    device in the precision their role prescribes."""
+
+    kind: str = ""
+
+    @classmethod
+    def tensor_rules(cls, params: Mapping[str, Any]) -> Dict[str, TensorRule]:
+        return {}
+
+    def __init__(self, params: Mapping[str, Any], tensors: Mapping[str, torch.Tensor],
+                 runtime: Runtime):
+        self.params = dict(params)
+        self.runtime = runtime
+
+
+class Mixer(Part):
+    @classmethod
+    def cache_need(cls, params: Mapping[str, Any]):
+        """``PagedNeed``, ``StateNeed`` or ``None``."""
+        return None
+
+    def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, step) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+    def add_forward(self, residual: torch.Tensor, delta: Optional[torch.Tensor],
+                    rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``residual`` (32-bit, updated in place) takes ``delta``; the result is
+        the norm of the sum.  With ``rows`` only those rows are produced and
+        ``residual`` is left alone.  Parts with a fused kernel override this."""
+        if rows is not None:
+            h = residual.index_select(0, rows.long())
+            if delta is not None:
+                h = h + delta.index_select(0, rows.long()).float()
+            return self.forward(h)
+        if delta is not None:
+            residual.add_(delta.float())
+        return self.forward(residual)
+
+
+class PositionEncoding(Part):
+    def apply(self, q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor):
+        """Generic path: return encoded ``(q, k)`` of shape ``[T, heads, head_dim]``."""
+        raise NotImplementedError
+
+
+# ---------------------------------------------------------------- registries
+_REGISTRIES: Dict[str, Dict[str, Any]] = {
+    "mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "arrangement": {},
+    "embedding": {}, "head": {},
+}
+
+
+def _register(family: str, kind: str, obj: Any) -> Any:
+    _REGISTRIES[family][kind] = obj
+    return obj
+
+
+def register_mixer(kind: str, cls: Any) -> Any:
+    return _register("mixer", kind, cls)
+
+
+def register_feed_forward(kind: str, cls: Any) -> Any:
+    return _register("feed_forward", kind, cls)
+
+
+def register_norm(kind: str, cls: Any) -> Any:
+    return _register("norm", kind, cls)
+
+
+def register_position(kind: str, cls: Any) -> Any:
+    return _register("position", kind, cls)
+
+
+def register_arrangement(kind: str, cls: Any) -> Any:
+    return _register("arrangement", kind, cls)
+
+
+def register_embedding(kind: str, cls: Any) -> Any:
+    return _register("embedding", kind, cls)
+
+
+def register_head(kind: str, cls: Any) -> Any:
+    return _register("head", kind, cls)
+
+
+def lookup(family: str, kind: str) -> Any:
+    table = _REGISTRIES[family]
+    if kind not in table:
+        raise KeyError(f"no {family} part named {kind!r}; registered: {', '.join(sorted(table))}")
+    return table[kind]

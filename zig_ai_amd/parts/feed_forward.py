@@ -1,0 +1,43 @@
+"""Dense SwiGLU feed-forward: ``(silu(x Wg^T) * (x Wu^T)) Wd^T`` without biases
+(/root/reference/src/transformer/ffn.zig:19-33).  Gate and up weights are fused
+into one ``[2I, H]`` matrix at load so the input is read once."""
+
+from __future__ import annotations
+
+from typing import Any, Dict, Mapping
+
+import torch
+
+from ..kernels import ops
+from .base import FeedForward, Runtime, TensorRule, register_feed_forward
+
+
+def fuse_rows(*mats: torch.Tensor) -> torch.Tensor:
+    """Stack weight matrices along the output dimension; mixed precisions are
+    widened to 32-bit rather than narrowed."""
+    if len({m.dtype for m in mats}) > 1:
+        mats = tuple(m.float() for m in mats)
+    return torch.cat(mats, dim=0).contiguous()
+
+
+class SwiGLU(FeedForward):
+    kind = "swiglu"
+    kernel_sources = ("gemm", "activation")
+
+    @classmethod
+    def tensor_rules(cls, params: Mapping[str, Any]) -> Dict[str, TensorRule]:
+        H, I = int(params["hidden_size"]), int(params["intermediate_size"])
+        return {"gate.weight": TensorRule(((I, H),)), "up.weight": TensorRule(((I, H),)),
+                "down.weight": TensorRule(((H, I),))}
+
+    def __init__(self, params, tensors, runtime: Runtime):
+        super().__init__(params, tensors, runtime)
+        self.gate_up = fuse_rows(tensors["gate.weight"], tensors["up.weight"])
+        self.down = tensors["down.weight"]
+
+    def forward(self, x: torch.Tensor, step=None) -> torch.Tensor:
+        gu = ops.linear(x, self.gate_up)
+        return ops.linear(ops.swiglu(gu), self.down)
+
+
+register_feed_forward(SwiGLU.kind, SwiGLU)

@@ -1,0 +1,66 @@
+"""The ShortConv mixer as a part: ``in_proj -> (B, C, x)``, ``u = B * x``, a
+causal depth-wise convolution of ``kernel_size`` taps over the request's own
+inputs (the last ones carried in a fixed-size state slot), ``y = C * conv(u)``,
+``out_proj``.  Biases on the three linear/conv maps when ``bias`` is set and the
+checkpoint holds them.
+
+The carried-state mechanics follow the reference's convolution
+(/root/reference/src/transformer/short_conv.zig:188-225: taps over [state rows;
+new rows], state <- last rows); the order project-gate-convolve-gate-project is
+the model's definition, which the reference's layer does not follow
+(short_conv.zig:174-277 convolves first and gates with SiLU).
+"""
+
+from __future__ import annotations
+
+from typing import Any, Dict, Mapping
+
+import torch
+
+from ..kernels import ops
+from .base import Mixer, Runtime, StateNeed, TensorRule, register_mixer
+
+
+class ShortConv(Mixer):
+    kind = "short_conv"
+    kernel_sources = ("gemm", "shortconv")
+
+    @classmethod
+    def tensor_rules(cls, params: Mapping[str, Any]) -> Dict[str, TensorRule]:
+        H, L = int(params["hidden_size"]), int(params["kernel_size"])
+        rules = {"in_proj.weight": TensorRule(((3 * H, H),)),
+                 "conv.weight": TensorRule(((H, L), (H, 1, L)), role="filter",
+                                           stored_shape=(H, 1, L)),
+                 "out_proj.weight": TensorRule(((H, H),))}
+        if params.get("bias"):
+            rules["conv.bias"] = TensorRule(((H,),), role="bias")
+            # the projections' biases are used when the checkpoint has them
+            rules["in_proj.bias"] = TensorRule(((3 * H,),), role="bias", required=False)
+            rules["out_proj.bias"] = TensorRule(((H,),), role="bias", required=False)
+        return rules
+
+    @classmethod
+    def cache_need(cls, params: Mapping[str, Any]):
+        return StateNeed((int(params["hidden_size"]), int(params["kernel_size"])))
+
+    def __init__(self, params, tensors, runtime: Runtime):
+        super().__init__(params, tensors, runtime)
+        self.hidden = int(params["hidden_size"])
+        self.kernel_size = int(params["kernel_size"])
+        if self.kernel_size > 8:
+            raise ValueError(f"conv kernel_size {self.kernel_size} exceeds the kernel's limit of 8")
+        self.w_in = tensors["in_proj.weight"]
+        self.w_out = tensors["out_proj.weight"]
+        self.w_conv = tensors["conv.weight"].reshape(self.hidden, self.kernel_size).contiguous()
+        self.b_in = tensors.get("in_proj.bias")
+        self.b_conv = tensors.get("conv.bias")
+        self.b_out = tensors.get("out_proj.bias")
+
+    def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
+        z = ops.linear(x, self.w_in, self.b_in)
+        y = ops.short_conv(z, self.w_conv, self.b_conv, cache.state, step.token_seq,
+                           step.seq_start, step.slot_id)
+        return ops.linear(y, self.w_out, self.b_out)
+
+
+register_mixer(ShortConv.kind, ShortConv)
