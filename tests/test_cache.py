@@ -1,0 +1,174 @@
+"""The cache manager on the CPU: no page lost, held twice or freed twice, under
+random orders of requests; block tables; windows; slots."""
+
+import random
+
+import pytest
+
+from zig_ai_amd.cache import FREED, CacheManager, OutOfPages, OutOfSlots, Pool, PoolError
+from zig_ai_amd.parts import PagedNeed, StateNeed
+
+
+def manager(num_pages=16, page_size=4, num_slots=4, window=0, extra=None):
+    needs = {0: StateNeed((8, 3)), 1: PagedNeed(2, 16, 0), 2: StateNeed((8, 3)), 3: PagedNeed(2, 16, 0)}
+    if window:
+        needs[4] = PagedNeed(2, 16, window)
+    needs.update(extra or {})
+    return CacheManager(needs, page_size, num_pages, num_slots, allocate=False)
+
+
+def test_pool_counts_like_the_reference():
+    """/root/reference/tests/test_paged_attention.zig:18-30: 16 -> alloc -> 15 -> release -> 16."""
+    p = Pool(16)
+    assert p.free_count == 16
+    page = p.take("x")
+    assert p.free_count == 15 and p.owner_of(page) == "x"
+    p.give(page, "x")
+    assert p.free_count == 16
+    p.check()
+
+
+def test_pool_refuses_double_free_and_foreign_free():
+    p = Pool(4)
+    a = p.take("x")
+    with pytest.raises(PoolError, match="belongs"):
+        p.give(a, "y")
+    p.give(a, "x")
+    with pytest.raises(PoolError, match="twice"):
+        p.give(a, "x")
+    with pytest.raises(PoolError, match="exist"):
+        p.give(9, "x")
+    for _ in range(4):
+        p.take("z")
+    with pytest.raises(OutOfPages):
+        p.take("z")
+    with pytest.raises(OutOfPages):
+        Pool(2).take_many("q", 3)
+
+
+def test_block_table_growth_like_the_reference():
+    """/root/reference/tests/test_paged_attention.zig:32-58 and
+    test_paged_attention_gpu.zig:51,294: 5 tokens at page 4 -> 2 pages, 7 -> 2, 9 -> 3;
+    40 at 16 -> 3; 4096 at 16 -> 256."""
+    for tokens, page, want in [(5, 4, 2), (7, 4, 2), (9, 4, 3), (40, 16, 3), (4096, 16, 256)]:
+        m = CacheManager({0: PagedNeed(1, 16)}, page, 300, 1, allocate=False)
+        m.admit("r")
+        m.reserve("r", tokens)
+        assert len(m.table("r", 0)) == want
+    m = manager(page_size=4)
+    m.admit("r")
+    m.reserve("r", 4)
+    m.commit("r", 4)
+    assert len(m.table("r", 0)) == 1
+    m.reserve("r", 1)                      # the fifth token opens a new page
+    assert len(m.table("r", 0)) == 2
+    m.commit("r", 1)
+    assert m.token_slots("r", 0, 0, 5) == [m.table("r", 0)[0] * 4 + i for i in range(4)] + \
+        [m.table("r", 0)[1] * 4]
+
+
+def test_groups_and_views():
+    m = manager(window=6)
+    assert len(m.groups) == 2                      # all keys; a window of keys
+    assert m.groups[0].cache_ids == [1, 3] and m.groups[1].cache_ids == [4]
+    assert m.view(1).kind == "paged" and m.view(1).group == 0 and m.view(4).group == 1
+    assert m.view(0).kind == "state" and m.view(7).kind == "none"
+    assert m.floats_per_slot == 2 * 8 * 3
+
+
+def test_reserve_is_all_or_nothing():
+    m = manager(num_pages=4, window=6)
+    m.admit("a")
+    m.admit("b")
+    m.reserve("a", 12)                              # 3 of 4 pages in both groups
+    with pytest.raises(OutOfPages):
+        m.reserve("b", 8)                           # needs 2
+    assert m.table("b", 0) == [] and m.table("b", 1) == []
+    assert not m.can_reserve("b", 8) and m.can_reserve("b", 4)
+    assert not m.can_reserve("b", 4, spare={0: 1})
+    m.check()
+
+
+def test_window_gives_pages_back():
+    m = manager(num_pages=8, page_size=4, window=6)
+    m.admit("r")
+    for step in range(40):
+        m.reserve("r", 1)
+        m.commit("r", 1)
+        m.check()
+        n = step + 1
+        table = m.table("r", 1)
+        first_needed = max(0, n - 6 + 1)
+        for p, page in enumerate(table):
+            assert (page == FREED) == ((p + 1) * 4 <= first_needed), (n, p)
+        assert len(m.table("r", 0)) == (n + 3) // 4 and FREED not in m.table("r", 0)
+        if n >= 32:
+            break
+    assert m.groups[1].pool.high_water <= 3           # never more than window/page + 2 pages
+    with pytest.raises(PoolError, match="given back"):
+        m.token_slots("r", 1, 0, 1)
+    m.release("r")
+    assert all(g.pool.free_count == g.pool.size for g in m.groups)
+
+
+def test_commit_beyond_reservation_is_an_error():
+    m = manager()
+    m.admit("r")
+    m.reserve("r", 3)
+    with pytest.raises(PoolError, match="beyond"):
+        m.commit("r", 5)
+
+
+def test_slots():
+    m = manager(num_slots=2)
+    assert m.admit("a") != m.admit("b")
+    with pytest.raises(OutOfSlots):
+        m.admit("c")
+    with pytest.raises(PoolError, match="already"):
+        m.admit("a")
+    m.release("a")
+    m.admit("c")
+    m.check()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_orders_keep_the_books(seed):
+    """Admissions, portions, decoding, finishing in random order: after every
+    action free + owned = total, no page in two tables, tables match the pools."""
+    rng = random.Random(seed)
+    m = manager(num_pages=24, page_size=4, num_slots=5, window=rng.choice([0, 5, 9]))
+    live, next_id = {}, 0
+    for _ in range(600):
+        action = rng.random()
+        if action < 0.25 and len(live) < 5:
+            m.admit(next_id)
+            live[next_id] = 0
+            next_id += 1
+        elif action < 0.85 and live:
+            r = rng.choice(list(live))
+            n = rng.choice([1, 1, 1, 2, 3, 7, 16])
+            try:
+                m.reserve(r, n)
+            except OutOfPages:
+                victim = rng.choice(list(live))       # what a scheduler would do: evict one
+                m.release(victim)
+                del live[victim]
+                m.check()
+                continue
+            m.commit(r, n)
+            live[r] += n
+            assert m.num_tokens(r) == live[r]
+        elif live:
+            r = rng.choice(list(live))
+            m.release(r)
+            del live[r]
+        m.check()
+        for g in m.groups:
+            held = sum(1 for r in live for p in m.table(r, g.index) if p != FREED)
+            assert held + g.pool.free_count == g.pool.size
+    for r in list(live):
+        m.release(r)
+    m.check()
+    assert all(g.pool.free_count == g.pool.size for g in m.groups)
+    assert m.slots.free_count == 5
+    assert m.pages_reused > 0

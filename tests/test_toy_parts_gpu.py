@@ -1,0 +1,173 @@
+"""Extending the framework from outside: a toy mixer with state of its own and a
+toy architecture around it, both defined here, are registered, built from a
+model folder, and stepped through the engine's step function, cache manager and
+run order without a change to the framework's files.  Also: a run order that
+names a layer twice, and a layer that reads another layer's cache.
+"""
+
+import pytest
+import torch
+
+import engine_util as eu
+import plain_lfm2 as plain
+
+pytestmark = pytest.mark.gpu
+
+
+# --------------------------------------------------------------- the toy mixer
+def toy_classes():
+    from zig_ai_amd.kernels import ops
+    from zig_ai_amd.parts import Mixer, StateNeed, TensorRule, register_mixer
+
+    class RunningMeanMixer(Mixer):
+        """y[t] = W * mean(x[0..t]): needs the sum of all earlier inputs and their
+        count, a state of ``width + 1`` floats per request."""
+        kind = "toy_running_mean"
+        kernel_sources = ("gemm",)
+
+        @classmethod
+        def tensor_rules(cls, params):
+            w = int(params["width"])
+            return {"mix.weight": TensorRule(((w, w),))}
+
+        @classmethod
+        def cache_need(cls, params):
+            return StateNeed((int(params["width"]) + 1,))
+
+        def __init__(self, params, tensors, runtime):
+            super().__init__(params, tensors, runtime)
+            self.width = int(params["width"])
+            self.weight = tensors["mix.weight"]
+
+        def forward(self, x, step, cache):
+            out = torch.empty_like(x, dtype=torch.float32)
+            row = 0
+            for n, slot in zip(step.seq_lens_host, step.slots_host):
+                state = cache.state[slot]
+                xs = x[row:row + n].float()
+                sums = state[: self.width] + torch.cumsum(xs, dim=0)
+                counts = state[self.width] + torch.arange(1, n + 1, device=x.device)
+                out[row:row + n] = sums / counts[:, None]
+                state[: self.width] = sums[-1]
+                state[self.width] = counts[-1]
+                row += n
+            return ops.linear(out.to(x.dtype), self.weight)
+
+    register_mixer(RunningMeanMixer.kind, RunningMeanMixer)
+    return RunningMeanMixer
+
+
+class ToyConfig:
+    """A whole toy architecture: layers alternate the toy mixer and attention."""
+
+    def __init__(self, data):
+        self.data = dict(data)
+
+    @classmethod
+    def from_dict(cls, data):
+        return cls(data)
+
+    def to_dict(self):
+        return dict(self.data)
+
+    def to_spec(self):
+        from zig_ai_amd.config.spec import LayerCall, LayerSpec, ModelSpec, PartSpec
+        d = self.data
+        H, V = d["width"], d["vocab_size"]
+        layers = []
+        for i, kind in enumerate(d["kinds"]):
+            p = f"layers.{i}."
+            if kind == "toy":
+                mixer = PartSpec("toy_running_mean", {"width": H}, {"mix.weight": (p + "mix.weight",)})
+            else:
+                rope = PartSpec("rope", {"head_dim": d["head_dim"], "rotary_dim": d["head_dim"] // 2,
+                                         "theta": 100.0, "pairing": "adjacent"})
+                mixer = PartSpec("gqa_attention",
+                                 {"hidden_size": H, "num_heads": d["heads"], "num_kv_heads": d["kv_heads"],
+                                  "head_dim": d["head_dim"], "qk_norm": False, "norm_eps": 1e-5,
+                                  "window": d.get("window", 0), "softmax_scale": d.get("scale"),
+                                  "bias": False, "position": rope},
+                                 {k + ".weight": (p + k + ".weight",)
+                                  for k in ("q_proj", "k_proj", "v_proj", "out_proj")})
+            ffn = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": d["ffn"]},
+                           {k + ".weight": (p + "ffn." + k + ".weight",) for k in ("gate", "up", "down")})
+            n1 = PartSpec("rms_norm", {"width": H, "eps": 1e-5}, {"weight": (p + "norm1.weight",)})
+            n2 = PartSpec("rms_norm", {"width": H, "eps": 1e-5}, {"weight": (p + "norm2.weight",)})
+            layers.append(LayerSpec(mixer, ffn, n1, n2))
+        schedule = tuple(LayerCall(*c) for c in d["schedule"])
+        return ModelSpec("ToyForCausalLM", H, V,
+                         PartSpec("token_embedding", {"vocab_size": V, "hidden_size": H},
+                                  {"weight": ("embed.weight",)}),
+                         tuple(layers), schedule,
+                         PartSpec("rms_norm", {"width": H, "eps": 1e-5}, {"weight": ("norm.weight",)}),
+                         PartSpec("linear_head", {"vocab_size": V, "hidden_size": H, "tied": True}, {}))
+
+
+TOY = {"architectures": ["ToyForCausalLM"], "width": 48, "vocab_size": 97, "ffn": 72,
+       "heads": 3, "kv_heads": 3, "head_dim": 16, "window": 9, "scale": 0.5,
+       "kinds": ["toy", "attn", "toy"],
+       # layer 0 runs twice (second time with a cache of its own), the last entry reads
+       # the keys and values that entry 1 wrote
+       "schedule": [(0, 0), (1, 1), (2, 2), (0, 3), (1, 1, False)]}
+
+
+def toy_oracle(folder, tokens):
+    """The toy model, whole sequence, float64, written out directly."""
+    from safetensors.torch import load_file
+    w = {k: v.double() for k, v in load_file(folder + "/model.safetensors").items()}
+    d = TOY
+    H, nh, hd = d["width"], d["heads"], d["head_dim"]
+    x = w["embed.weight"][torch.tensor(tokens)]
+    pos = torch.arange(len(tokens))
+    kv_of_entry = {}
+    for layer, cache, *rest in d["schedule"]:
+        writes = not rest or rest[0]
+        p = f"layers.{layer}."
+        n1 = plain.rms_norm(x, w[p + "norm1.weight"], 1e-5)
+        if d["kinds"][layer] == "toy":
+            mean = torch.cumsum(n1, 0) / torch.arange(1, len(tokens) + 1)[:, None]
+            m = mean @ w[p + "mix.weight"].T
+        else:
+            T = len(tokens)
+            q = (n1 @ w[p + "q_proj.weight"].T).view(T, nh, hd)
+            q = plain.apply_rope(q, pos, 100.0, hd // 2, "adjacent")
+            if writes:
+                k = (n1 @ w[p + "k_proj.weight"].T).view(T, nh, hd)
+                k = plain.apply_rope(k, pos, 100.0, hd // 2, "adjacent")
+                v = (n1 @ w[p + "v_proj.weight"].T).view(T, nh, hd)
+                kv_of_entry[cache] = (k, v)
+            k, v = kv_of_entry[cache]
+            o = plain.causal_attention(q, k, v, pos, window=d["window"], scale=d["scale"])
+            m = o.reshape(T, nh * hd) @ w[p + "out_proj.weight"].T
+        h = x + m
+        n2 = plain.rms_norm(h, w[p + "norm2.weight"], 1e-5)
+        x = h + plain.swiglu_ffn(n2, w[p + "ffn.gate.weight"], w[p + "ffn.up.weight"],
+                                 w[p + "ffn.down.weight"])
+    return plain.rms_norm(x, w["norm.weight"], 1e-5) @ w["embed.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_steps_through_the_engine(dtype):
+    from zig_ai_amd.config import register_architecture
+    from zig_ai_amd.engine import DecoderModel, ModelRunner
+    toy_classes()
+    register_architecture("ToyForCausalLM", ToyConfig)
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    folder = eu.model_folder(TOY, 11, store, std=0.2, norm_init="around_one",
+                             role_std={"norm": 0.2})
+    model = DecoderModel.from_folder(folder, dtype)
+    # four cache entries: two states (layer 0 twice), one state (layer 2), one paged group
+    assert len(model.cache_needs) == 4
+    lengths = [40, 9, 23]
+    prompts = [eu.random_tokens(n, 97, 600 + n) for n in lengths]
+    expect = [toy_oracle(folder, p) for p in prompts]
+    tol = 1e-4 if dtype == "float32" else 2.5e-2
+    for schedule in (eu.whole(lengths), eu.changing_portions(lengths, 1),
+                     eu.mixed(lengths, seed=3, max_live=3, decode_tail=5)):
+        runner = ModelRunner(model, page_size=4, num_pages=24, num_slots=3)
+        got = eu.run_schedule(runner, prompts, schedule)
+        for g, e in zip(got, expect):
+            assert eu.rel_err(g, e) < tol
+        # the window of 9 lets pages behind it go back while the request still runs
+        assert runner.cache.stats()["groups"][0]["pages_high_water"] < sum(
+            (n + 3) // 4 for n in lengths)

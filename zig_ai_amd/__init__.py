@@ -18,3 +18,14 @@ compiled and loaded the first time one of them is called.
 __version__ = "0.1.0"
 
 from .config import load_config, register_architecture, known_architectures  # noqa: F401
+
+
+def __getattr__(name):
+    # The engine classes import torch-heavy modules; load them on first use.
+    if name in ("Engine", "DecoderModel", "ModelRunner", "StepEntry", "Scheduler", "Request"):
+        from . import engine
+        return getattr(engine, name)
+    if name in ("SamplingParams",):
+        from . import sampling
+        return getattr(sampling, name)
+    raise AttributeError(name)

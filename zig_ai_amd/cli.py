@@ -1,0 +1,124 @@
+"""Command line in the manner of the reference's
+(/root/reference/src/main.zig:177-319): the same option names with the same
+meanings and defaults where the reference has them, the rest dropped with the
+subsystems they belonged to (quantisation, offload, speculative decoding, chat
+templates), and a few of this engine's own.
+
+    python -m zig_ai_amd -m MODEL_DIR --prompt "12 7 99" -n 32 --temperature 0
+
+``--prompt`` is text when the model folder holds a ``tokenizer.json`` (and the
+``tokenizers`` package is there), otherwise token ids separated by spaces or
+commas; ``--prompt-ids`` is always ids.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import re
+import sys
+import time
+from typing import List, Optional
+
+
+def build_parser() -> argparse.ArgumentParser:
+    ap = argparse.ArgumentParser(prog="zig-ai", description="LFM2 inference on one MI355X")
+    ap.add_argument("-m", "--model", required=True, help="model folder (config.json + safetensors)")
+    ap.add_argument("--prompt", default=None, help="prompt text, or token ids without a tokenizer")
+    ap.add_argument("--prompt-ids", default=None, help="prompt as token ids: \"5 17 3\" or \"5,17,3\"")
+    ap.add_argument("--prompt-file", default=None,
+                    help="JSON file with a list of prompts, each a list of token ids")
+    ap.add_argument("-n", "--max-tokens", type=int, default=128, help="most new tokens (default 128)")
+    ap.add_argument("--temperature", type=float, default=1.0, help="default 1.0; <= 0 is greedy")
+    ap.add_argument("--top-k", type=int, default=0, help="default 0 = off")
+    ap.add_argument("--top-p", type=float, default=1.0, help="default 1.0 = off")
+    ap.add_argument("--repetition-penalty", type=float, default=1.0, help="default 1.0 = off")
+    ap.add_argument("--seed", type=int, default=42, help="seed of the sampling streams (default 42)")
+    ap.add_argument("-b", "--batch-size", type=int, default=2048,
+                    help="token budget of one step (default 2048)")
+    ap.add_argument("-ub", "--ubatch-size", type=int, default=512,
+                    help="largest portion of one prompt in a step (default 512)")
+    ap.add_argument("-np", type=int, default=1, dest="num_parallel",
+                    help="run the prompt as this many parallel requests (default 1)")
+    ap.add_argument("--backend", choices=["auto", "gpu", "cpu"], default="auto",
+                    help="auto and gpu run on the GPU; cpu is refused (there is no CPU path)")
+    ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    ap.add_argument("--page-size", type=int, default=16)
+    ap.add_argument("--num-pages", type=int, default=None)
+    ap.add_argument("--max-num-seqs", type=int, default=64)
+    ap.add_argument("--eos", type=int, default=None, help="stop token id (default: the config's)")
+    ap.add_argument("--json", action="store_true", help="print one JSON object instead of text")
+    return ap
+
+
+def parse_ids(text: str) -> List[int]:
+    parts = [p for p in re.split(r"[\s,]+", text.strip()) if p]
+    try:
+        return [int(p) for p in parts]
+    except ValueError:
+        raise SystemExit(f"not a list of token ids: {text!r}")
+
+
+def load_tokenizer(model_dir: str):
+    path = os.path.join(model_dir, "tokenizer.json")
+    if not os.path.isfile(path):
+        return None
+    try:
+        from tokenizers import Tokenizer
+    except ImportError:
+        return None
+    return Tokenizer.from_file(path)
+
+
+def main(argv: Optional[List[str]] = None) -> int:
+    args = build_parser().parse_args(argv)
+    if args.backend == "cpu":
+        print("this engine has no CPU path; use --backend gpu", file=sys.stderr)
+        return 2
+    tokenizer = load_tokenizer(args.model)
+    prompts: List[List[int]]
+    if args.prompt_file:
+        with open(args.prompt_file) as f:
+            prompts = [[int(t) for t in p] for p in json.load(f)]
+    elif args.prompt_ids is not None:
+        prompts = [parse_ids(args.prompt_ids)]
+    elif args.prompt is not None:
+        if tokenizer is not None:
+            prompts = [tokenizer.encode(args.prompt).ids]
+        else:
+            prompts = [parse_ids(args.prompt)]
+    else:
+        print("give --prompt, --prompt-ids or --prompt-file", file=sys.stderr)
+        return 2
+    prompts = [p for p in prompts for _ in range(max(1, args.num_parallel))]
+
+    from .engine.engine import Engine
+    load_start = time.perf_counter()
+    engine = Engine(args.model, dtype=args.dtype, page_size=args.page_size,
+                    num_pages=args.num_pages, max_num_seqs=args.max_num_seqs,
+                    max_num_batched_tokens=args.batch_size, chunk_size=args.ubatch_size)
+    load_s = time.perf_counter() - load_start
+    start = time.perf_counter()
+    outputs = engine.generate(prompts, max_new_tokens=args.max_tokens,
+                              temperature=args.temperature, top_k=args.top_k, top_p=args.top_p,
+                              repetition_penalty=args.repetition_penalty, seed=args.seed,
+                              eos_token_id=args.eos)
+    import torch
+    torch.cuda.synchronize()
+    total_s = time.perf_counter() - start
+    n_new = sum(len(o) for o in outputs)
+    if args.json:
+        print(json.dumps({"outputs": outputs, "load_s": load_s, "generate_s": total_s,
+                          "tokens_per_s": n_new / total_s if total_s > 0 else 0.0,
+                          "stats": engine.stats()}))
+        return 0
+    for i, out in enumerate(outputs):
+        head = f"[{i}] " if len(outputs) > 1 else ""
+        if tokenizer is not None:
+            print(head + tokenizer.decode(out))
+        print(head + " ".join(str(t) for t in out))
+    print(f"load {load_s * 1e3:.0f} ms; {sum(len(p) for p in prompts)} prompt tokens, "
+          f"{n_new} new tokens in {total_s * 1e3:.0f} ms ({n_new / total_s:.1f} tok/s)",
+          file=sys.stderr)
+    return 0

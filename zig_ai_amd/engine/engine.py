@@ -1,0 +1,115 @@
+"""The Python entry point: ``Engine(model_dir).generate(prompts, ...)``.
+
+The reference is driven from its command line only (/root/reference/src/main.zig:
+573-1417: load, prefill in chunks, decode token by token, print); this class is
+the same loop around the scheduler and the step function, for any number of
+requests at once.
+"""
+
+from __future__ import annotations
+
+import time
+from typing import Dict, Hashable, List, Optional, Sequence
+
+import torch
+
+from ..sampling.sampler import SamplingParams, UniformStream, sample_rows
+from .batch import StepEntry
+from .model import DecoderModel
+from .runner import ModelRunner
+from .scheduler import Request, ScheduledEntry, Scheduler
+
+
+class Engine:
+    def __init__(self, model_dir: str, dtype: str = "bfloat16", page_size: int = 16,
+                 num_pages: Optional[int] = None, max_num_seqs: int = 64,
+                 max_num_batched_tokens: int = 2048, chunk_size: int = 512,
+                 max_model_len: Optional[int] = None):
+        """``num_pages``: pages per cache group; by default enough for
+        ``max_num_seqs`` requests of ``max_model_len`` tokens (the model's
+        ``max_position_embeddings`` if not given, capped at 8192)."""
+        self.model = DecoderModel.from_folder(model_dir, dtype)
+        limit = max_model_len or self.model.spec.max_position or 8192
+        if max_model_len is None:
+            limit = min(limit, 8192)
+        self.max_model_len = limit
+        if num_pages is None:
+            num_pages = max_num_seqs * ((limit + page_size - 1) // page_size)
+        self.runner = ModelRunner(self.model, page_size, num_pages, max_num_seqs)
+        self.scheduler = Scheduler(self.runner.cache, max_num_seqs, max_num_batched_tokens,
+                                   chunk_size, limit)
+        self._streams: Dict[Hashable, UniformStream] = {}
+        self._next_id = 0
+        self.timings = {"steps": 0, "step_seconds": 0.0, "tokens_run": 0, "tokens_generated": 0}
+
+    # ---------------------------------------------------------------- requests
+    def add_request(self, prompt: Sequence[int], max_new_tokens: int,
+                    sampling: Optional[SamplingParams] = None,
+                    eos_token_id: Optional[int] = None, request_id: Hashable = None) -> Request:
+        vocab = self.model.spec.vocab_size
+        prompt = [int(t) for t in prompt]
+        for t in prompt:
+            if not 0 <= t < vocab:
+                raise ValueError(f"token id {t} is outside the vocabulary of {vocab}")
+        if len(prompt) + max_new_tokens > self.max_model_len:
+            raise ValueError(f"prompt of {len(prompt)} tokens plus {max_new_tokens} new ones "
+                             f"exceeds max_model_len {self.max_model_len}")
+        if request_id is None:
+            request_id = self._next_id
+            self._next_id += 1
+        req = Request(request_id, prompt, max_new_tokens, sampling or SamplingParams(),
+                      eos_token_id)
+        self.scheduler.add(req)
+        self._streams[req.id] = UniformStream(req.sampling.seed, req.number)
+        return req
+
+    def step(self) -> List[Request]:
+        """One scheduled step; returns the requests that finished in it."""
+        plan = self.scheduler.schedule()
+        if not plan:
+            return []
+        start = time.perf_counter()
+        entries = []
+        for e in plan:
+            tokens = e.request.tokens[e.start:e.start + e.count]
+            entries.append(StepEntry(e.request.id, tokens, [e.count - 1] if e.samples else []))
+        logits = self.runner.step(entries)
+        sampling = [e for e in plan if e.samples]
+        drawn = sample_rows(
+            logits, [e.request.sampling for e in sampling],
+            [self._streams[e.request.id].at(len(e.request.output)) for e in sampling],
+            [e.request.output for e in sampling])
+        done = self.scheduler.update(plan, {e.request.id: t for e, t in zip(sampling, drawn)})
+        for req in done:
+            self._streams.pop(req.id, None)
+        self.timings["steps"] += 1
+        self.timings["step_seconds"] += time.perf_counter() - start
+        self.timings["tokens_run"] += sum(e.count for e in plan)
+        self.timings["tokens_generated"] += len(sampling)
+        return done
+
+    def run(self) -> None:
+        while self.scheduler.has_work():
+            self.step()
+
+    # ---------------------------------------------------------------- generate
+    def generate(self, prompt_token_ids: Sequence[Sequence[int]], max_new_tokens: int = 128,
+                 temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0,
+                 repetition_penalty: float = 1.0, seed: int = 42,
+                 eos_token_id: Optional[int] = None) -> List[List[int]]:
+        """Generate for every prompt; returns the new tokens of each, in order.
+        ``temperature <= 0`` is greedy.  Each request draws from its own random
+        stream keyed by ``(seed, its number)``."""
+        params = SamplingParams(temperature, top_k, top_p, repetition_penalty, seed)
+        if eos_token_id is None:
+            eos_token_id = getattr(getattr(self.model, "config", None), "eos_token_id", None)
+        reqs = [self.add_request(p, max_new_tokens, params, eos_token_id)
+                for p in prompt_token_ids]
+        self.run()
+        return [list(r.output) for r in reqs]
+
+    def stats(self) -> dict:
+        out = self.runner.cache.stats()
+        out.update(self.timings)
+        out["preemptions"] = self.scheduler.preemption_count
+        return out

@@ -107,6 +107,38 @@ class DecoderModel:
         model.config = config
         return model
 
+    @classmethod
+    def from_random(cls, config, seed: int = 0, dtype="bfloat16",
+                    device: Optional[torch.device] = None, std: float = 0.02,
+                    norm_init: str = "ones"):
+        """A model with random weights drawn on the device, for benchmarks: the same
+        distributions as the random model writer, without the trip through a file.
+        ``config`` is a typed configuration or a config.json dictionary."""
+        from ..config import config_from_dict
+        from ..weights.loader import expected_tensors, keep_dtype
+        device = device or require_gpu()
+        if isinstance(config, Mapping):
+            config = config_from_dict(config)
+        spec = config.to_spec()
+        rt = parts.Runtime(device=device, dtype=run_dtype(dtype))
+        gen = torch.Generator(device=device)
+        gen.manual_seed(int(seed))
+        tensors: Dict[Any, Dict[str, torch.Tensor]] = {}
+        for exp in expected_tensors(spec):
+            shape = exp.rule.shapes[0]
+            if exp.rule.role == "norm" and norm_init == "ones":
+                t = torch.ones(shape, dtype=torch.float32, device=device)
+            else:
+                t = torch.empty(shape, dtype=torch.float32, device=device)
+                t.normal_(0.0, std, generator=gen)
+                if exp.rule.role == "norm" and norm_init == "around_one":
+                    t += 1.0
+            tensors.setdefault(exp.owner, {})[exp.local] = t.to(
+                keep_dtype(rt.dtype, exp.rule.role, rt.dtype))
+        model = cls(spec, tensors, rt)
+        model.config = config
+        return model
+
     def make_cache(self, page_size: int, num_pages, num_slots: int) -> CacheManager:
         return CacheManager(self.cache_needs, page_size, num_pages, num_slots,
                             device=self.runtime.device, dtype=self.runtime.dtype)
