@@ -153,8 +153,11 @@ def test_toy_architecture_steps_through_the_engine(dtype):
     toy_classes()
     register_architecture("ToyForCausalLM", ToyConfig)
     store = torch.float32 if dtype == "float32" else torch.bfloat16
+    # query/key weights sized so that scores spread over about one unit: sharper
+    # scores would turn bfloat16's rounding of q and k into percent-sized changes
+    # of the softmax, which is the number format's doing, not the engine's
     folder = eu.model_folder(TOY, 11, store, std=0.2, norm_init="around_one",
-                             role_std={"norm": 0.2})
+                             role_std={"norm": 0.2, "q_proj.weight": 0.08, "k_proj.weight": 0.08})
     model = DecoderModel.from_folder(folder, dtype)
     # four cache entries: two states (layer 0 twice), one state (layer 2), one paged group
     assert len(model.cache_needs) == 4
