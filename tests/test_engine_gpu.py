@@ -130,6 +130,55 @@ def test_long_decoding(dtype):
     for p in range(7, len(tokens)):
         got.append(runner.step([StepEntry("r", tokens[p:p + 1], [0])]).cpu())
     assert eu.rel_err(torch.cat(got), expect) < TOL[dtype]
+    # the single-token steps were replays of a recorded HIP graph ...
+    assert runner.graphs is not None and runner.graphs.replays >= 290
+    assert runner.graphs.captures <= 3
+    # ... and replaying changes nothing but rounding (a recorded step cuts long
+    # contexts at fixed places, an eager one by the step's own longest context)
+    from zig_ai_amd.engine import ModelRunner
+    eager = ModelRunner(model, page_size=16, num_pages=32, num_slots=4, use_graphs=False)
+    eager.admit("r")
+    again = [eager.step([StepEntry("r", tokens[:7], list(range(7)))]).cpu()]
+    for p in range(7, len(tokens)):
+        again.append(eager.step([StepEntry("r", tokens[p:p + 1], [0])]).cpu())
+    assert eu.rel_err(torch.cat(again), torch.cat(got).double()) < (2e-5 if dtype == "float32" else TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replays_between_other_work(dtype):
+    """Replays of a recorded step interleaved with eager steps (portions of other
+    requests), with synchronisations between them, each compared with the plain
+    implementation; requests change slots and pages between replays."""
+    from zig_ai_amd.engine import StepEntry
+    model, expect, prompts = setup("B", dtype)
+    runner = runner_for(model, 8, 64, num_slots=4)
+    got = {i: [] for i in range(len(prompts))}
+    # requests 3 and 4 (64 and 100 tokens) decode one token per step after a bulk
+    # portion; requests 0..2 come and go between those steps
+    for i, head in ((3, 30), (4, 50)):
+        runner.admit(i)
+        got[i].append(runner.step([StepEntry(i, prompts[i][:head], list(range(head)))]).cpu())
+    cursor = {3: 30, 4: 50}
+    others = [0, 1, 2, 0, 1, 2]
+    step = 0
+    while cursor[3] < 64 or cursor[4] < 100:
+        batch = [StepEntry(i, prompts[i][cursor[i]:cursor[i] + 1], [0])
+                 for i in (3, 4) if cursor[i] < len(prompts[i])]
+        out = runner.step(batch).cpu()
+        for row, e in enumerate(batch):
+            got[e.request].append(out[row:row + 1])
+            cursor[e.request] += 1
+        torch.cuda.synchronize()
+        if step % 5 == 0 and others:
+            j = others.pop(0)
+            runner.admit(("x", j))
+            o = runner.step([StepEntry(("x", j), prompts[j], list(range(len(prompts[j]))))]).cpu()
+            assert eu.rel_err(o, expect[j]) < TOL[dtype]
+            runner.release(("x", j))
+        step += 1
+    for i in (3, 4):
+        assert eu.rel_err(torch.cat(got[i]), expect[i]) < TOL[dtype]
+    assert runner.graphs.replays >= 40
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

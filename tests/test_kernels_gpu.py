@@ -141,17 +141,36 @@ def test_gemm_bf16_skinny_and_tiled_agree(M):
 
 
 def test_gemm_rows_do_not_depend_on_batch():
-    """A token's projection is the same whatever else is in the step (bitwise,
-    within one kernel)."""
+    """A token's projection is the same whatever else is in the step: bitwise
+    within one kernel (each sums over k in an order fixed by K alone), within
+    rounding between kernels."""
     x, w = rand((64, 256), torch.bfloat16, 18), rand((80, 256), torch.bfloat16, 19)
-    full = ops().linear(x.to(dev()), w.to(dev()), out_dtype=torch.float32).cpu()
-    for m in (1, 5, 16, 33):
-        part = ops().linear(x[:m].contiguous().to(dev()), w.to(dev()), out_dtype=torch.float32).cpu()
-        assert torch.equal(part, full[:m])
+
+    def run(m, **kw):
+        return ops().linear(x[:m].contiguous().to(dev()), w.to(dev()), out_dtype=torch.float32, **kw).cpu()
+
+    for group in ((1, 5, 16), (17, 33, 64)):              # the kernels' ranges of M
+        full = run(group[-1])
+        for m in group[:-1]:
+            assert torch.equal(run(m), full[:m])
+    tiled = run(64, force_tiled=True)
+    for m in (3, 40):
+        assert torch.equal(run(m, force_tiled=True), tiled[:m])
+    assert rel_err(run(16), tiled[:16].double()) < F32_TOL
+    assert rel_err(run(64), tiled.double()) < F32_TOL
     x32, w32 = x.float(), w.float()
     full32 = ops().linear(x32.to(dev()), w32.to(dev())).cpu()
     part32 = ops().linear(x32[:3].contiguous().to(dev()), w32.to(dev())).cpu()
     assert torch.equal(part32, full32[:3])
+
+
+@pytest.mark.parametrize("K", [8, 72, 512, 520, 2048, 2056, 4096, 8192, 8200])
+@pytest.mark.parametrize("M,N", [(1, 48), (8, 50), (16, 33)])
+def test_gemm_bf16_decode_rows_all_k_ranges(M, N, K):
+    """The decode kernel picks its shape by K; every range, with tails."""
+    x, w, b = rand((M, K), torch.bfloat16, 27), rand((N, K), torch.bfloat16, 28), rand((N,), torch.float32, 29)
+    out = ops().linear(x.to(dev()), w.to(dev()), b.to(dev()), out_dtype=torch.float32)
+    assert rel_err(out, x.double() @ w.double().T + b.double()) < F32_TOL
 
 
 def test_gemm_bf16_refuses_odd_k():

@@ -6,6 +6,7 @@
 //   gemm_f32_kernel          true 32-bit: LDS-tiled FMA, no matrix-core rounding modes
 //   gemm_bf16_mfma_kernel    bfloat16 operands on the matrix cores (16x16x32), any M
 //   gemm_bf16_skinny_kernel  bfloat16, M <= 64: streams W once, K split over the waves
+//   gemm_bf16_rows16_kernel  bfloat16, M <= 16 (decoding): activations held in registers
 //
 // In all three every output element is a sum over k in an order that depends
 // only on K, never on M or on the tile it falls in, so a token's result does
@@ -253,6 +254,75 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__
   }
 }
 
+// ------------------------------------------- bfloat16, at most 16 rows (decode)
+// The activations of a decode step are few: every wave keeps its slice of them
+// (16 tokens x KSTEPS * 32 elements of K) in registers for the whole kernel and
+// streams weight rows past them, 16 rows at a time with all of a row group's
+// loads in flight at once.  The NW waves of a workgroup split K; their partial
+// tiles meet in LDS (double-buffered, one barrier per row group) and wave 0
+// writes the sum.  A workgroup walks `groups_per_block` consecutive row groups.
+template <int NW, int KSTEPS, typename TC>
+__global__ void __launch_bounds__(NW * 64)
+gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
+                        const float* __restrict__ bias, TC* __restrict__ C, int M, int N, int K,
+                        int groups_per_block) {
+  __shared__ float red[2][NW][64][4];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int frag_row = lane & 15, frag_k = (lane >> 4) * 8;
+  const int kbase = wave * KSTEPS * 32 + frag_k;
+  const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  constexpr int HALF = KSTEPS > 16 ? 16 : KSTEPS;   // weight fragments in flight at once
+
+  bf16x8_t xa[KSTEPS];
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s) {
+    const int k = kbase + s * 32;
+    xa[s] = (frag_row < M && k < K) ? *reinterpret_cast<const bf16x8_t*>(A + (size_t)frag_row * K + k)
+                                    : zero8;
+  }
+
+  for (int g = 0; g < groups_per_block; ++g) {
+    const int n0 = (blockIdx.x * groups_per_block + g) * 16;
+    if (n0 >= N) break;
+    const int wrow = n0 + frag_row;
+    const bool wvalid = wrow < N;
+    const bf16_t* wp = W + (size_t)(wvalid ? wrow : 0) * K + kbase;
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int h = 0; h < KSTEPS; h += HALF) {
+      bf16x8_t fw[HALF];
+#pragma unroll
+      for (int s = 0; s < HALF; ++s) {
+        const int k = kbase + (h + s) * 32;
+        fw[s] = (wvalid && k < K) ? *reinterpret_cast<const bf16x8_t*>(wp + (h + s) * 32) : zero8;
+      }
+#pragma unroll
+      for (int s = 0; s < HALF; ++s)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[s], xa[h + s], acc, 0, 0, 0);
+    }
+    float* mine = red[g & 1][wave][lane];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) mine[r] = acc[r];
+    __syncthreads();
+    if (wave == 0) {
+      const int m = lane & 15, nn = n0 + (lane >> 4) * 4;
+      if (m < M) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int n = nn + r;
+          if (n >= N) continue;
+          float v = red[g & 1][0][lane][r];
+#pragma unroll
+          for (int w = 1; w < NW; ++w) v += red[g & 1][w][lane][r];
+          if (bias) v += bias[n];
+          C[(size_t)m * N + n] = from_f32<TC>(v);
+        }
+      }
+    }
+  }
+}
+
 // ------------------------------------------------------------------ launchers
 // dtype codes: 0 = float32, 1 = bfloat16
 extern "C" int za_gemm_f32(const void* A, int a_dtype, const float* W, const float* bias, void* C,
@@ -282,6 +352,30 @@ extern "C" int za_gemm_bf16(const void* A, const void* W, const float* bias, voi
   if (c_dtype != 0 && c_dtype != 1) return ZA_ERR_UNSUPPORTED;
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
+  if (M <= 16 && K <= 8192 && !force_tiled) {
+    const int groups = (N + 15) / 16;
+    // enough workgroups to cover the machine a few times, few enough to amortise
+    // loading the activations
+    int per_block = 1;
+    while (per_block < 8 && groups / (per_block * 2) >= 1024) per_block *= 2;
+    dim3 grid((groups + per_block - 1) / per_block);
+#define ZA_R16_CASE(NW, KS)                                                                    \
+  {                                                                                            \
+    dim3 block(NW * 64);                                                                       \
+    if (c_dtype == 0)                                                                          \
+      hipLaunchKernelGGL((gemm_bf16_rows16_kernel<NW, KS, float>), grid, block, 0, stream, a,  \
+                         w, bias, (float*)C, M, N, K, per_block);                              \
+    else                                                                                       \
+      hipLaunchKernelGGL((gemm_bf16_rows16_kernel<NW, KS, bf16_t>), grid, block, 0, stream, a, \
+                         w, bias, (bf16_t*)C, M, N, K, per_block);                             \
+    return za_launch_status();                                                                 \
+  }
+    if (K <= 512) ZA_R16_CASE(1, 16)
+    if (K <= 2048) ZA_R16_CASE(4, 16)
+    if (K <= 4096) ZA_R16_CASE(8, 16)
+    ZA_R16_CASE(8, 32)
+#undef ZA_R16_CASE
+  }
   if (M <= 64 && !force_tiled) {
     dim3 grid((N + 15) / 16), block(256);
     const int mt = (M + 15) / 16;

@@ -81,9 +81,16 @@ def _make_items(seq_lens: Sequence[int], rows_per_item: int):
 
 def build_step(entries: Sequence[StepEntry], cache: CacheManager, device: torch.device,
                vocab_size: int, item_granularities: Sequence[int] = (),
-               max_position: int = 0) -> StepContext:
+               max_position: int = 0, min_pages: int = 0, max_keys: int = 0,
+               into: Optional[torch.Tensor] = None) -> StepContext:
     """Lay out the step.  Every request must be admitted and its pages for this
-    step reserved beforehand; nothing is committed here."""
+    step reserved beforehand; nothing is committed here.
+
+    The layout is a function of (tokens per entry, wanted rows per entry, width of
+    the block tables) only.  ``min_pages`` widens the block tables, ``max_keys``
+    overrides the context length used for planning, and ``into`` is a device
+    buffer to fill instead of a new one: together they let a replayed HIP graph
+    find every array at the address it was captured with."""
     if not entries:
         raise StepError("a step needs at least one entry")
     seen = set()
@@ -116,6 +123,7 @@ def build_step(entries: Sequence[StepEntry], cache: CacheManager, device: torch.
     for e in entries:
         for g in groups:
             max_pages = max(max_pages, len(cache.table(e.request, g.index)))
+    max_pages = max(max_pages, min_pages)
 
     sections: List[Tuple[str, int]] = [
         ("token_ids", T), ("positions", T), ("token_seq", T), ("seq_start", S + 1),
@@ -166,7 +174,14 @@ def build_step(entries: Sequence[StepEntry], cache: CacheManager, device: torch.
         put(f"irow{gran}", row0)
         put(f"icnt{gran}", cnt)
 
-    dev = torch.from_numpy(host).to(device)
+    if into is None:
+        dev = torch.from_numpy(host).to(device)
+    else:
+        if into.numel() < host.size or into.dtype != torch.int32:
+            raise StepError(f"the step needs {host.size} int32 entries, the buffer holds "
+                            f"{into.numel()}")
+        dev = into
+        dev[:host.size].copy_(torch.from_numpy(host))
 
     def view(name: str) -> torch.Tensor:
         off, n = offsets[name]
@@ -174,7 +189,7 @@ def build_step(entries: Sequence[StepEntry], cache: CacheManager, device: torch.
 
     ctx = StepContext(
         n_tokens=T, n_seqs=S, n_logit_rows=R,
-        max_keys=max(c + n for c, n in zip(ctx_lens, seq_lens)),
+        max_keys=max(max_keys, max(c + n for c, n in zip(ctx_lens, seq_lens))),
         token_ids=view("token_ids"), positions=view("positions"), token_seq=view("token_seq"),
         seq_start=view("seq_start"), ctx_len=view("ctx_len"), slot_id=view("slot_id"),
         logit_rows=view("logit_rows"),

@@ -91,6 +91,12 @@ class DecoderModel:
         self.item_granularities = sorted({
             b.mixer.rows_per_item for b in self.blocks if hasattr(b.mixer, "rows_per_item")})
         self.kernel_sources = sorted(sources)
+        # A step may be recorded into a HIP graph only if no part looks at the step's
+        # numbers on the host while it runs.
+        every = [self.embedding, self.final_norm, self.head]
+        for b in self.blocks:
+            every += [b.mixer_norm, b.mixer, b.feed_forward_norm, b.feed_forward]
+        self.graph_safe = all(getattr(p, "graph_safe", False) for p in every)
         # Compile what this model's parts use, together, before the first step.
         if self.kernel_sources:
             kernel_build.build_all(self.kernel_sources, jobs=len(self.kernel_sources))

@@ -21,17 +21,21 @@ import torch
 from ..cache.manager import CacheManager
 from ..cache.pages import OutOfPages
 from .batch import StepContext, StepEntry, StepError, build_step
+from .graphs import DecodeGraphs
 from .model import DecoderModel
 
 
 class ModelRunner:
     def __init__(self, model: DecoderModel, page_size: int = 16, num_pages: int = 1024,
-                 num_slots: int = 64):
+                 num_slots: int = 64, use_graphs: bool = True):
+        """``use_graphs``: replay steps of single tokens as HIP graphs when every part
+        of the model declares itself safe to record (``graph_safe``)."""
         self.model = model
         self.device = model.runtime.device
         self.cache = model.make_cache(page_size, num_pages, num_slots)
         self.views = model.cache_views(self.cache)
         self.steps_run = 0
+        self.graphs = DecodeGraphs() if (use_graphs and model.graph_safe) else None
 
     # ----------------------------------------------------------------- requests
     def admit(self, request: Hashable) -> None:
@@ -44,8 +48,8 @@ class ModelRunner:
         return request in self.cache.requests
 
     # --------------------------------------------------------------------- step
-    def prepare(self, entries: Sequence[StepEntry]) -> StepContext:
-        """Reserve pages for the entries (all of them or none) and lay out the step."""
+    def reserve(self, entries: Sequence[StepEntry]) -> None:
+        """Pages for every entry of the step, all of them or none."""
         wanted = {}
         for e in entries:
             if e.request not in self.cache.requests:
@@ -59,15 +63,36 @@ class ModelRunner:
                                  f"{pool.free_count} of {pool.size} are free")
         for e in entries:
             self.cache.reserve(e.request, len(e.tokens))
+
+    def prepare(self, entries: Sequence[StepEntry]) -> StepContext:
+        """Reserve pages for the entries and lay out the step."""
+        self.reserve(entries)
         return build_step(entries, self.cache, self.device, self.model.spec.vocab_size,
                           self.model.item_granularities, self.model.spec.max_position)
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Logits ``[R, vocab]`` (32-bit) at the wanted places, in the order of the
         entries and of each entry's ``want``."""
-        ctx = self.prepare(entries)
-        logits = self.model.forward(ctx, self.views)
+        if self.graphs is not None and entries and all(len(e.tokens) == 1 for e in entries):
+            logits = self._graph_step(entries)
+        else:
+            ctx = self.prepare(entries)
+            logits = self.model.forward(ctx, self.views)
         for e in entries:
             self.cache.commit(e.request, len(e.tokens))
         self.steps_run += 1
         return logits
+
+    def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        self.reserve(entries)
+        for e in entries:
+            for w in e.want:
+                if int(w) != 0:
+                    raise StepError(f"request {e.request!r} wants logits at place {w} of 1 token")
+        logits = self.graphs.run(self, entries)
+        rows = [i for i, e in enumerate(entries) for _ in e.want]
+        if rows == list(range(len(entries))):
+            return logits
+        if not rows:
+            return logits[:0]
+        return logits.index_select(0, torch.tensor(rows, dtype=torch.long, device=logits.device))

@@ -46,6 +46,7 @@ def plan_split(n_items: int, num_kv_heads: int, max_keys: int):
 
 class GroupedQueryAttention(Mixer):
     kind = "gqa_attention"
+    graph_safe = True
     kernel_sources = ("gemm", "rope_kv", "attention", "norm")
 
     @classmethod

@@ -16,6 +16,7 @@ from .base import Part, Runtime, TensorRule, register_embedding, register_head
 
 class TokenEmbedding(Part):
     kind = "token_embedding"
+    graph_safe = True
     kernel_sources = ("norm",)
 
     @classmethod
@@ -34,6 +35,7 @@ class TokenEmbedding(Part):
 
 class LinearHead(Part):
     kind = "linear_head"
+    graph_safe = True
     kernel_sources = ("gemm",)
 
     @classmethod

@@ -22,6 +22,7 @@ def fuse_rows(*mats: torch.Tensor) -> torch.Tensor:
 
 class SwiGLU(FeedForward):
     kind = "swiglu"
+    graph_safe = True
     kernel_sources = ("gemm", "activation")
 
     @classmethod

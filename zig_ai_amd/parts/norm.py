@@ -14,6 +14,7 @@ from .base import Norm, Runtime, TensorRule, register_norm
 
 class RMSNorm(Norm):
     kind = "rms_norm"
+    graph_safe = True
     kernel_sources = ("norm",)
 
     @classmethod

@@ -23,6 +23,7 @@ from .base import Mixer, Runtime, StateNeed, TensorRule, register_mixer
 
 class ShortConv(Mixer):
     kind = "short_conv"
+    graph_safe = True
     kernel_sources = ("gemm", "shortconv")
 
     @classmethod
