@@ -15,13 +15,13 @@ import torch
 
 import engine_util as eu
 import plain_lfm2 as plain
-from tiny_configs import TINY_A, TINY_B, TINY_C
+from tiny_configs import TINY_A, TINY_B, TINY_C, TINY_D
 
 pytestmark = pytest.mark.gpu
 
 TOL = {"float32": 1e-4, "bfloat16": 2.5e-2}
-CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
-LENGTHS = {"A": [5, 17, 33, 70], "B": [1, 8, 31, 64, 100], "C": [40, 3, 77]}
+CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3)}
+LENGTHS = {"A": [5, 17, 33, 70], "B": [1, 8, 31, 64, 100], "C": [40, 3, 77], "D": [150, 9, 66, 40]}
 
 _cache = {}
 
@@ -54,7 +54,7 @@ def check(got, expect, dtype, what):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_whole_requests(name, dtype):
     model, expect, prompts = setup(name, dtype)
     runner = runner_for(model, 16, 16)
@@ -65,7 +65,7 @@ def test_whole_requests(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_bulk_then_last_32_one_by_one(name, dtype):
     model, expect, prompts = setup(name, dtype)
     runner = runner_for(model, 4 if name == "A" else 8, 64)
@@ -74,7 +74,7 @@ def test_bulk_then_last_32_one_by_one(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_portions_of_changing_size(name, dtype):
     model, expect, prompts = setup(name, dtype)
     for seed in (0, 3):
@@ -84,7 +84,7 @@ def test_portions_of_changing_size(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_mixed_steps_with_page_reuse(name, dtype):
     model, expect, prompts = setup(name, dtype)
     # the same requests twice over, so that late ones land on pages early ones used

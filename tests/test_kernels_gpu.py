@@ -268,7 +268,7 @@ def items_for(seq_lens, rows_per_item):
 
 
 def run_attention(dtype, nh, nkv, d, page_size, ctx, new, window=0, keys_per_split=0, nsplit=1,
-                  seed=30, sharpen=False):
+                  seed=30, sharpen=False, mfma=False):
     """ctx[s] cached tokens and new[s] query tokens per request."""
     G = nh // nkv
     ks, vs, qs, pos = [], [], [], []
@@ -287,10 +287,14 @@ def run_attention(dtype, nh, nkv, d, page_size, ctx, new, window=0, keys_per_spl
     cache, table = paged_from_dense(ks, vs, page_size, dtype, seed=seed)
     q_all = torch.cat(qs).to(dev())
     positions = torch.tensor(pos, dtype=torch.int32, device=dev())
-    rows = max(1, 32 // G)
-    out = ops().paged_attention(q_all, cache.to(dev()), table.to(dev()), positions,
-                                *items_for(new, rows), 1.0 / math.sqrt(d), window,
-                                keys_per_split, nsplit)
+    if mfma:
+        out = ops().paged_attention_mfma(q_all, cache.to(dev()), table.to(dev()), positions,
+                                         *items_for(new, max(1, 64 // G)), 1.0 / math.sqrt(d),
+                                         window)
+    else:
+        out = ops().paged_attention(q_all, cache.to(dev()), table.to(dev()), positions,
+                                    *items_for(new, max(1, 32 // G)), 1.0 / math.sqrt(d), window,
+                                    keys_per_split, nsplit)
     expect = []
     for s, (c, n) in enumerate(zip(ctx, new)):
         full_q = torch.zeros((c + n, nh, d), dtype=torch.float64)
@@ -322,6 +326,23 @@ def test_paged_attention_reference_shapes(dtype):
                                      (32, 8, 128, 16, [39], [1])]:
         out, expect = run_attention(dtype, nh, nkv, d, ps, ctx, new)
         assert rel_err(out, expect) < tol_of(dtype)
+
+
+@pytest.mark.parametrize("nh,nkv,d,page_size", [
+    (32, 8, 64, 16), (4, 4, 64, 4), (8, 4, 128, 16), (16, 2, 64, 8), (16, 1, 128, 32), (2, 1, 64, 16)])
+@pytest.mark.parametrize("window", [0, 70])
+def test_paged_attention_matrix_cores(nh, nkv, d, page_size, window):
+    """The matrix-core kernel on mixed steps: long portions, portions that do not fill
+    a work item, single tokens with long contexts."""
+    ctx = [0, 37, 129, 5, 300]
+    new = [150, 1, 17, 70, 2]
+    out, expect = run_attention(torch.bfloat16, nh, nkv, d, page_size, ctx, new, window=window,
+                                mfma=True)
+    assert rel_err(out, expect) < BF16_TOL
+    out, expect = run_attention(torch.bfloat16, nh, nkv, d, page_size, [700, 300], [1, 40],
+                                sharpen=True, mfma=True)
+    assert rel_err(out, expect) < BF16_TOL
+    assert float(expect.abs().max()) > 0.5
 
 
 def test_single_token_attention_returns_value():

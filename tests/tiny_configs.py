@@ -32,3 +32,14 @@ TINY_C = {
     "rope_theta": 50000.0, "norm_eps": 3e-6, "conv_L_cache": 2, "conv_bias": True,
     "tie_embedding": True, "max_position_embeddings": 4096,
 }
+
+# sizes the matrix-core attention kernel takes (head_dim 64, four query heads per group)
+TINY_D = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 128, "num_hidden_layers": 3, "num_attention_heads": 8,
+    "num_key_value_heads": 2, "head_dim": 64, "vocab_size": 384,
+    "layer_types": ["full_attention", "conv", "full_attention"],
+    "block_ff_dim": 320, "block_auto_adjust_ff_dim": False,
+    "rope_theta": 1000000.0, "norm_eps": 1e-5, "conv_L_cache": 3, "conv_bias": False,
+    "tie_embedding": True, "max_position_embeddings": 4096,
+}

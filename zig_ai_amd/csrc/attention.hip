@@ -221,6 +221,195 @@ attention_combine_kernel(const float* __restrict__ part_acc, const float* __rest
   }
 }
 
+// ------------------------------------------------------------ matrix-core path
+// bfloat16, head_dim 64 or 128, query heads per key/value head dividing 16: the
+// same streaming softmax with both products on the matrix cores.
+//
+// A workgroup serves up to 64 rows (token, head) of one work item and one
+// key/value head; each of its four waves owns 16 rows.  Per tile of 64 keys:
+//   S^T = K Q^T   (keys as the rows of the first operand, the wave's 16 query rows as
+//                  columns; a lane ends up with the scores of ONE query row for 16 keys)
+//   p   = exp(S^T * scale - m)  in 32-bit, running maximum and sum kept per lane
+//   O^T += V^T P^T  (P^T goes from the accumulator registers straight into the second
+//                  operand: the matrix core does not care in which order the 32 keys of
+//                  a step are numbered as long as both operands agree, so V^T is stored
+//                  in LDS with its keys in the order the accumulator yields them)
+// Operand layout of v_mfma_f32_16x16x32_bf16: lane l supplies row (l % 16), k-slots
+// (l / 16) * 8 .. + 7 of either operand and receives rows (l / 16) * 4 .. + 3, column
+// (l % 16) of the product.
+#define AM_KT 64
+
+template <int D>
+__global__ void __launch_bounds__(256)
+paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
+                            const bf16_t* __restrict__ kv, const int* __restrict__ block_table,
+                            int bt_stride, const int* __restrict__ positions,
+                            const int* __restrict__ wi_seq, const int* __restrict__ wi_row0,
+                            const int* __restrict__ wi_count, int nh, int nkv, int page_size,
+                            float scale, int window) {
+  constexpr int LDK = D + 8;        // padded rows, in elements
+  constexpr int LDV = AM_KT + 8;
+  constexpr int KSTEPS = D / 32;    // matrix-core steps over the head dimension
+  constexpr int DBLK = D / 16;      // 16-wide blocks of the head dimension
+  constexpr int VEC_PER_ROW = D / 8;
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[AM_KT * LDK];   // [key][dim]
+  __shared__ __attribute__((aligned(16))) bf16_t Vt[D * LDV];       // [dim][key slot]
+
+  const int item = blockIdx.x, gkv = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r16 = lane & 15, grp = lane >> 4;
+  const int G = nh / nkv;
+  const int seq = wi_seq[item];
+  const int row0 = wi_row0[item];
+  int count = wi_count[item];
+  if (count * G > 64) count = 64 / G;   // the host never asks for more
+  const int rows = count * G;
+  const int* table = block_table + (size_t)seq * bt_stride;
+
+  const int rr = wave * 16 + r16;
+  const bool row_valid = rr < rows;
+  const int tok = row0 + (row_valid ? rr / G : 0);
+  const int head = gkv * G + (row_valid ? rr % G : 0);
+  const int pos_row = row_valid ? positions[tok] : -1;
+  const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  bf16x8_t qf[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks)
+    qf[ks] = row_valid ? *reinterpret_cast<const bf16x8_t*>(
+                             q + ((size_t)tok * nh + head) * D + ks * 32 + grp * 8)
+                       : zero8;
+
+  const int pos_first = positions[row0];
+  const int pos_last = positions[row0 + count - 1];
+  const int lo = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
+  const int hi = pos_last;
+  // what this wave's rows can see at most
+  const int wave_first_row = wave * 16;
+  const bool wave_active = wave_first_row < rows;
+  int wave_last_tok = (wave_first_row + 15) / G;
+  if (wave_last_tok > count - 1) wave_last_tok = count - 1;
+  const int wave_hi = wave_active ? positions[row0 + wave_last_tok] : -1;
+
+  f32x4_t o[DBLK];
+#pragma unroll
+  for (int db = 0; db < DBLK; ++db) o[db] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  const size_t vofs = (size_t)nkv * page_size * D;
+  for (int tile0 = (lo / AM_KT) * AM_KT; tile0 <= hi; tile0 += AM_KT) {
+    __syncthreads();
+    // keys: lanes run along the head dimension (coalesced rows)
+#pragma unroll
+    for (int v = 0; v < AM_KT * VEC_PER_ROW / 256; ++v) {
+      const int idx = tid + v * 256;
+      const int j = idx / VEC_PER_ROW, c = (idx % VEC_PER_ROW) * 8;
+      const int kp = tile0 + j;
+      bf16x8_t kx = zero8;
+      if (kp >= lo && kp <= hi) {
+        const int page = table[kp / page_size];
+        if (page >= 0)
+          kx = *reinterpret_cast<const bf16x8_t*>(
+              kv + ((((size_t)page * 2) * nkv + gkv) * page_size + kp % page_size) * D + c);
+      }
+      *reinterpret_cast<bf16x8_t*>(Ks + j * LDK + c) = kx;
+    }
+    // values, transposed: lanes run along the keys so that the 2-byte stores of one
+    // instruction fall side by side
+#pragma unroll
+    for (int v = 0; v < AM_KT * VEC_PER_ROW / 256; ++v) {
+      const int idx = tid + v * 256;
+      const int j = idx % AM_KT, c = (idx / AM_KT) * 8;
+      const int kp = tile0 + j;
+      bf16x8_t vx = zero8;
+      if (kp >= lo && kp <= hi) {
+        const int page = table[kp / page_size];
+        if (page >= 0)
+          vx = *reinterpret_cast<const bf16x8_t*>(
+              kv + ((((size_t)page * 2) * nkv + gkv) * page_size + kp % page_size) * D + vofs + c);
+      }
+      // key j of the tile sits in slot: 32-key step, then lane group, then block, then i
+      const int slot = (j & 32) + ((j & 15) >> 2) * 8 + ((j >> 4) & 1) * 4 + (j & 3);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) Vt[(c + e) * LDV + slot] = vx[e];
+    }
+    __syncthreads();
+
+    if (wave_active && tile0 <= wave_hi) {
+      f32x4_t s[4];
+#pragma unroll
+      for (int jb = 0; jb < 4; ++jb) {
+        s[jb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(
+              Ks + (jb * 16 + r16) * LDK + ks * 32 + grp * 8);
+          s[jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], s[jb], 0, 0, 0);
+        }
+      }
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int jb = 0; jb < 4; ++jb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int kp = tile0 + jb * 16 + grp * 4 + i;
+          bool valid = kp <= pos_row && kp >= lo;
+          if (window > 0 && kp <= pos_row - window) valid = false;
+          const float v = valid ? s[jb][i] * scale : -INFINITY;
+          s[jb][i] = v;
+          tmax = fmaxf(tmax, v);
+        }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float m_new = fmaxf(m, tmax);
+      const float m_use = m_new > -INFINITY ? m_new : 0.f;
+      const float alpha = expf(m - m_use);          // m = -inf gives 0
+      float psum = 0.f;
+#pragma unroll
+      for (int jb = 0; jb < 4; ++jb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float p = expf(s[jb][i] - m_use);   // masked scores give 0
+          s[jb][i] = p;
+          psum += p;
+        }
+      psum += __shfl_xor(psum, 16, 64);
+      psum += __shfl_xor(psum, 32, 64);
+      l = l * alpha + psum;
+      m = m_new;
+#pragma unroll
+      for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[db][i] *= alpha;
+      bf16x8_t pf[2];
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          pf[kk][i] = (bf16_t)s[2 * kk][i];
+          pf[kk][4 + i] = (bf16_t)s[2 * kk + 1][i];
+        }
+#pragma unroll
+      for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+          const bf16x8_t vf = *reinterpret_cast<const bf16x8_t*>(
+              Vt + (db * 16 + r16) * LDV + kk * 32 + grp * 8);
+          o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[kk], o[db], 0, 0, 0);
+        }
+    }
+  }
+
+  if (row_valid) {
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    bf16_t* dst = out + ((size_t)tok * nh + head) * D;
+#pragma unroll
+    for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) dst[db * 16 + grp * 4 + i] = (bf16_t)(o[db][i] * inv);
+  }
+}
+
 template <typename T, int KT>
 static int launch_attention(const void* q, void* out, const void* kv, const int* block_table,
                             int bt_stride, const int* positions, const int* wi_seq,
@@ -281,5 +470,31 @@ extern "C" int za_paged_attention(const void* q, void* out, const void* kv, cons
   else
     hipLaunchKernelGGL((attention_combine_kernel<bf16_t>), grid, block, 0, stream, part_acc,
                        part_ml, (bf16_t*)out, d, nsplit);
+  return za_launch_status();
+}
+
+// Matrix-core variant: bfloat16 only, head_dim 64 or 128, (nh / nkv) dividing 16, work
+// items of at most 64 / (nh / nkv) query rows.  Returns ZA_ERR_UNSUPPORTED otherwise.
+extern "C" int za_paged_attention_mfma(const void* q, void* out, const void* kv,
+                                       const int* block_table, int bt_stride,
+                                       const int* positions, const int* wi_seq,
+                                       const int* wi_row0, const int* wi_count, int n_items,
+                                       int nh, int nkv, int d, int page_size, float scale,
+                                       int window, hipStream_t stream) {
+  if (n_items == 0) return 0;
+  if (n_items < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || page_size <= 0 || bt_stride <= 0 ||
+      !q || !out || !kv || !block_table || !positions || !wi_seq || !wi_row0 || !wi_count)
+    return ZA_ERR_ARG;
+  const int G = nh / nkv;
+  if ((d != 64 && d != 128) || G > 16 || 16 % G != 0 || nkv > 65535) return ZA_ERR_UNSUPPORTED;
+  dim3 grid(n_items, nkv), block(256);
+  if (d == 64)
+    hipLaunchKernelGGL((paged_attention_mfma_kernel<64>), grid, block, 0, stream,
+                       (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
+                       positions, wi_seq, wi_row0, wi_count, nh, nkv, page_size, scale, window);
+  else
+    hipLaunchKernelGGL((paged_attention_mfma_kernel<128>), grid, block, 0, stream,
+                       (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
+                       positions, wi_seq, wi_row0, wi_count, nh, nkv, page_size, scale, window);
   return za_launch_status();
 }

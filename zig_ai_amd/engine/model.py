@@ -89,7 +89,7 @@ class DecoderModel:
             if self.cache_needs[call.cache] is not None and call.cache not in writers:
                 raise ValueError(f"cache {call.cache} is read but no run-order entry writes it")
         self.item_granularities = sorted({
-            b.mixer.rows_per_item for b in self.blocks if hasattr(b.mixer, "rows_per_item")})
+            g for b in self.blocks for g in getattr(b.mixer, "item_granularities", ())})
         self.kernel_sources = sorted(sources)
         # A step may be recorded into a HIP graph only if no part looks at the step's
         # numbers on the host while it runs.

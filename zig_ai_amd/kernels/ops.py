@@ -36,6 +36,10 @@ _SIGNATURES = {
                                           c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                           c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
                                           c_int, c_int, c_int, c_void_p],
+    ("attention", "za_paged_attention_mfma"): [c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                               c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                               c_int, c_int, c_int, c_int, c_float, c_int,
+                                               c_void_p],
     ("shortconv", "za_short_conv"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_longlong,
                                      c_void_p],
@@ -151,12 +155,19 @@ def embed_gather(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
 
 
 # --------------------------------------------------------------------- gemm
+# Above this many rows a bfloat16 projection without bias goes to the library.
+LIBRARY_GEMM_ROWS = 64
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
            out_dtype: Optional[torch.dtype] = None, force_tiled: bool = False) -> torch.Tensor:
     """``x [M, K] @ weight[N, K]^T + bias`` with 32-bit accumulation.
 
-    bfloat16 weights use the matrix-core kernels (``x`` must be bfloat16); 32-bit
-    weights use the all-32-bit kernel (``x`` may be either type and is widened)."""
+    bfloat16 weights use the matrix-core kernels of csrc/gemm.hip up to
+    ``LIBRARY_GEMM_ROWS`` rows, and always when a bias or 32-bit output is asked
+    for; larger plain products go to the GEMM library.  32-bit weights use the
+    all-32-bit kernel (``x`` may be either type and is widened): no library, no
+    reduced-precision matrix mode."""
     if x.dim() != 2 or weight.dim() != 2:
         raise KernelError(f"linear takes x [M, K] and weight [N, K], got {tuple(x.shape)} and "
                           f"{tuple(weight.shape)}")
@@ -177,6 +188,12 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
             raise KernelError("a bfloat16 weight needs bfloat16 activations")
         if K % 8:
             raise KernelError(f"the bfloat16 GEMM needs K to be a multiple of 8, got K={K}")
+        if M > LIBRARY_GEMM_ROWS and bias is None and out_dtype == torch.bfloat16 \
+                and not force_tiled:
+            # Many rows: the vendor's GEMM library, as the reference does for every
+            # projection (/root/reference/src/matmul/root.zig:292-313 calls cuBLAS).
+            torch.mm(x, weight.t(), out=out)
+            return out
         rc = _fn("gemm", "za_gemm_bf16")(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out),
                                          _code(out_dtype), M, N, K, 1 if force_tiled else 0,
                                          _stream())
@@ -285,6 +302,53 @@ def paged_attention(q: torch.Tensor, kv_cache: torch.Tensor, block_table: torch.
         _ptr(part_acc), _ptr(part_ml), _code(q.dtype), nh, nkv, d, page_size, float(scale),
         int(window), int(keys_per_split), int(nsplit), _stream())
     _check(rc, "paged_attention")
+    return out
+
+
+ATTENTION_MFMA_ROWS = 64
+
+
+def attention_mfma_supported(dtype: torch.dtype, num_heads: int, num_kv_heads: int,
+                             head_dim: int) -> bool:
+    """Whether the matrix-core attention kernel takes these sizes."""
+    group = num_heads // num_kv_heads
+    return (dtype == torch.bfloat16 and head_dim in (64, 128) and group <= 16
+            and 16 % group == 0)
+
+
+def paged_attention_mfma(q: torch.Tensor, kv_cache: torch.Tensor, block_table: torch.Tensor,
+                         positions: torch.Tensor, item_seq: torch.Tensor,
+                         item_row0: torch.Tensor, item_count: torch.Tensor, n_items: int,
+                         scale: float, window: int = 0) -> torch.Tensor:
+    """The same attention on the matrix cores (bfloat16, head_dim 64 or 128, query
+    heads per key/value head dividing 16).  Work items hold at most
+    ``ATTENTION_MFMA_ROWS // (heads // kv_heads)`` query rows; contexts are not cut."""
+    if q.dim() != 3:
+        raise KernelError(f"q must be [T, heads, head_dim], got {tuple(q.shape)}")
+    T, nh, d = q.shape
+    _need(q, "q", torch.bfloat16)
+    _need(kv_cache, "kv_cache", torch.bfloat16)
+    if kv_cache.dim() != 5 or kv_cache.shape[1] != 2 or kv_cache.shape[4] != d:
+        raise KernelError(f"kv_cache has shape {tuple(kv_cache.shape)}, expected "
+                          f"[pages, 2, kv_heads, page_size, {d}]")
+    nkv, page_size = kv_cache.shape[2], kv_cache.shape[3]
+    if nh % nkv or not attention_mfma_supported(q.dtype, nh, nkv, d):
+        raise KernelError(f"the matrix-core attention kernel does not take {nh} heads, {nkv} "
+                          f"key/value heads, head_dim {d}")
+    _need(block_table, "block_table", torch.int32)
+    if block_table.dim() != 2:
+        raise KernelError("block_table must be [requests, max_pages]")
+    _need(positions, "positions", torch.int32, (T,))
+    for name, t in (("item_seq", item_seq), ("item_row0", item_row0), ("item_count", item_count)):
+        _need(t, name, torch.int32)
+        if t.numel() < n_items:
+            raise KernelError(f"{name} holds {t.numel()} entries, fewer than {n_items} items")
+    out = torch.empty_like(q)
+    rc = _fn("attention", "za_paged_attention_mfma")(
+        _ptr(q), _ptr(out), _ptr(kv_cache), _ptr(block_table), block_table.shape[1],
+        _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, nh, nkv, d,
+        page_size, float(scale), int(window), _stream())
+    _check(rc, "paged_attention_mfma")
     return out
 
 

@@ -85,7 +85,13 @@ class GroupedQueryAttention(Mixer):
                              f"kernel's limit of {ops.ATTENTION_MAX_ROWS}")
         if self.head_dim % 16 or self.head_dim > 256:
             raise ValueError(f"head_dim {self.head_dim} must be a multiple of 16, at most 256")
+        # tokens per work item of the two attention kernels
         self.rows_per_item = max(1, ops.ATTENTION_MAX_ROWS // self.group)
+        self.mfma = ops.attention_mfma_supported(runtime.dtype, self.num_heads,
+                                                 self.num_kv_heads, self.head_dim)
+        self.mfma_rows_per_item = max(1, ops.ATTENTION_MFMA_ROWS // self.group)
+        self.item_granularities = [self.rows_per_item] + (
+            [self.mfma_rows_per_item] if self.mfma else [])
         self.window = int(params.get("window") or 0)
         scale = params.get("softmax_scale")
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
@@ -133,11 +139,18 @@ class GroupedQueryAttention(Mixer):
             q = ops.qk_norm_rope_kv_write(packed.contiguous(), step.positions, slots, None, None,
                                           None, cache.kv, nh, nkv, d, 0, False, self.eps,
                                           write_kv=cache.writes)
-        item_seq, item_row0, item_count, n_items = step.attention_items(self.rows_per_item)
-        keys, nsplit = plan_split(n_items, nkv, step.max_keys)
-        o = ops.paged_attention(q, cache.kv, step.block_tables[cache.group], step.positions,
-                                item_seq, item_row0, item_count, n_items, self.scale, self.window,
-                                keys, nsplit)
+        if self.mfma and step.n_tokens > step.n_seqs:
+            # prompt portions in the step: both products on the matrix cores
+            o = ops.paged_attention_mfma(q, cache.kv, step.block_tables[cache.group],
+                                         step.positions,
+                                         *step.attention_items(self.mfma_rows_per_item),
+                                         self.scale, self.window)
+        else:
+            item_seq, item_row0, item_count, n_items = step.attention_items(self.rows_per_item)
+            keys, nsplit = plan_split(n_items, nkv, step.max_keys)
+            o = ops.paged_attention(q, cache.kv, step.block_tables[cache.group], step.positions,
+                                    item_seq, item_row0, item_count, n_items, self.scale,
+                                    self.window, keys, nsplit)
         return ops.linear(o.view(T, nh * d), self.w_out, self.b_out)
 
 
