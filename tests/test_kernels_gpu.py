@@ -81,6 +81,20 @@ def test_add_rmsnorm_selected_rows(dtype):
     assert rel_err(out, expect) < tol_of(dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width", [64, 100, 2048, 3000, 4096, 5000])
+def test_add_rmsnorm_partial_sums(dtype, width):
+    """A stack of partial sums as delta is added up while it is read."""
+    x = rand((5, width), torch.float32, 1)
+    parts = rand((3, 5, width), torch.float32, 2)
+    w = rand((width,), torch.float32, 3)
+    res = x.clone().to(dev())
+    out = ops().add_rmsnorm(res, parts.to(dev()), w.to(dev()), 1e-5, dtype)
+    h = x.double() + parts.double().sum(0)
+    assert rel_err(res, h) < F32_TOL
+    assert rel_err(out, plain.rms_norm(h, w.double(), 1e-5)) < tol_of(dtype)
+
+
 def test_rmsnorm_reference_vectors():
     """The inputs of /root/reference/src/transformer/norm.zig:83-103 ([1,2,3,4] and
     [1,1,1,1], weight 1): the values follow from the formula; ones stay ones."""
@@ -171,6 +185,18 @@ def test_gemm_bf16_decode_rows_all_k_ranges(M, N, K):
     x, w, b = rand((M, K), torch.bfloat16, 27), rand((N, K), torch.bfloat16, 28), rand((N,), torch.float32, 29)
     out = ops().linear(x.to(dev()), w.to(dev()), b.to(dev()), out_dtype=torch.float32)
     assert rel_err(out, x.double() @ w.double().T + b.double()) < F32_TOL
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 64, 4096), (8, 2048, 8192), (16, 2048, 8192), (8, 100, 4128),
+                                   (3, 4096, 4096)])
+def test_gemm_bf16_partial_sums(M, N, K):
+    """K split over workgroups: the stack of partial results sums to the product."""
+    x, w, b = rand((M, K), torch.bfloat16, 30), rand((N, K), torch.bfloat16, 31), rand((N,), torch.float32, 32)
+    stack = ops().linear(x.to(dev()), w.to(dev()), b.to(dev()), partial_ok=True)
+    assert stack.dim() == 3 and stack.dtype == torch.float32 and stack.shape[0] in (2, 4)
+    assert rel_err(stack.sum(0), x.double() @ w.double().T + b.double()) < F32_TOL
+    big = ops().linear(rand((40, K), torch.bfloat16, 33).to(dev()), w.to(dev()), partial_ok=True)
+    assert big.dim() == 2                                   # only decode batches are split
 
 
 def test_gemm_bf16_refuses_odd_k():
@@ -508,6 +534,19 @@ def test_argmax_first_occurrence():
     out = ops().argmax(logits.to(dev())).cpu().tolist()
     assert out == [plain.argmax_first(r) for r in logits]
     assert out[0] == 17 and out[1] == 999 and out[2] == 0 and out[3] == 0
+
+
+@pytest.mark.parametrize("rows,vocab", [(1, 65536), (8, 65536), (3, 10000), (70, 65536), (2, 301)])
+def test_argmax_long_rows(rows, vocab):
+    """Few rows of a long vocabulary are cut into chunks; ties across chunks still
+    go to the first index."""
+    logits = rand((rows, vocab), torch.float32, 102)
+    logits[0, vocab - 1] = logits[0, 7] = 99.0
+    if rows > 1:
+        logits[1, vocab // 2] = logits[1, vocab // 2 + 4097 if vocab > 9000 else vocab - 2] = 99.0
+    out = ops().argmax(logits.to(dev())).cpu().tolist()
+    assert out == logits.argmax(dim=1).tolist() or out == [plain.argmax_first(r) for r in logits]
+    assert out[0] == 7
 
 
 @pytest.mark.parametrize("vocab", [50, 1000, 65536])

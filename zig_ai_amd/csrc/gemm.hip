@@ -261,6 +261,10 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__
 // loads in flight at once.  The NW waves of a workgroup split K; their partial
 // tiles meet in LDS (double-buffered, one barrier per row group) and wave 0
 // writes the sum.  A workgroup walks `groups_per_block` consecutive row groups.
+//
+// K may also be split over workgroups (gridDim.y ranges of NW * KSTEPS * 32): each
+// range then writes a 32-bit partial result [range][M][N] that the consumer adds up
+// (the bias goes into range 0).
 template <int NW, int KSTEPS, typename TC>
 __global__ void __launch_bounds__(NW * 64)
 gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
@@ -270,7 +274,7 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int frag_row = lane & 15, frag_k = (lane >> 4) * 8;
-  const int kbase = wave * KSTEPS * 32 + frag_k;
+  const int kbase = (blockIdx.y * NW + wave) * KSTEPS * 32 + frag_k;
   const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   constexpr int HALF = KSTEPS > 16 ? 16 : KSTEPS;   // weight fragments in flight at once
 
@@ -282,6 +286,7 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__
                                     : zero8;
   }
 
+  const bool partial = gridDim.y > 1;
   for (int g = 0; g < groups_per_block; ++g) {
     const int n0 = (blockIdx.x * groups_per_block + g) * 16;
     if (n0 >= N) break;
@@ -301,10 +306,12 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__
       for (int s = 0; s < HALF; ++s)
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[s], xa[h + s], acc, 0, 0, 0);
     }
-    float* mine = red[g & 1][wave][lane];
+    if (NW > 1) {
+      float* mine = red[g & 1][wave][lane];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) mine[r] = acc[r];
-    __syncthreads();
+      for (int r = 0; r < 4; ++r) mine[r] = acc[r];
+      __syncthreads();
+    }
     if (wave == 0) {
       const int m = lane & 15, nn = n0 + (lane >> 4) * 4;
       if (m < M) {
@@ -312,15 +319,51 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__
         for (int r = 0; r < 4; ++r) {
           const int n = nn + r;
           if (n >= N) continue;
-          float v = red[g & 1][0][lane][r];
+          float v = acc[r];
+          if (NW > 1) {
+            v = red[g & 1][0][lane][r];
 #pragma unroll
-          for (int w = 1; w < NW; ++w) v += red[g & 1][w][lane][r];
-          if (bias) v += bias[n];
-          C[(size_t)m * N + n] = from_f32<TC>(v);
+            for (int w = 1; w < NW; ++w) v += red[g & 1][w][lane][r];
+          }
+          if (bias && blockIdx.y == 0) v += bias[n];
+          if (partial)
+            reinterpret_cast<float*>(C)[((size_t)blockIdx.y * M + m) * N + n] = v;
+          else
+            C[(size_t)m * N + n] = from_f32<TC>(v);
         }
       }
     }
   }
+}
+
+static int launch_rows16(const bf16_t* a, const bf16_t* w, const float* bias, void* C, int c_dtype,
+                         int M, int N, int K, int ksplit, hipStream_t stream) {
+  if (ksplit < 1 || (ksplit > 1 && (c_dtype != 0 || K % (ksplit * 32) != 0))) return ZA_ERR_ARG;
+  const int kper = (K + ksplit - 1) / ksplit;   // K range of one workgroup
+  if (kper > 8192) return ZA_ERR_UNSUPPORTED;
+  const int groups = (N + 15) / 16;
+  // enough workgroups to cover the machine a few times, few enough to amortise
+  // loading the activations
+  int per_block = 1;
+  while (per_block < 8 && groups / (per_block * 2) >= 1024) per_block *= 2;
+  dim3 grid((groups + per_block - 1) / per_block, ksplit);
+#define ZA_R16_CASE(NW, KS)                                                                   \
+  {                                                                                           \
+    dim3 block(NW * 64);                                                                      \
+    if (c_dtype == 0)                                                                         \
+      hipLaunchKernelGGL((gemm_bf16_rows16_kernel<NW, KS, float>), grid, block, 0,    \
+                         stream, a, w, bias, (float*)C, M, N, K, per_block);                  \
+    else                                                                                      \
+      hipLaunchKernelGGL((gemm_bf16_rows16_kernel<NW, KS, bf16_t>), grid, block, 0,   \
+                         stream, a, w, bias, (bf16_t*)C, M, N, K, per_block);                 \
+    return za_launch_status();                                                                \
+  }
+  if (kper <= 512) ZA_R16_CASE(1, 16)
+  if (kper <= 1024) ZA_R16_CASE(2, 16)
+  if (kper <= 2048) ZA_R16_CASE(4, 16)
+  if (kper <= 4096) ZA_R16_CASE(8, 16)
+  ZA_R16_CASE(8, 32)
+#undef ZA_R16_CASE
 }
 
 // ------------------------------------------------------------------ launchers
@@ -352,30 +395,8 @@ extern "C" int za_gemm_bf16(const void* A, const void* W, const float* bias, voi
   if (c_dtype != 0 && c_dtype != 1) return ZA_ERR_UNSUPPORTED;
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
-  if (M <= 16 && K <= 8192 && !force_tiled) {
-    const int groups = (N + 15) / 16;
-    // enough workgroups to cover the machine a few times, few enough to amortise
-    // loading the activations
-    int per_block = 1;
-    while (per_block < 8 && groups / (per_block * 2) >= 1024) per_block *= 2;
-    dim3 grid((groups + per_block - 1) / per_block);
-#define ZA_R16_CASE(NW, KS)                                                                    \
-  {                                                                                            \
-    dim3 block(NW * 64);                                                                       \
-    if (c_dtype == 0)                                                                          \
-      hipLaunchKernelGGL((gemm_bf16_rows16_kernel<NW, KS, float>), grid, block, 0, stream, a,  \
-                         w, bias, (float*)C, M, N, K, per_block);                              \
-    else                                                                                       \
-      hipLaunchKernelGGL((gemm_bf16_rows16_kernel<NW, KS, bf16_t>), grid, block, 0, stream, a, \
-                         w, bias, (bf16_t*)C, M, N, K, per_block);                             \
-    return za_launch_status();                                                                 \
-  }
-    if (K <= 512) ZA_R16_CASE(1, 16)
-    if (K <= 2048) ZA_R16_CASE(4, 16)
-    if (K <= 4096) ZA_R16_CASE(8, 16)
-    ZA_R16_CASE(8, 32)
-#undef ZA_R16_CASE
-  }
+  if (M <= 16 && K <= 8192 && !force_tiled)
+    return launch_rows16(a, w, bias, C, c_dtype, M, N, K, 1, stream);
   if (M <= 64 && !force_tiled) {
     dim3 grid((N + 15) / 16), block(256);
     const int mt = (M + 15) / 16;
@@ -403,4 +424,16 @@ extern "C" int za_gemm_bf16(const void* A, const void* W, const float* bias, voi
     hipLaunchKernelGGL((gemm_bf16_mfma_kernel<bf16_t>), grid, block, 0, stream, a, w, bias,
                        (bf16_t*)C, M, N, K);
   return za_launch_status();
+}
+
+// The decode kernel with K split over workgroups: 32-bit partial results
+// [ksplit][M][N] go into C (c_dtype must then be float32 and K a multiple of 32 * ksplit).
+extern "C" int za_gemm_bf16_rows16(const void* A, const void* W, const float* bias, void* C,
+                                   int c_dtype, int M, int N, int K, int ksplit,
+                                   hipStream_t stream) {
+  if (M == 0 || N == 0) return 0;
+  if (M < 0 || N < 0 || K <= 0 || !A || !W || !C) return ZA_ERR_ARG;
+  if (M > 16 || K % 8 != 0 || (c_dtype != 0 && c_dtype != 1)) return ZA_ERR_UNSUPPORTED;
+  return launch_rows16((const bf16_t*)A, (const bf16_t*)W, bias, C, c_dtype, M, N, K, ksplit,
+                       stream);
 }

@@ -11,11 +11,23 @@
 // squares, weight multiplied after the scale, no bias).
 #include "common.h"
 
+// `delta` may be a stack of `n_partials` partial sums (each `partial_stride`
+// elements apart): the pieces a projection split along K leaves to its consumer.
+template <typename TD>
+__device__ __forceinline__ float delta_at(const TD* dl, size_t i, int n_partials,
+                                          size_t partial_stride) {
+  float v = to_f32<TD>(dl[i]);
+  for (int p = 1; p < n_partials; ++p) v += to_f32<TD>(dl[i + p * partial_stride]);
+  return v;
+}
+
+// General form: two passes over the row, any width.
 template <typename TD, typename TO>
 __global__ void __launch_bounds__(256)
 add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
                    const float* __restrict__ weight, TO* __restrict__ out,
-                   const int* __restrict__ rows, int width, float eps, int write_residual) {
+                   const int* __restrict__ rows, int width, float eps, int write_residual,
+                   int n_partials, size_t partial_stride) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const size_t src = rows ? (size_t)rows[r] : (size_t)r;
@@ -26,7 +38,7 @@ add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
   float ss = 0.f;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float h = x ? x[i] : 0.f;
-    if (dl) h += to_f32<TD>(dl[i]);
+    if (dl) h += delta_at<TD>(dl, i, n_partials, partial_stride);
     if (write_residual) x[i] = h;
     ss += h * h;
   }
@@ -38,9 +50,60 @@ add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
       h = x[i];  // this thread stored it above
     } else {
       h = x ? x[i] : 0.f;
-      if (dl) h += to_f32<TD>(dl[i]);
+      if (dl) h += delta_at<TD>(dl, i, n_partials, partial_stride);
     }
     o[i] = from_f32<TO>(h * scale * weight[i]);
+  }
+}
+
+// Rows of at most 256 * 4 * VPT elements with width % 4 == 0: the row stays in
+// registers between the sum of squares and the scaling, one pass over memory.
+template <typename TD, typename TO, int VPT>
+__global__ void __launch_bounds__(256)
+add_rmsnorm_regs_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
+                        const float* __restrict__ weight, TO* __restrict__ out,
+                        const int* __restrict__ rows, int width, float eps, int write_residual,
+                        int n_partials, size_t partial_stride) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+  float* x = residual ? residual + src * width : nullptr;
+  const TD* dl = delta ? delta + src * width : nullptr;
+  TO* o = out + (size_t)r * width;
+  float h[VPT][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int v = 0; v < VPT; ++v) {
+    const int i = (threadIdx.x + v * 256) * 4;
+    if (i < width) {
+      if (x) {
+        const float4 t = *reinterpret_cast<const float4*>(x + i);
+        h[v][0] = t.x; h[v][1] = t.y; h[v][2] = t.z; h[v][3] = t.w;
+      } else {
+        h[v][0] = h[v][1] = h[v][2] = h[v][3] = 0.f;
+      }
+      if (dl) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) h[v][e] += delta_at<TD>(dl, i + e, n_partials, partial_stride);
+      }
+      if (write_residual)
+        *reinterpret_cast<float4*>(x + i) = make_float4(h[v][0], h[v][1], h[v][2], h[v][3]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ss += h[v][e] * h[v][e];
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float scale = 1.0f / sqrtf(ss / (float)width + eps);
+#pragma unroll
+  for (int v = 0; v < VPT; ++v) {
+    const int i = (threadIdx.x + v * 256) * 4;
+    if (i < width) {
+      const float4 w = *reinterpret_cast<const float4*>(weight + i);
+      o[i] = from_f32<TO>(h[v][0] * scale * w.x);
+      o[i + 1] = from_f32<TO>(h[v][1] * scale * w.y);
+      o[i + 2] = from_f32<TO>(h[v][2] * scale * w.z);
+      o[i + 3] = from_f32<TO>(h[v][3] * scale * w.w);
+    }
   }
 }
 
@@ -64,16 +127,25 @@ embed_gather_kernel(const int* __restrict__ tokens, const T* __restrict__ table,
 extern "C" int za_add_rmsnorm(void* residual, const void* delta, int delta_dtype,
                               const float* weight, void* out, int out_dtype, const int* rows,
                               int n_rows, int width, float eps, int write_residual,
-                              hipStream_t stream) {
+                              int n_partials, long long partial_stride, hipStream_t stream) {
   if (n_rows == 0) return 0;
-  if (n_rows < 0 || width <= 0 || (!residual && !delta) || !weight || !out) return ZA_ERR_ARG;
+  if (n_rows < 0 || width <= 0 || (!residual && !delta) || !weight || !out || n_partials < 1)
+    return ZA_ERR_ARG;
+  if (n_partials > 1 && (!delta || partial_stride <= 0)) return ZA_ERR_ARG;
   if (!residual || rows) write_residual = 0;
   dim3 grid(n_rows), block(256);
   float* res = (float*)residual;
+  const int vpt = width % 4 == 0 ? (width / 4 + 255) / 256 : 0;   // vectors per thread
+#define ZA_NORM_LAUNCH(KERNEL, TD, TO)                                                      \
+  hipLaunchKernelGGL((KERNEL), grid, block, 0, stream, res, (const TD*)delta, weight,       \
+                     (TO*)out, rows, width, eps, write_residual, n_partials,                \
+                     (size_t)partial_stride)
 #define ZA_NORM_CASE(DD, TD, OD, TO)                                                        \
   if (delta_dtype == DD && out_dtype == OD) {                                               \
-    hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TO>), grid, block, 0, stream, res,           \
-                       (const TD*)delta, weight, (TO*)out, rows, width, eps, write_residual); \
+    if (vpt == 1) ZA_NORM_LAUNCH((add_rmsnorm_regs_kernel<TD, TO, 1>), TD, TO);             \
+    else if (vpt == 2) ZA_NORM_LAUNCH((add_rmsnorm_regs_kernel<TD, TO, 2>), TD, TO);        \
+    else if (vpt >= 3 && vpt <= 4) ZA_NORM_LAUNCH((add_rmsnorm_regs_kernel<TD, TO, 4>), TD, TO); \
+    else ZA_NORM_LAUNCH((add_rmsnorm_kernel<TD, TO>), TD, TO);                              \
     return za_launch_status();                                                              \
   }
   ZA_NORM_CASE(0, float, 0, float)
@@ -81,6 +153,7 @@ extern "C" int za_add_rmsnorm(void* residual, const void* delta, int delta_dtype
   ZA_NORM_CASE(1, bf16_t, 0, float)
   ZA_NORM_CASE(1, bf16_t, 1, bf16_t)
 #undef ZA_NORM_CASE
+#undef ZA_NORM_LAUNCH
   return ZA_ERR_UNSUPPORTED;
 }
 

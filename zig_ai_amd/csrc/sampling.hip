@@ -50,6 +50,61 @@ argmax_kernel(const float* __restrict__ logits, int vocab, int* __restrict__ out
   }
 }
 
+// Greedy choice for few rows of a large vocabulary: the row is cut into
+// gridDim.y chunks so that more than a handful of workgroups read it; each
+// writes its (maximum, first index) and `argmax_merge_kernel` picks the winner,
+// the lower index among equal maxima.
+__global__ void __launch_bounds__(SM_THREADS)
+argmax_chunk_kernel(const float* __restrict__ logits, int vocab, float* __restrict__ part_v,
+                    int* __restrict__ part_i) {
+  __shared__ float best_v[SM_THREADS / 64];
+  __shared__ int best_i[SM_THREADS / 64];
+  const int chunk = (vocab + gridDim.y - 1) / gridDim.y;
+  const int begin = blockIdx.y * chunk;
+  const int end = begin + chunk < vocab ? begin + chunk : vocab;
+  const float* row = logits + (size_t)blockIdx.x * vocab;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = begin + threadIdx.x; i < end; i += SM_THREADS) {
+    const float v = row[i];
+    if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, 64);
+    const int oi = __shfl_xor(bi, o, 64);
+    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) { best_v[wave] = bv; best_i[wave] = bi; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < SM_THREADS / 64; ++w)
+      if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) { bv = best_v[w]; bi = best_i[w]; }
+    part_v[blockIdx.x * gridDim.y + blockIdx.y] = bv;
+    part_i[blockIdx.x * gridDim.y + blockIdx.y] = bi;
+  }
+}
+
+__global__ void __launch_bounds__(64)
+argmax_merge_kernel(const float* __restrict__ part_v, const int* __restrict__ part_i, int chunks,
+                    int* __restrict__ out) {
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int c = threadIdx.x; c < chunks; c += 64) {
+    const float v = part_v[blockIdx.x * chunks + c];
+    const int i = part_i[blockIdx.x * chunks + c];
+    if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, 64);
+    const int oi = __shfl_xor(bi, o, 64);
+    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+  }
+  if (threadIdx.x == 0) out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+}
+
 __global__ void __launch_bounds__(SM_THREADS)
 sample_kernel(const float* __restrict__ logits, int vocab, const float* __restrict__ temperature,
               const int* __restrict__ top_k, const float* __restrict__ top_p,
@@ -183,11 +238,23 @@ repetition_penalty_kernel(float* __restrict__ logits, int vocab, const int* __re
   else if (v < 0.f) *p = v * factors[e];
 }
 
-extern "C" int za_argmax(const float* logits, int n_rows, int vocab, int* out,
-                         hipStream_t stream) {
+// `part_v` / `part_i`: workspace of n_rows * chunks entries each when chunks > 1.
+extern "C" int za_argmax(const float* logits, int n_rows, int vocab, int* out, float* part_v,
+                         int* part_i, int chunks, hipStream_t stream) {
   if (n_rows == 0) return 0;
-  if (n_rows < 0 || vocab <= 0 || !logits || !out) return ZA_ERR_ARG;
-  hipLaunchKernelGGL(argmax_kernel, dim3(n_rows), dim3(SM_THREADS), 0, stream, logits, vocab, out);
+  if (n_rows < 0 || vocab <= 0 || !logits || !out || chunks < 1) return ZA_ERR_ARG;
+  if (chunks == 1) {
+    hipLaunchKernelGGL(argmax_kernel, dim3(n_rows), dim3(SM_THREADS), 0, stream, logits, vocab,
+                       out);
+    return za_launch_status();
+  }
+  if (!part_v || !part_i || chunks > 65535) return ZA_ERR_ARG;
+  hipLaunchKernelGGL(argmax_chunk_kernel, dim3(n_rows, chunks), dim3(SM_THREADS), 0, stream,
+                     logits, vocab, part_v, part_i);
+  int rc = za_launch_status();
+  if (rc != 0) return rc;
+  hipLaunchKernelGGL(argmax_merge_kernel, dim3(n_rows), dim3(64), 0, stream, part_v, part_i,
+                     chunks, out);
   return za_launch_status();
 }
 

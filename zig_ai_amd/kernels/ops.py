@@ -22,7 +22,7 @@ _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 
 _SIGNATURES = {
     ("norm", "za_add_rmsnorm"): [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p,
-                                 c_int, c_int, c_float, c_int, c_void_p],
+                                 c_int, c_int, c_float, c_int, c_int, c_longlong, c_void_p],
     ("norm", "za_embed_gather"): [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
     ("gemm", "za_gemm_f32"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                               c_int, c_void_p],
@@ -45,7 +45,10 @@ _SIGNATURES = {
                                      c_void_p],
     ("activation", "za_swiglu"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     ("activation", "za_cast"): [c_void_p, c_int, c_void_p, c_int, c_longlong, c_void_p],
-    ("sampling", "za_argmax"): [c_void_p, c_int, c_int, c_void_p, c_void_p],
+    ("sampling", "za_argmax"): [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                                c_void_p],
+    ("gemm", "za_gemm_bf16_rows16"): [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                      c_int, c_int, c_void_p],
     ("sampling", "za_sample"): [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                 c_void_p, c_void_p],
     ("sampling", "za_repetition_penalty"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
@@ -114,28 +117,37 @@ def _need(t: torch.Tensor, name: str, dtype=None, shape: Optional[Tuple[int, ...
 def add_rmsnorm(residual: Optional[torch.Tensor], delta: Optional[torch.Tensor],
                 weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
                 rows: Optional[torch.Tensor] = None, write_residual: bool = True) -> torch.Tensor:
-    """``out = rmsnorm(residual + delta) * weight``; see csrc/norm.hip."""
+    """``out = rmsnorm(residual + delta) * weight``; see csrc/norm.hip.  ``delta`` may
+    be a stack ``[P, rows, width]`` of 32-bit partial sums, which are added up."""
     if residual is None and delta is None:
         raise KernelError("add_rmsnorm needs residual or delta")
-    ref = residual if residual is not None else delta
-    if ref.dim() != 2:
-        raise KernelError(f"add_rmsnorm takes [rows, width], got {tuple(ref.shape)}")
-    n, width = ref.shape
+    n_partials, partial_stride = 1, 0
+    if delta is not None and delta.dim() == 3:
+        _need(delta, "delta", torch.float32)
+        n_partials = delta.shape[0]
+        partial_stride = delta.shape[1] * delta.shape[2]
+        shape2 = tuple(delta.shape[1:])
+    else:
+        shape2 = tuple((residual if residual is not None else delta).shape)
+    if len(shape2) != 2:
+        raise KernelError(f"add_rmsnorm takes [rows, width], got {shape2}")
+    n, width = shape2
     if residual is not None:
         _need(residual, "residual", torch.float32, (n, width))
-    if delta is not None:
+    if delta is not None and delta.dim() == 2:
         _need(delta, "delta", (torch.float32, torch.bfloat16), (n, width))
     _need(weight, "weight", torch.float32, (width,))
     n_out = n
     if rows is not None:
         _need(rows, "rows", torch.int32)
         n_out = rows.numel()
+    ref = residual if residual is not None else delta
     out = torch.empty((n_out, width), dtype=out_dtype, device=ref.device)
     rc = _fn("norm", "za_add_rmsnorm")(
         _ptr(residual), _ptr(delta), _code(delta.dtype) if delta is not None else 0, _ptr(weight),
         _ptr(out), _code(out_dtype), _ptr(rows), n_out, width, float(eps),
         1 if (write_residual and residual is not None and delta is not None and rows is None) else 0,
-        _stream())
+        n_partials, partial_stride, _stream())
     _check(rc, "add_rmsnorm")
     return out
 
@@ -159,15 +171,32 @@ def embed_gather(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
 LIBRARY_GEMM_ROWS = 64
 
 
+def _k_splits(M: int, N: int, K: int) -> int:
+    """Into how many ranges the decode kernel cuts K when its consumer accepts
+    partial sums: enough to give every compute unit work when N alone is too
+    small, each range at least 512 long."""
+    if M > 16 or N > 4096 or K < 4096:
+        return 1       # measured: below this the consumer's extra reads cost more than is won
+    for split in (4, 2):
+        if K % (split * 32) == 0:
+            return split
+    return 1
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
-           out_dtype: Optional[torch.dtype] = None, force_tiled: bool = False) -> torch.Tensor:
+           out_dtype: Optional[torch.dtype] = None, force_tiled: bool = False,
+           partial_ok: bool = False) -> torch.Tensor:
     """``x [M, K] @ weight[N, K]^T + bias`` with 32-bit accumulation.
 
     bfloat16 weights use the matrix-core kernels of csrc/gemm.hip up to
     ``LIBRARY_GEMM_ROWS`` rows, and always when a bias or 32-bit output is asked
     for; larger plain products go to the GEMM library.  32-bit weights use the
     all-32-bit kernel (``x`` may be either type and is widened): no library, no
-    reduced-precision matrix mode."""
+    reduced-precision matrix mode.
+
+    With ``partial_ok`` the result may come back as a stack ``[P, M, N]`` of 32-bit
+    partial sums (K split over more workgroups when N is small and M is a decode
+    batch); ``add_rmsnorm`` adds such a stack up while it reads it."""
     if x.dim() != 2 or weight.dim() != 2:
         raise KernelError(f"linear takes x [M, K] and weight [N, K], got {tuple(x.shape)} and "
                           f"{tuple(weight.shape)}")
@@ -188,6 +217,13 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
             raise KernelError("a bfloat16 weight needs bfloat16 activations")
         if K % 8:
             raise KernelError(f"the bfloat16 GEMM needs K to be a multiple of 8, got K={K}")
+        splits = _k_splits(M, N, K) if (partial_ok and not force_tiled and K <= 8192 * 4) else 1
+        if splits > 1:
+            stack = torch.empty((splits, M, N), dtype=torch.float32, device=x.device)
+            rc = _fn("gemm", "za_gemm_bf16_rows16")(_ptr(x), _ptr(weight), _ptr(bias), _ptr(stack),
+                                                    0, M, N, K, splits, _stream())
+            _check(rc, "gemm_bf16_rows16", f"M={M} N={N} K={K} splits={splits}")
+            return stack
         if M > LIBRARY_GEMM_ROWS and bias is None and out_dtype == torch.bfloat16 \
                 and not force_tiled:
             # Many rows: the vendor's GEMM library, as the reference does for every
@@ -414,12 +450,20 @@ def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
 
 # ------------------------------------------------------------------ sampling
 def argmax(logits: torch.Tensor) -> torch.Tensor:
+    """First index of each row's maximum."""
     _need(logits, "logits", torch.float32)
     if logits.dim() != 2:
         raise KernelError("argmax takes [rows, vocab]")
-    out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
-    rc = _fn("sampling", "za_argmax")(_ptr(logits), logits.shape[0], logits.shape[1], _ptr(out),
-                                      _stream())
+    R, V = logits.shape
+    out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    # few rows of a long vocabulary: cut each row so that the machine is busy
+    chunks = 1 if R >= 64 else max(1, min(64, V // 4096))
+    part_v = part_i = None
+    if chunks > 1:
+        part_v = torch.empty((R, chunks), dtype=torch.float32, device=logits.device)
+        part_i = torch.empty((R, chunks), dtype=torch.int32, device=logits.device)
+    rc = _fn("sampling", "za_argmax")(_ptr(logits), R, V, _ptr(out), _ptr(part_v), _ptr(part_i),
+                                      chunks, _stream())
     _check(rc, "argmax")
     return out
 

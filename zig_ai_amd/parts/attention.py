@@ -151,7 +151,7 @@ class GroupedQueryAttention(Mixer):
             o = ops.paged_attention(q, cache.kv, step.block_tables[cache.group], step.positions,
                                     item_seq, item_row0, item_count, n_items, self.scale,
                                     self.window, keys, nsplit)
-        return ops.linear(o.view(T, nh * d), self.w_out, self.b_out)
+        return ops.linear(o.view(T, nh * d), self.w_out, self.b_out, partial_ok=True)
 
 
 register_mixer(GroupedQueryAttention.kind, GroupedQueryAttention)

@@ -6,6 +6,8 @@ never learns which model it is in.  Five families exist:
 
   mixer              ``forward(x, step, cache) -> y``; declares a cache need
   feed-forward       ``forward(x, step) -> y``
+                     (``y`` is ``[T, width]`` or a stack ``[P, T, width]`` of 32-bit
+                     partial sums that the following norm adds up)
   norm               ``forward(x) -> y`` and ``add_forward(residual, delta) -> y``
   position encoding  used by mixers: a rotation table, or ``apply(q, k, positions)``
   arrangement        wires two norms, a mixer and a feed-forward into a block
@@ -112,7 +114,11 @@ class Norm(Part):
                     rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``residual`` (32-bit, updated in place) takes ``delta``; the result is
         the norm of the sum.  With ``rows`` only those rows are produced and
-        ``residual`` is left alone.  Parts with a fused kernel override this."""
+        ``residual`` is left alone.  ``delta`` is what a mixer or feed-forward
+        returned: ``[T, width]``, or a stack ``[P, T, width]`` of 32-bit partial
+        sums whose sum over ``P`` is meant.  Parts with a fused kernel override this."""
+        if delta is not None and delta.dim() == 3:
+            delta = delta.sum(dim=0)
         if rows is not None:
             h = residual.index_select(0, rows.long())
             if delta is not None:

@@ -1,6 +1,7 @@
 """Dense SwiGLU feed-forward: ``(silu(x Wg^T) * (x Wu^T)) Wd^T`` without biases
 (/root/reference/src/transformer/ffn.zig:19-33).  Gate and up weights are fused
-into one ``[2I, H]`` matrix at load so the input is read once."""
+into one ``[2I, H]`` matrix at load so the input is read once.  The result may be
+a stack of partial sums (see ``Norm.add_forward``)."""
 
 from __future__ import annotations
 
@@ -38,7 +39,7 @@ class SwiGLU(FeedForward):
 
     def forward(self, x: torch.Tensor, step=None) -> torch.Tensor:
         gu = ops.linear(x, self.gate_up)
-        return ops.linear(ops.swiglu(gu), self.down)
+        return ops.linear(ops.swiglu(gu), self.down, partial_ok=True)
 
 
 register_feed_forward(SwiGLU.kind, SwiGLU)

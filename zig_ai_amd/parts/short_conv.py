@@ -61,7 +61,7 @@ class ShortConv(Mixer):
         z = ops.linear(x, self.w_in, self.b_in)
         y = ops.short_conv(z, self.w_conv, self.b_conv, cache.state, step.token_seq,
                            step.seq_start, step.slot_id)
-        return ops.linear(y, self.w_out, self.b_out)
+        return ops.linear(y, self.w_out, self.b_out, partial_ok=True)
 
 
 register_mixer(ShortConv.kind, ShortConv)
