@@ -81,6 +81,9 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None,
                     help="run fewer layers than the configuration has (both numbers are reported)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points")
+    ap.add_argument("--phase", choices=["all", "prefill", "decode"], default="all",
+                    help="measure only one phase (for profiling); the JSON line then holds "
+                         "only that phase")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -135,6 +138,12 @@ def main() -> int:
 
     # ---- prefill of 2,048 tokens, one request, one step
     T = 2048
+    if args.phase == "decode":
+        dt, ctx_mid = decode_run(args.batch, args.prompt_len, args.steps, args.warmup)
+        print(json.dumps({"phase": "decode", "batch": args.batch, "steps": args.steps,
+                          "ms_per_step": dt / args.steps * 1e3,
+                          "value": args.batch * args.steps / dt, "unit": "tokens/s"}), flush=True)
+        return 0
     runner = ModelRunner(model, page_size=page, num_pages=4 * (T // page + 1), num_slots=4)
     for r in range(2):                                  # warm-up
         runner.admit(("w", r))
@@ -157,6 +166,9 @@ def main() -> int:
         + 2.0 * vocab * cfg["hidden_size"]
     prefill = {"value": T / prefill_s, "tokens": T, "ms": prefill_s * 1e3,
                "frac": prefill_flops / prefill_s / PEAK_FLOPS["bf16"]}
+    if args.phase == "prefill":
+        print(json.dumps({"phase": "prefill", **prefill}), flush=True)
+        return 0
 
     # ---- the headline: batch 8 decoding from a 2,048-token context
     dt, ctx_mid = decode_run(args.batch, args.prompt_len, args.steps, args.warmup)
