@@ -294,7 +294,7 @@ def items_for(seq_lens, rows_per_item):
 
 
 def run_attention(dtype, nh, nkv, d, page_size, ctx, new, window=0, keys_per_split=0, nsplit=1,
-                  seed=30, sharpen=False, mfma=False):
+                  seed=30, sharpen=False, mfma=False, mfma_decode=False):
     """ctx[s] cached tokens and new[s] query tokens per request."""
     G = nh // nkv
     ks, vs, qs, pos = [], [], [], []
@@ -313,7 +313,11 @@ def run_attention(dtype, nh, nkv, d, page_size, ctx, new, window=0, keys_per_spl
     cache, table = paged_from_dense(ks, vs, page_size, dtype, seed=seed)
     q_all = torch.cat(qs).to(dev())
     positions = torch.tensor(pos, dtype=torch.int32, device=dev())
-    if mfma:
+    if mfma_decode:
+        out = ops().paged_attention_decode_mfma(q_all, cache.to(dev()), table.to(dev()), positions,
+                                                *items_for(new, max(1, 16 // G)),
+                                                1.0 / math.sqrt(d), window, keys_per_split, nsplit)
+    elif mfma:
         out = ops().paged_attention_mfma(q_all, cache.to(dev()), table.to(dev()), positions,
                                          *items_for(new, max(1, 64 // G)), 1.0 / math.sqrt(d),
                                          window)
@@ -369,6 +373,21 @@ def test_paged_attention_matrix_cores(nh, nkv, d, page_size, window):
                                 sharpen=True, mfma=True)
     assert rel_err(out, expect) < BF16_TOL
     assert float(expect.abs().max()) > 0.5
+
+
+@pytest.mark.parametrize("nh,nkv,d,page_size", [
+    (32, 8, 64, 16), (4, 4, 64, 4), (8, 4, 128, 16), (16, 1, 64, 8), (2, 1, 128, 32)])
+@pytest.mark.parametrize("keys,nsplit", [(0, 1), (64, 12), (256, 3)])
+@pytest.mark.parametrize("window", [0, 70])
+def test_paged_attention_decode_matrix_cores(nh, nkv, d, page_size, keys, nsplit, window):
+    """The decode kernel: single tokens (and pairs) with contexts from nothing to
+    several hundred keys, whole and cut."""
+    ctx = [700, 0, 255, 64, 1, 300]
+    new = [1, 1, 1, 1, 2, 3]
+    out, expect = run_attention(torch.bfloat16, nh, nkv, d, page_size, ctx, new, window=window,
+                                keys_per_split=keys, nsplit=nsplit, sharpen=True,
+                                mfma_decode=True)
+    assert rel_err(out, expect) < BF16_TOL
 
 
 def test_single_token_attention_returns_value():

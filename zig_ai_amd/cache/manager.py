@@ -57,6 +57,7 @@ class RequestCache:
     num_tokens: int = 0
     tables: Dict[int, List[int]] = field(default_factory=dict)   # group index -> page ids
     reserved: int = 0                                            # tokens the tables cover
+    serial: int = 0                                              # number of this admission
 
 
 @dataclass
@@ -125,6 +126,7 @@ class CacheManager:
                                                dtype=torch.float32, device=device)
         self.requests: Dict[Hashable, RequestCache] = {}
         self.pages_reused = 0
+        self._admissions = 0
         self._ever_used: List[set] = [set() for _ in self.groups]
 
     # ------------------------------------------------------------------ views
@@ -151,7 +153,9 @@ class CacheManager:
         if req in self.requests:
             raise PoolError(f"request {req!r} is already admitted")
         slot = self.slots.take(req)
-        self.requests[req] = RequestCache(slot, 0, {g.index: [] for g in self.groups}, 0)
+        self._admissions += 1
+        self.requests[req] = RequestCache(slot, 0, {g.index: [] for g in self.groups}, 0,
+                                          self._admissions)
         if self.slot_memory is not None:
             self.slot_memory[slot].zero_()
         return slot
@@ -224,6 +228,10 @@ class CacheManager:
 
     def num_tokens(self, req: Hashable) -> int:
         return self.requests[req].num_tokens
+
+    def serial_of(self, req: Hashable) -> int:
+        """A number that differs between two admissions, also of the same id."""
+        return self.requests[req].serial
 
     def table(self, req: Hashable, group: int) -> List[int]:
         return self.requests[req].tables[group]

@@ -410,6 +410,230 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
   }
 }
 
+// Decoding on the matrix cores: work items of at most 16 rows (one or a few
+// tokens times the query heads of the group), which become the 16 columns of the
+// second operand.  The four waves of a workgroup take the key tiles of the
+// workgroup's key range in turn and never wait for each other inside the loop:
+// keys go from global memory straight into first-operand registers (a lane needs
+// 8 consecutive head-dim elements of one key), values are turned through a
+// wave-private LDS tile into the key-major order the second product needs.  At the
+// end the four partial (m, l, O) are merged in LDS; with `nsplit` > 1 the merged
+// partial goes to `attention_combine_kernel` like those of the plain kernel.
+template <int D>
+__global__ void __launch_bounds__(256)
+paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
+                                   const bf16_t* __restrict__ kv,
+                                   const int* __restrict__ block_table, int bt_stride,
+                                   const int* __restrict__ positions,
+                                   const int* __restrict__ wi_seq, const int* __restrict__ wi_row0,
+                                   const int* __restrict__ wi_count, float* __restrict__ part_acc,
+                                   float* __restrict__ part_ml, int nh, int nkv, int page_size,
+                                   float scale, int window, int keys_per_split, int nsplit) {
+  constexpr int LDV = AM_KT + 8;
+  constexpr int KSTEPS = D / 32;
+  constexpr int DBLK = D / 16;
+  constexpr int VEC_PER_ROW = D / 8;
+  __shared__ __attribute__((aligned(16))) bf16_t Vt_all[4 * D * LDV];   // [wave][dim][key slot]
+  __shared__ float mg_m[4][16], mg_l[4][16];
+  __shared__ float mg_o[4][DBLK][64][4];
+
+  const int item = blockIdx.x, gkv = blockIdx.y, z = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r16 = lane & 15, grp = lane >> 4;
+  const int G = nh / nkv;
+  const int seq = wi_seq[item];
+  const int row0 = wi_row0[item];
+  int count = wi_count[item];
+  if (count * G > 16) count = 16 / G;   // the host never asks for more
+  const int rows = count * G;
+  const int* table = block_table + (size_t)seq * bt_stride;
+  bf16_t* Vt = Vt_all + wave * D * LDV;
+
+  const bool row_valid = r16 < rows;
+  const int tok = row0 + (row_valid ? r16 / G : 0);
+  const int head = gkv * G + (row_valid ? r16 % G : 0);
+  const int pos_row = row_valid ? positions[tok] : -1;
+  const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  bf16x8_t qf[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks)
+    qf[ks] = row_valid ? *reinterpret_cast<const bf16x8_t*>(
+                             q + ((size_t)tok * nh + head) * D + ks * 32 + grp * 8)
+                       : zero8;
+
+  const int pos_first = positions[row0];
+  const int pos_last = positions[row0 + count - 1];
+  const int lo = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
+  const int hi = pos_last;
+  int range_lo = z * keys_per_split;
+  int range_hi = range_lo + keys_per_split - 1;
+  if (nsplit == 1) { range_lo = 0; range_hi = hi; }
+  if (range_hi > hi) range_hi = hi;
+  int tile_first = (lo / AM_KT) * AM_KT;
+  if (tile_first < range_lo) tile_first = range_lo;
+
+  f32x4_t o[DBLK];
+#pragma unroll
+  for (int db = 0; db < DBLK; ++db) o[db] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const size_t vofs = (size_t)nkv * page_size * D;
+
+  // One tile's keys (first-operand fragments) and values (rows along the head
+  // dimension, lane = key) in registers; the next tile is fetched while this one is
+  // being computed.
+  bf16x8_t kf[4][KSTEPS], vx[VEC_PER_ROW];
+  auto fetch = [&](int tile0, bf16x8_t (&kfr)[4][KSTEPS], bf16x8_t (&vxr)[VEC_PER_ROW]) {
+#pragma unroll
+    for (int jb = 0; jb < 4; ++jb) {
+      const int kp = tile0 + jb * 16 + r16;
+      const bf16_t* krow = nullptr;
+      if (kp >= lo && kp <= range_hi) {
+        const int page = table[kp / page_size];
+        if (page >= 0)
+          krow = kv + ((((size_t)page * 2) * nkv + gkv) * page_size + kp % page_size) * D;
+      }
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks)
+        kfr[jb][ks] = krow ? *reinterpret_cast<const bf16x8_t*>(krow + ks * 32 + grp * 8) : zero8;
+    }
+    const int kp = tile0 + lane;
+    const bf16_t* vrow = nullptr;
+    if (kp >= lo && kp <= range_hi) {
+      const int page = table[kp / page_size];
+      if (page >= 0)
+        vrow = kv + ((((size_t)page * 2) * nkv + gkv) * page_size + kp % page_size) * D + vofs;
+    }
+#pragma unroll
+    for (int v = 0; v < VEC_PER_ROW; ++v)
+      vxr[v] = vrow ? *reinterpret_cast<const bf16x8_t*>(vrow + v * 8) : zero8;
+  };
+
+  int tile0 = tile_first + wave * AM_KT;
+  if (tile0 <= range_hi) fetch(tile0, kf, vx);
+  for (; tile0 <= range_hi; tile0 += 4 * AM_KT) {
+    bf16x8_t kfn[4][KSTEPS], vxn[VEC_PER_ROW];
+    const int next = tile0 + 4 * AM_KT;
+    if (next <= range_hi) fetch(next, kfn, vxn);
+
+    f32x4_t s[4];
+#pragma unroll
+    for (int jb = 0; jb < 4; ++jb) {
+      s[jb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks)
+        s[jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[jb][ks], qf[ks], s[jb], 0, 0, 0);
+    }
+    // values into this wave's LDS tile, key-major (lane = key j of the tile)
+    {
+      const int j = lane;
+      const int slot = (j & 32) + ((j & 15) >> 2) * 8 + ((j >> 4) & 1) * 4 + (j & 3);
+#pragma unroll
+      for (int v = 0; v < VEC_PER_ROW; ++v)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) Vt[(v * 8 + e) * LDV + slot] = vx[v][e];
+    }
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int jb = 0; jb < 4; ++jb)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int kp = tile0 + jb * 16 + grp * 4 + i;
+        bool valid = kp <= pos_row && kp >= lo && kp <= range_hi;
+        if (window > 0 && kp <= pos_row - window) valid = false;
+        const float v = valid ? s[jb][i] * scale : -INFINITY;
+        s[jb][i] = v;
+        tmax = fmaxf(tmax, v);
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m, tmax);
+    const float m_use = m_new > -INFINITY ? m_new : 0.f;
+    const float alpha = expf(m - m_use);
+    float psum = 0.f;
+#pragma unroll
+    for (int jb = 0; jb < 4; ++jb)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = expf(s[jb][i] - m_use);
+        s[jb][i] = p;
+        psum += p;
+      }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * alpha + psum;
+    m = m_new;
+#pragma unroll
+    for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[db][i] *= alpha;
+    bf16x8_t pf[2];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        pf[kk][i] = (bf16_t)s[2 * kk][i];
+        pf[kk][4 + i] = (bf16_t)s[2 * kk + 1][i];
+      }
+    __builtin_amdgcn_wave_barrier();   // this wave's stores to Vt precede its loads below
+#pragma unroll
+    for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        const bf16x8_t vf = *reinterpret_cast<const bf16x8_t*>(
+            Vt + (db * 16 + r16) * LDV + kk * 32 + grp * 8);
+        o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[kk], o[db], 0, 0, 0);
+      }
+    __builtin_amdgcn_wave_barrier();   // and those loads precede the next tile's stores
+    if (next <= range_hi) {
+#pragma unroll
+      for (int jb = 0; jb < 4; ++jb)
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) kf[jb][ks] = kfn[jb][ks];
+#pragma unroll
+      for (int v = 0; v < VEC_PER_ROW; ++v) vx[v] = vxn[v];
+    }
+  }
+
+  // merge the four waves' partial results
+  if (grp == 0) { mg_m[wave][r16] = m; mg_l[wave][r16] = l; }
+#pragma unroll
+  for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) mg_o[wave][db][lane][i] = o[db][i];
+  __syncthreads();
+  if (wave == 0 && row_valid) {
+    float mx = mg_m[0][r16];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) mx = fmaxf(mx, mg_m[w][r16]);
+    const float mu = mx > -INFINITY ? mx : 0.f;
+    float wgt[4], total = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      wgt[w] = expf(mg_m[w][r16] - mu);
+      total += mg_l[w][r16] * wgt[w];
+    }
+    const size_t orow = (size_t)tok * nh + head;
+#pragma unroll
+    for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float acc = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) acc = fmaf(mg_o[w][db][lane][i], wgt[w], acc);
+        const int dim = db * 16 + grp * 4 + i;
+        if (nsplit == 1)
+          out[orow * D + dim] = (bf16_t)(total > 0.f ? acc / total : 0.f);
+        else
+          part_acc[(orow * nsplit + z) * D + dim] = acc;
+      }
+    if (nsplit > 1 && grp == 0) {
+      part_ml[(orow * nsplit + z) * 2] = mx;
+      part_ml[(orow * nsplit + z) * 2 + 1] = total;
+    }
+  }
+}
+
 template <typename T, int KT>
 static int launch_attention(const void* q, void* out, const void* kv, const int* block_table,
                             int bt_stride, const int* positions, const int* wi_seq,
@@ -496,5 +720,47 @@ extern "C" int za_paged_attention_mfma(const void* q, void* out, const void* kv,
     hipLaunchKernelGGL((paged_attention_mfma_kernel<128>), grid, block, 0, stream,
                        (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
                        positions, wi_seq, wi_row0, wi_count, nh, nkv, page_size, scale, window);
+  return za_launch_status();
+}
+
+// Matrix-core decode variant: bfloat16, head_dim 64 or 128, work items of at most
+// 16 / (nh / nkv) query rows (nh / nkv dividing 16), contexts optionally cut as in
+// za_paged_attention (the partial results are merged by the same combine kernel).
+extern "C" int za_paged_attention_decode_mfma(const void* q, void* out, const void* kv,
+                                              const int* block_table, int bt_stride,
+                                              const int* positions, const int* wi_seq,
+                                              const int* wi_row0, const int* wi_count,
+                                              int n_items, int n_tokens, float* part_acc,
+                                              float* part_ml, int nh, int nkv, int d,
+                                              int page_size, float scale, int window,
+                                              int keys_per_split, int nsplit,
+                                              hipStream_t stream) {
+  if (n_items == 0 || n_tokens == 0) return 0;
+  if (n_items < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || page_size <= 0 || bt_stride <= 0 ||
+      nsplit < 1 || !q || !out || !kv || !block_table || !positions || !wi_seq || !wi_row0 ||
+      !wi_count)
+    return ZA_ERR_ARG;
+  const int G = nh / nkv;
+  if ((d != 64 && d != 128) || G > 16 || 16 % G != 0 || nkv > 65535 || nsplit > 65535)
+    return ZA_ERR_UNSUPPORTED;
+  if (nsplit > 1 && (!part_acc || !part_ml || keys_per_split <= 0 || keys_per_split % 64 != 0))
+    return ZA_ERR_ARG;
+  dim3 grid(n_items, nkv, nsplit), block(256);
+  if (d == 64) {
+    hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<64>), grid, block, 0, stream,
+                       (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
+                       positions, wi_seq, wi_row0, wi_count, part_acc, part_ml, nh, nkv,
+                       page_size, scale, window, keys_per_split, nsplit);
+  } else {
+    hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<128>), grid, block, 0, stream,
+                       (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
+                       positions, wi_seq, wi_row0, wi_count, part_acc, part_ml, nh, nkv,
+                       page_size, scale, window, keys_per_split, nsplit);
+  }
+  int rc = za_launch_status();
+  if (rc != 0 || nsplit == 1) return rc;
+  dim3 cgrid((unsigned)((size_t)n_tokens * nh)), cblock(64);
+  hipLaunchKernelGGL((attention_combine_kernel<bf16_t>), cgrid, cblock, 0, stream, part_acc,
+                     part_ml, (bf16_t*)out, d, nsplit);
   return za_launch_status();
 }

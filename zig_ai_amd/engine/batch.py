@@ -50,6 +50,10 @@ class StepContext:
     seq_lens_host: List[int] = field(default_factory=list)
     ctx_lens_host: List[int] = field(default_factory=list)
     slots_host: List[int] = field(default_factory=list)
+    # the host image of the integer buffer and where each array sits in it
+    host: Optional[np.ndarray] = None
+    offsets: Dict[str, Tuple[int, int]] = field(default_factory=dict)
+    table_width: int = 0
 
     def attention_items(self, rows_per_item: int):
         """Work items of at most ``rows_per_item`` consecutive query rows of one
@@ -193,7 +197,8 @@ def build_step(entries: Sequence[StepEntry], cache: CacheManager, device: torch.
         token_ids=view("token_ids"), positions=view("positions"), token_seq=view("token_seq"),
         seq_start=view("seq_start"), ctx_len=view("ctx_len"), slot_id=view("slot_id"),
         logit_rows=view("logit_rows"),
-        seq_lens_host=seq_lens, ctx_lens_host=ctx_lens, slots_host=slots)
+        seq_lens_host=seq_lens, ctx_lens_host=ctx_lens, slots_host=slots,
+        host=host, offsets=offsets, table_width=max_pages)
     for g in groups:
         ctx.slot_mapping[g.index] = view(f"slots{g.index}")
         ctx.block_tables[g.index] = view(f"table{g.index}").view(S, max_pages)

@@ -35,7 +35,8 @@ class ModelRunner:
         self.cache = model.make_cache(page_size, num_pages, num_slots)
         self.views = model.cache_views(self.cache)
         self.steps_run = 0
-        self.graphs = DecodeGraphs() if (use_graphs and model.graph_safe) else None
+        self.graphs = (DecodeGraphs(model.spec.vocab_size, model.item_granularities, model.spec.max_position)
+                       if (use_graphs and model.graph_safe) else None)
 
     # ----------------------------------------------------------------- requests
     def admit(self, request: Hashable) -> None:

@@ -40,6 +40,11 @@ _SIGNATURES = {
                                                c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                                c_int, c_int, c_int, c_int, c_float, c_int,
                                                c_void_p],
+    ("attention", "za_paged_attention_decode_mfma"): [c_void_p, c_void_p, c_void_p, c_void_p,
+                                                      c_int, c_void_p, c_void_p, c_void_p,
+                                                      c_void_p, c_int, c_int, c_void_p, c_void_p,
+                                                      c_int, c_int, c_int, c_int, c_float, c_int,
+                                                      c_int, c_int, c_void_p],
     ("shortconv", "za_short_conv"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_longlong,
                                      c_void_p],
@@ -385,6 +390,54 @@ def paged_attention_mfma(q: torch.Tensor, kv_cache: torch.Tensor, block_table: t
         _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, nh, nkv, d,
         page_size, float(scale), int(window), _stream())
     _check(rc, "paged_attention_mfma")
+    return out
+
+
+ATTENTION_MFMA_DECODE_ROWS = 16
+
+
+def paged_attention_decode_mfma(q: torch.Tensor, kv_cache: torch.Tensor,
+                                block_table: torch.Tensor, positions: torch.Tensor,
+                                item_seq: torch.Tensor, item_row0: torch.Tensor,
+                                item_count: torch.Tensor, n_items: int, scale: float,
+                                window: int = 0, keys_per_split: int = 0,
+                                nsplit: int = 1) -> torch.Tensor:
+    """The matrix-core kernel for decoding: work items of at most
+    ``ATTENTION_MFMA_DECODE_ROWS // (heads // kv_heads)`` query rows, long contexts
+    optionally cut into ``nsplit`` ranges of ``keys_per_split`` keys."""
+    if q.dim() != 3:
+        raise KernelError(f"q must be [T, heads, head_dim], got {tuple(q.shape)}")
+    T, nh, d = q.shape
+    _need(q, "q", torch.bfloat16)
+    _need(kv_cache, "kv_cache", torch.bfloat16)
+    if kv_cache.dim() != 5 or kv_cache.shape[1] != 2 or kv_cache.shape[4] != d:
+        raise KernelError(f"kv_cache has shape {tuple(kv_cache.shape)}, expected "
+                          f"[pages, 2, kv_heads, page_size, {d}]")
+    nkv, page_size = kv_cache.shape[2], kv_cache.shape[3]
+    if nh % nkv or not attention_mfma_supported(q.dtype, nh, nkv, d):
+        raise KernelError(f"the matrix-core attention kernel does not take {nh} heads, {nkv} "
+                          f"key/value heads, head_dim {d}")
+    _need(block_table, "block_table", torch.int32)
+    if block_table.dim() != 2:
+        raise KernelError("block_table must be [requests, max_pages]")
+    _need(positions, "positions", torch.int32, (T,))
+    for name, t in (("item_seq", item_seq), ("item_row0", item_row0), ("item_count", item_count)):
+        _need(t, name, torch.int32)
+        if t.numel() < n_items:
+            raise KernelError(f"{name} holds {t.numel()} entries, fewer than {n_items} items")
+    out = torch.empty_like(q)
+    part_acc = part_ml = None
+    if nsplit > 1:
+        if keys_per_split <= 0 or keys_per_split % 64:
+            raise KernelError("keys_per_split must be a positive multiple of 64")
+        part_acc = torch.empty((T, nh, nsplit, d), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((T, nh, nsplit, 2), dtype=torch.float32, device=q.device)
+    rc = _fn("attention", "za_paged_attention_decode_mfma")(
+        _ptr(q), _ptr(out), _ptr(kv_cache), _ptr(block_table), block_table.shape[1],
+        _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
+        _ptr(part_acc), _ptr(part_ml), nh, nkv, d, page_size, float(scale), int(window),
+        int(keys_per_split), int(nsplit), _stream())
+    _check(rc, "paged_attention_decode_mfma")
     return out
 
 

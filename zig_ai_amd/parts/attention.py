@@ -90,8 +90,9 @@ class GroupedQueryAttention(Mixer):
         self.mfma = ops.attention_mfma_supported(runtime.dtype, self.num_heads,
                                                  self.num_kv_heads, self.head_dim)
         self.mfma_rows_per_item = max(1, ops.ATTENTION_MFMA_ROWS // self.group)
+        self.mfma_decode_rows_per_item = max(1, ops.ATTENTION_MFMA_DECODE_ROWS // self.group)
         self.item_granularities = [self.rows_per_item] + (
-            [self.mfma_rows_per_item] if self.mfma else [])
+            [self.mfma_rows_per_item, self.mfma_decode_rows_per_item] if self.mfma else [])
         self.window = int(params.get("window") or 0)
         scale = params.get("softmax_scale")
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
@@ -145,6 +146,14 @@ class GroupedQueryAttention(Mixer):
                                          step.positions,
                                          *step.attention_items(self.mfma_rows_per_item),
                                          self.scale, self.window)
+        elif self.mfma:
+            # single tokens only: the matrix-core kernel whose waves split the keys
+            item_seq, item_row0, item_count, n_items = step.attention_items(
+                self.mfma_decode_rows_per_item)
+            keys, nsplit = plan_split(n_items, nkv, step.max_keys)
+            o = ops.paged_attention_decode_mfma(q, cache.kv, step.block_tables[cache.group],
+                                                step.positions, item_seq, item_row0, item_count,
+                                                n_items, self.scale, self.window, keys, nsplit)
         else:
             item_seq, item_row0, item_count, n_items = step.attention_items(self.rows_per_item)
             keys, nsplit = plan_split(n_items, nkv, step.max_keys)
