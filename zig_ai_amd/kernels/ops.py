@@ -53,7 +53,7 @@ _SIGNATURES = {
     ("sampling", "za_argmax"): [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int,
                                 c_void_p],
     ("gemm", "za_gemm_bf16_rows16"): [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                                      c_int, c_int, c_void_p],
+                                      c_int, c_int, c_int, c_void_p],
     ("sampling", "za_sample"): [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                 c_void_p, c_void_p],
     ("sampling", "za_repetition_penalty"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
@@ -226,7 +226,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
         if splits > 1:
             stack = torch.empty((splits, M, N), dtype=torch.float32, device=x.device)
             rc = _fn("gemm", "za_gemm_bf16_rows16")(_ptr(x), _ptr(weight), _ptr(bias), _ptr(stack),
-                                                    0, M, N, K, splits, _stream())
+                                                    0, M, N, K, splits, 0, _stream())
             _check(rc, "gemm_bf16_rows16", f"M={M} N={N} K={K} splits={splits}")
             return stack
         if M > LIBRARY_GEMM_ROWS and bias is None and out_dtype == torch.bfloat16 \
