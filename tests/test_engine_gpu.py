@@ -15,7 +15,7 @@ import torch
 
 import engine_util as eu
 import plain_lfm2 as plain
-from tiny_configs import TINY_A, TINY_B, TINY_C, TINY_D
+from tiny_configs import REAL_2L, TINY_A, TINY_B, TINY_C, TINY_D
 
 pytestmark = pytest.mark.gpu
 
@@ -230,3 +230,26 @@ def test_step_errors():
     with pytest.raises(OutOfPages):
         runner.step([StepEntry("a", list(range(17)), [0])])
     runner.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_real_layer_sizes(dtype):
+    """Two layers (ShortConv, attention) at the sizes of the LFM2-1.2B shape, vocabulary
+    65,536: whole, in portions with single tokens, and batched with another request."""
+    from zig_ai_amd.engine import DecoderModel, ModelRunner, StepEntry
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    folder = eu.model_folder(REAL_2L, 7, store, std=0.02, norm_init="around_one",
+                             role_std={"norm": 0.2, "filter": 0.5, "q_proj.weight": 0.05,
+                                       "k_proj.weight": 0.05})
+    model = DecoderModel.from_folder(folder, dtype)
+    oracle = plain.PlainLfm2(folder)
+    prompts = [eu.random_tokens(n, 65536, 900 + n) for n in (40, 21)]
+    expect = [oracle.logits(p) for p in prompts]
+    runner = ModelRunner(model, page_size=16, num_pages=16, num_slots=2)
+    got = eu.run_schedule(runner, prompts, eu.whole([40, 21]))
+    check(got, expect, dtype, "whole")
+    schedule = [([(0, 0, 20)], []), ([(0, 20, 21), (1, 0, 17)], []), ([(0, 21, 22), (1, 17, 18)], []),
+                ([(0, 22, 38), (1, 18, 19)], []), ([(0, 38, 39), (1, 19, 20)], []),
+                ([(0, 39, 40), (1, 20, 21)], [0, 1])]
+    got = eu.run_schedule(runner, prompts, schedule)
+    check(got, expect, dtype, "portions beside single tokens")

@@ -43,3 +43,14 @@ TINY_D = {
     "rope_theta": 1000000.0, "norm_eps": 1e-5, "conv_L_cache": 3, "conv_bias": False,
     "tie_embedding": True, "max_position_embeddings": 4096,
 }
+
+# two layers at the sizes of the LFM2-1.2B shape: the kernels' large-size paths
+REAL_2L = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 2048, "num_hidden_layers": 2, "num_attention_heads": 32,
+    "num_key_value_heads": 8, "vocab_size": 65536, "layer_types": ["conv", "full_attention"],
+    "block_ff_dim": 12288, "block_auto_adjust_ff_dim": True, "block_multiple_of": 256,
+    "block_ffn_dim_multiplier": 1.0, "rope_theta": 1000000.0, "norm_eps": 1e-5,
+    "conv_L_cache": 3, "conv_bias": False, "tie_embedding": True,
+    "max_position_embeddings": 128000,
+}

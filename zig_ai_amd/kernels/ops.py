@@ -172,8 +172,9 @@ def embed_gather(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
 
 
 # --------------------------------------------------------------------- gemm
-# Above this many rows a bfloat16 projection without bias goes to the library.
-LIBRARY_GEMM_ROWS = 64
+# Above this many rows a bfloat16 projection without bias goes to the library
+# (measured: the decode kernel wins up to 16 rows, the library from there on).
+LIBRARY_GEMM_ROWS = 16
 
 
 def _k_splits(M: int, N: int, K: int) -> int:
@@ -194,8 +195,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     """``x [M, K] @ weight[N, K]^T + bias`` with 32-bit accumulation.
 
     bfloat16 weights use the matrix-core kernels of csrc/gemm.hip up to
-    ``LIBRARY_GEMM_ROWS`` rows, and always when a bias or 32-bit output is asked
-    for; larger plain products go to the GEMM library.  32-bit weights use the
+    ``LIBRARY_GEMM_ROWS`` rows (a decode batch), and always when a bias or 32-bit
+    output is asked for; larger plain products go to the GEMM library.  32-bit weights use the
     all-32-bit kernel (``x`` may be either type and is widened): no library, no
     reduced-precision matrix mode.
 
