@@ -199,6 +199,17 @@ def test_gemm_bf16_partial_sums(M, N, K):
     assert big.dim() == 2                                   # only decode batches are split
 
 
+@pytest.mark.parametrize("M,I,K", [(1, 48, 64), (8, 8192, 2048), (16, 100, 520), (5, 176, 96),
+                                   (3, 40, 8192), (8, 33000, 64)])
+def test_linear_swiglu(M, I, K):
+    """The gate applied to the projection's accumulators equals projection, then gate."""
+    x, w = rand((M, K), torch.bfloat16, 34), rand((2 * I, K), torch.bfloat16, 35, 0.1)
+    out = ops().linear_swiglu(x.to(dev()), w.to(dev()))
+    gu = x.double() @ w.double().T
+    assert out.shape == (M, I) and out.dtype == torch.bfloat16
+    assert rel_err(out, torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]) < BF16_TOL
+
+
 def test_gemm_bf16_refuses_odd_k():
     from zig_ai_amd.kernels import KernelError
     x, w = rand((4, 12), torch.bfloat16, 20), rand((8, 12), torch.bfloat16, 21)

@@ -338,6 +338,88 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__
   }
 }
 
+// The same kernel for the fused gate|up projection of a SwiGLU feed-forward,
+// W = [gate rows (I); up rows (I)]: a workgroup computes a row group of the gate
+// and the matching row group of the up projection and writes
+//   C[m, n] = silu(gate[m, n]) * up[m, n],   silu(g) = g / (1 + exp(-g)),
+// from the 32-bit accumulators (/root/reference/src/transformer/ffn.zig:24-30), so
+// the [M, 2I] intermediate never goes to memory.  K is not split over workgroups.
+template <int NW, int KSTEPS>
+__global__ void __launch_bounds__(NW * 64)
+gemm_bf16_rows16_swiglu_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
+                               bf16_t* __restrict__ C, int M, int I, int K,
+                               int groups_per_block) {
+  __shared__ float red[2][2][NW][64][4];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int frag_row = lane & 15, frag_k = (lane >> 4) * 8;
+  const int kbase = wave * KSTEPS * 32 + frag_k;
+  const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  constexpr int CHUNK = KSTEPS > 8 ? 8 : KSTEPS;   // fragments of each operand in flight
+
+  bf16x8_t xa[KSTEPS];
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s) {
+    const int k = kbase + s * 32;
+    xa[s] = (frag_row < M && k < K) ? *reinterpret_cast<const bf16x8_t*>(A + (size_t)frag_row * K + k)
+                                    : zero8;
+  }
+
+  for (int g = 0; g < groups_per_block; ++g) {
+    const int n0 = (blockIdx.x * groups_per_block + g) * 16;
+    if (n0 >= I) break;
+    const int wrow = n0 + frag_row;
+    const bool wvalid = wrow < I;
+    const bf16_t* gp = W + (size_t)(wvalid ? wrow : 0) * K + kbase;
+    const bf16_t* up = gp + (size_t)I * K;
+    f32x4_t ag = {0.f, 0.f, 0.f, 0.f}, au = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int h = 0; h < KSTEPS; h += CHUNK) {
+      bf16x8_t fg[CHUNK], fu[CHUNK];
+#pragma unroll
+      for (int s = 0; s < CHUNK; ++s) {
+        const bool ok = wvalid && kbase + (h + s) * 32 < K;
+        fg[s] = ok ? *reinterpret_cast<const bf16x8_t*>(gp + (h + s) * 32) : zero8;
+        fu[s] = ok ? *reinterpret_cast<const bf16x8_t*>(up + (h + s) * 32) : zero8;
+      }
+#pragma unroll
+      for (int s = 0; s < CHUNK; ++s) {
+        ag = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fg[s], xa[h + s], ag, 0, 0, 0);
+        au = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fu[s], xa[h + s], au, 0, 0, 0);
+      }
+    }
+    if (NW > 1) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        red[g & 1][0][wave][lane][r] = ag[r];
+        red[g & 1][1][wave][lane][r] = au[r];
+      }
+      __syncthreads();
+    }
+    if (wave == 0) {
+      const int m = lane & 15, nn = n0 + (lane >> 4) * 4;
+      if (m < M) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int n = nn + r;
+          if (n >= I) continue;
+          float gv = ag[r], uv = au[r];
+          if (NW > 1) {
+            gv = red[g & 1][0][0][lane][r];
+            uv = red[g & 1][1][0][lane][r];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) {
+              gv += red[g & 1][0][w][lane][r];
+              uv += red[g & 1][1][w][lane][r];
+            }
+          }
+          C[(size_t)m * I + n] = (bf16_t)(gv * (1.0f / (1.0f + expf(-gv))) * uv);
+        }
+      }
+    }
+  }
+}
+
 static int launch_rows16(const bf16_t* a, const bf16_t* w, const float* bias, void* C, int c_dtype,
                          int M, int N, int K, int ksplit, hipStream_t stream,
                          int groups_per_block = 0) {
@@ -444,4 +526,29 @@ extern "C" int za_gemm_bf16_rows16(const void* A, const void* W, const float* bi
   if (M > 16 || K % 8 != 0 || (c_dtype != 0 && c_dtype != 1)) return ZA_ERR_UNSUPPORTED;
   return launch_rows16((const bf16_t*)A, (const bf16_t*)W, bias, C, c_dtype, M, N, K, ksplit,
                        stream, groups_per_block);
+}
+
+// Fused gate|up projection with the SwiGLU gate applied to the accumulators:
+// W is [2 * I, K] (gate rows, then up rows), C is bfloat16 [M, I], M <= 16, K <= 8192.
+extern "C" int za_gemm_bf16_rows16_swiglu(const void* A, const void* W, void* C, int M, int I,
+                                          int K, hipStream_t stream) {
+  if (M == 0 || I == 0) return 0;
+  if (M < 0 || I < 0 || K <= 0 || !A || !W || !C) return ZA_ERR_ARG;
+  if (M > 16 || K % 8 != 0 || K > 8192) return ZA_ERR_UNSUPPORTED;
+  const int groups = (I + 15) / 16;
+  const int per_block = groups >= 2048 ? 4 : 1;
+  dim3 grid((groups + per_block - 1) / per_block);
+#define ZA_SG_CASE(NW, KS)                                                                    \
+  {                                                                                           \
+    hipLaunchKernelGGL((gemm_bf16_rows16_swiglu_kernel<NW, KS>), grid, dim3(NW * 64), 0,      \
+                       stream, (const bf16_t*)A, (const bf16_t*)W, (bf16_t*)C, M, I, K,       \
+                       per_block);                                                            \
+    return za_launch_status();                                                                \
+  }
+  if (K <= 512) ZA_SG_CASE(1, 16)
+  if (K <= 1024) ZA_SG_CASE(2, 16)
+  if (K <= 2048) ZA_SG_CASE(4, 16)
+  if (K <= 4096) ZA_SG_CASE(8, 16)
+  ZA_SG_CASE(8, 32)
+#undef ZA_SG_CASE
 }

@@ -54,6 +54,8 @@ _SIGNATURES = {
                                 c_void_p],
     ("gemm", "za_gemm_bf16_rows16"): [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                       c_int, c_int, c_int, c_void_p],
+    ("gemm", "za_gemm_bf16_rows16_swiglu"): [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                             c_void_p],
     ("sampling", "za_sample"): [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                 c_void_p, c_void_p],
     ("sampling", "za_repetition_penalty"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
@@ -240,6 +242,28 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
                                          _code(out_dtype), M, N, K, 1 if force_tiled else 0,
                                          _stream())
         _check(rc, "gemm_bf16", f"M={M} N={N} K={K}")
+    return out
+
+
+def linear_swiglu(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor:
+    """``silu(x Wg^T) * (x Wu^T)`` for ``gate_up_weight = [Wg; Wu]`` of shape ``[2I, K]``
+    and at most 16 rows of bfloat16 ``x``: the gate is applied to the 32-bit
+    accumulators, the ``[M, 2I]`` intermediate is never stored."""
+    if x.dim() != 2 or gate_up_weight.dim() != 2 or gate_up_weight.shape[0] % 2 \
+            or gate_up_weight.shape[1] != x.shape[1]:
+        raise KernelError(f"linear_swiglu takes x [M, K] and a weight [2I, K], got "
+                          f"{tuple(x.shape)} and {tuple(gate_up_weight.shape)}")
+    M, K = x.shape
+    I = gate_up_weight.shape[0] // 2
+    _need(x, "x", torch.bfloat16)
+    _need(gate_up_weight, "gate_up_weight", torch.bfloat16)
+    if M > 16 or K % 8 or K > 8192:
+        raise KernelError(f"linear_swiglu takes at most 16 rows and K <= 8192 in multiples of "
+                          f"8, got M={M} K={K}")
+    out = torch.empty((M, I), dtype=torch.bfloat16, device=x.device)
+    rc = _fn("gemm", "za_gemm_bf16_rows16_swiglu")(_ptr(x), _ptr(gate_up_weight), _ptr(out), M, I,
+                                                   K, _stream())
+    _check(rc, "linear_swiglu", f"M={M} I={I} K={K}")
     return out
 
 

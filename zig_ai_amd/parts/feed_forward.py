@@ -38,8 +38,13 @@ class SwiGLU(FeedForward):
         self.down = tensors["down.weight"]
 
     def forward(self, x: torch.Tensor, step=None) -> torch.Tensor:
-        gu = ops.linear(x, self.gate_up)
-        return ops.linear(ops.swiglu(gu), self.down, partial_ok=True)
+        if x.shape[0] <= 16 and x.dtype == torch.bfloat16 and self.gate_up.dtype == torch.bfloat16 \
+                and x.shape[1] <= 8192:
+            # a decode batch: the gate is applied to the projection's accumulators
+            a = ops.linear_swiglu(x, self.gate_up)
+        else:
+            a = ops.swiglu(ops.linear(x, self.gate_up))
+        return ops.linear(a, self.down, partial_ok=True)
 
 
 register_feed_forward(SwiGLU.kind, SwiGLU)
