@@ -441,9 +441,10 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, grp = lane >> 4;
   const int G = nh / nkv;
-  const int seq = wi_seq[item];
-  const int row0 = wi_row0[item];
-  int count = wi_count[item];
+  // without work-item arrays item i is request i's single token (a pure decode step)
+  const int seq = wi_seq ? wi_seq[item] : item;
+  const int row0 = wi_seq ? wi_row0[item] : item;
+  int count = wi_seq ? wi_count[item] : 1;
   if (count * G > 16) count = 16 / G;   // the host never asks for more
   const int rows = count * G;
   const int* table = block_table + (size_t)seq * bt_stride;
@@ -483,27 +484,33 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
   // dimension, lane = key) in registers; the next tile is fetched while this one is
   // being computed.
   bf16x8_t kf[4][KSTEPS], vx[VEC_PER_ROW];
+  // The block-table entries are read whether or not the key turns out to be in
+  // range (unused entries hold -1), so that these loads do not wait for the
+  // positions the range is computed from.
+  const int last_entry = bt_stride - 1;
   auto fetch = [&](int tile0, bf16x8_t (&kfr)[4][KSTEPS], bf16x8_t (&vxr)[VEC_PER_ROW]) {
+    int kpage[4];
+#pragma unroll
+    for (int jb = 0; jb < 4; ++jb) {
+      const int e = (tile0 + jb * 16 + r16) / page_size;
+      kpage[jb] = table[e < last_entry ? e : last_entry];
+    }
+    const int ve = (tile0 + lane) / page_size;
+    const int vpage = table[ve < last_entry ? ve : last_entry];
 #pragma unroll
     for (int jb = 0; jb < 4; ++jb) {
       const int kp = tile0 + jb * 16 + r16;
       const bf16_t* krow = nullptr;
-      if (kp >= lo && kp <= range_hi) {
-        const int page = table[kp / page_size];
-        if (page >= 0)
-          krow = kv + ((((size_t)page * 2) * nkv + gkv) * page_size + kp % page_size) * D;
-      }
+      if (kp >= lo && kp <= range_hi && kpage[jb] >= 0)
+        krow = kv + ((((size_t)kpage[jb] * 2) * nkv + gkv) * page_size + kp % page_size) * D;
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks)
         kfr[jb][ks] = krow ? *reinterpret_cast<const bf16x8_t*>(krow + ks * 32 + grp * 8) : zero8;
     }
     const int kp = tile0 + lane;
     const bf16_t* vrow = nullptr;
-    if (kp >= lo && kp <= range_hi) {
-      const int page = table[kp / page_size];
-      if (page >= 0)
-        vrow = kv + ((((size_t)page * 2) * nkv + gkv) * page_size + kp % page_size) * D + vofs;
-    }
+    if (kp >= lo && kp <= range_hi && vpage >= 0)
+      vrow = kv + ((((size_t)vpage * 2) * nkv + gkv) * page_size + kp % page_size) * D + vofs;
 #pragma unroll
     for (int v = 0; v < VEC_PER_ROW; ++v)
       vxr[v] = vrow ? *reinterpret_cast<const bf16x8_t*>(vrow + v * 8) : zero8;
@@ -737,9 +744,10 @@ extern "C" int za_paged_attention_decode_mfma(const void* q, void* out, const vo
                                               hipStream_t stream) {
   if (n_items == 0 || n_tokens == 0) return 0;
   if (n_items < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || page_size <= 0 || bt_stride <= 0 ||
-      nsplit < 1 || !q || !out || !kv || !block_table || !positions || !wi_seq || !wi_row0 ||
-      !wi_count)
+      nsplit < 1 || !q || !out || !kv || !block_table || !positions)
     return ZA_ERR_ARG;
+  if (wi_seq && (!wi_row0 || !wi_count)) return ZA_ERR_ARG;
+  if (!wi_seq && n_items != n_tokens) return ZA_ERR_ARG;   // identity items: one token each
   const int G = nh / nkv;
   if ((d != 64 && d != 128) || G > 16 || 16 % G != 0 || nkv > 65535 || nsplit > 65535)
     return ZA_ERR_UNSUPPORTED;

@@ -423,13 +423,15 @@ ATTENTION_MFMA_DECODE_ROWS = 16
 
 def paged_attention_decode_mfma(q: torch.Tensor, kv_cache: torch.Tensor,
                                 block_table: torch.Tensor, positions: torch.Tensor,
-                                item_seq: torch.Tensor, item_row0: torch.Tensor,
-                                item_count: torch.Tensor, n_items: int, scale: float,
+                                item_seq: Optional[torch.Tensor],
+                                item_row0: Optional[torch.Tensor],
+                                item_count: Optional[torch.Tensor], n_items: int, scale: float,
                                 window: int = 0, keys_per_split: int = 0,
                                 nsplit: int = 1) -> torch.Tensor:
     """The matrix-core kernel for decoding: work items of at most
     ``ATTENTION_MFMA_DECODE_ROWS // (heads // kv_heads)`` query rows, long contexts
-    optionally cut into ``nsplit`` ranges of ``keys_per_split`` keys."""
+    optionally cut into ``nsplit`` ranges of ``keys_per_split`` keys.  With
+    ``item_seq=None`` row ``i`` of ``q`` is the single token of request ``i``."""
     if q.dim() != 3:
         raise KernelError(f"q must be [T, heads, head_dim], got {tuple(q.shape)}")
     T, nh, d = q.shape
@@ -446,10 +448,15 @@ def paged_attention_decode_mfma(q: torch.Tensor, kv_cache: torch.Tensor,
     if block_table.dim() != 2:
         raise KernelError("block_table must be [requests, max_pages]")
     _need(positions, "positions", torch.int32, (T,))
-    for name, t in (("item_seq", item_seq), ("item_row0", item_row0), ("item_count", item_count)):
-        _need(t, name, torch.int32)
-        if t.numel() < n_items:
-            raise KernelError(f"{name} holds {t.numel()} entries, fewer than {n_items} items")
+    if item_seq is None:
+        if n_items != T or block_table.shape[0] < T:
+            raise KernelError("without work items every request brings exactly one token")
+    else:
+        for name, t in (("item_seq", item_seq), ("item_row0", item_row0),
+                        ("item_count", item_count)):
+            _need(t, name, torch.int32)
+            if t.numel() < n_items:
+                raise KernelError(f"{name} holds {t.numel()} entries, fewer than {n_items} items")
     out = torch.empty_like(q)
     part_acc = part_ml = None
     if nsplit > 1:

@@ -25,23 +25,31 @@ from ..kernels import ops
 from .base import (Mixer, PagedNeed, Runtime, TensorRule, lookup, register_mixer)
 from .feed_forward import fuse_rows
 
-# Contexts shorter than this are never cut; longer ones are cut into ranges of
-# this many keys (doubled while that would make more than SPLIT_MAX ranges).
-SPLIT_KEYS = 256
+# Cutting long contexts pays only when the launch would otherwise leave most of the
+# machine idle (decoding few requests).  Measured on one MI355X with 8 key/value
+# heads: from 512 workgroups on nothing is gained; below, the longest range (of
+# 1024, 512 or 256 keys) that still yields SPLIT_TARGET workgroups is best.
+BUSY_WORKGROUPS = 512
+SPLIT_TARGET = 256
+SPLIT_KEYS_MIN = 256
 SPLIT_MAX = 64
-# Enough workgroups to occupy the machine without cutting contexts.
-BUSY_WORKGROUPS = 1024
 
 
 def plan_split(n_items: int, num_kv_heads: int, max_keys: int):
-    """(keys per range, number of ranges) for one launch.  Cutting pays only when
-    the launch would otherwise leave most of the machine idle (decoding)."""
-    if n_items * num_kv_heads >= BUSY_WORKGROUPS or max_keys <= 2 * SPLIT_KEYS:
+    """(keys per range, number of ranges) for one launch; a function of the batch
+    shape and of the longest context only."""
+    groups = n_items * num_kv_heads
+    if groups >= BUSY_WORKGROUPS or max_keys <= 2 * SPLIT_KEYS_MIN:
         return 0, 1
-    keys = SPLIT_KEYS
+    keys = SPLIT_KEYS_MIN
+    for cand in (1024, 512):
+        if groups * ((max_keys + cand - 1) // cand) >= SPLIT_TARGET:
+            keys = cand
+            break
     while (max_keys + keys - 1) // keys > SPLIT_MAX:
         keys *= 2
-    return keys, (max_keys + keys - 1) // keys
+    nsplit = (max_keys + keys - 1) // keys
+    return (keys, nsplit) if nsplit > 1 else (0, 1)
 
 
 class GroupedQueryAttention(Mixer):
@@ -148,8 +156,9 @@ class GroupedQueryAttention(Mixer):
                                          self.scale, self.window)
         elif self.mfma:
             # single tokens only: the matrix-core kernel whose waves split the keys
-            item_seq, item_row0, item_count, n_items = step.attention_items(
-                self.mfma_decode_rows_per_item)
+            # (every request brings one token: row i is request i, no work-item arrays)
+            item_seq = item_row0 = item_count = None
+            n_items = step.n_seqs
             keys, nsplit = plan_split(n_items, nkv, step.max_keys)
             o = ops.paged_attention_decode_mfma(q, cache.kv, step.block_tables[cache.group],
                                                 step.positions, item_seq, item_row0, item_count,
