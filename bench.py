@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Default run: the layer sizes of the LFM2-1.2B shape (BASELINE.json configs[2])
+Default run: the layer sizes of the LFM2-1.2B shape (16 layers, hidden 2048, vocabulary 65,536)
 with random bfloat16 weights N(0, 0.02), a batch of 8 requests, each prefilled
 with 2,048 synthetic tokens and decoded from there (context 4,096).  A step is
 one decode step of the whole batch through the engine's own step function and

@@ -76,6 +76,18 @@ def test_config_errors(change, match):
         config_from_dict(bad)
 
 
+def test_defaults_of_the_width_keys():
+    only_width = {k: v for k, v in TINY_A.items() if not k.startswith("block_")}
+    only_width["intermediate_size"] = 192
+    assert config_from_dict(only_width).intermediate_size == 192          # taken as it is
+    pre = dict(only_width, block_ff_dim=12288)
+    del pre["intermediate_size"]
+    assert config_from_dict(pre).intermediate_size == 8192                # adjusted, multiple of 256
+    nested = {k: v for k, v in TINY_A.items() if k != "rope_theta"}
+    nested["rope_parameters"] = {"rope_theta": 12345.0, "rope_type": "default"}
+    assert config_from_dict(nested).rope_theta == 12345.0
+
+
 def test_load_config_from_folder(tmp_path):
     (tmp_path / "config.json").write_text(json.dumps(TINY_A))
     assert load_config(str(tmp_path)).hidden_size == 64

@@ -15,7 +15,7 @@ import torch
 
 import engine_util as eu
 import plain_lfm2 as plain
-from tiny_configs import REAL_2L, TINY_A, TINY_B, TINY_C, TINY_D
+from tiny_configs import REAL_2L, TINY_A, TINY_B, TINY_C, TINY_D, TINY_E
 
 pytestmark = pytest.mark.gpu
 
@@ -253,3 +253,20 @@ def test_real_layer_sizes(dtype):
                 ([(0, 39, 40), (1, 20, 21)], [0, 1])]
     got = eu.run_schedule(runner, prompts, schedule)
     check(got, expect, dtype, "portions beside single tokens")
+
+
+def test_widths_that_are_no_multiple_of_eight():
+    """Any width runs in 32-bit; bfloat16 projections need rows that start on 16-byte
+    boundaries and say so when the model is built, before anything runs."""
+    from zig_ai_amd.engine import DecoderModel, ModelRunner
+    from zig_ai_amd.kernels import KernelError
+    folder = eu.model_folder(TINY_E, 4, torch.float32, **eu.sharp_kwargs())
+    model = DecoderModel.from_folder(folder, "float32")
+    oracle = plain.PlainLfm2(folder)
+    prompts = [eu.random_tokens(n, 131, 40 + n) for n in (37, 6)]
+    expect = [oracle.logits(p) for p in prompts]
+    got = eu.run_schedule(ModelRunner(model, 4, 32, 2), prompts, eu.changing_portions([37, 6], 2))
+    check(got, expect, "float32", "odd widths")
+    narrow = eu.model_folder(TINY_E, 4, torch.bfloat16, **eu.sharp_kwargs())
+    with pytest.raises(KernelError, match="multiple of 8"):
+        DecoderModel.from_folder(narrow, "bfloat16")

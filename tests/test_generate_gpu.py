@@ -23,7 +23,7 @@ def folder_for(cfg, seed, dtype=torch.float32):
 
 
 def test_greedy_generation_tiny_a():
-    """BASELINE tiny-A workload: prompts of 5/17/33 tokens, 16 greedy tokens each,
+    """The tiny-A workload: prompts of 5/17/33 tokens, 16 greedy tokens each,
     page size 4, in 32-bit: the same tokens as the plain implementation."""
     from zig_ai_amd.engine import Engine
     folder = folder_for(TINY_A, 0)
@@ -63,7 +63,7 @@ def follow_sampling(oracle, prompt, tokens, params, number):
     dict(temperature=0.0, repetition_penalty=1.5, seed=1),
 ])
 def test_sampled_generation_tiny_b(params):
-    """BASELINE tiny-B workload: prompts of 1/8/31/64/100 tokens, chunked prefill of
+    """The tiny-B workload: prompts of 1/8/31/64/100 tokens, chunked prefill of
     16, temperature 0.7 with a fixed sampling seed, page size 8; and the sampler's
     other options."""
     from zig_ai_amd.engine import Engine

@@ -123,7 +123,7 @@ def test_one_error_lists_everything(tmp_path):
     del tensors["model.layers.2.self_attn.k_proj.weight"]
     del tensors["model.embedding_norm.weight"]
     tensors["model.layers.9.surprise.weight"] = torch.zeros(2)
-    tensors["lm_head.weight"] = torch.zeros(256, 64)                      # tied: not expected
+    tensors["lm_head.weight"] = torch.zeros(256, 64)                      # tied: present, not read
     tensors["model.layers.0.conv.in_proj.weight"] = torch.zeros(100, 64)  # should be [192, 64]
     tensors["model.layers.1.ffn_norm.weight"] = torch.zeros(64, dtype=torch.float64)
     write_safetensors(str(tmp_path / "model.safetensors"), tensors)
@@ -131,11 +131,11 @@ def test_one_error_lists_everything(tmp_path):
         load_tensors(str(tmp_path), spec, torch.bfloat16, "cpu")
     err = e.value
     assert err.missing == ["model.layers.2.self_attn.k_proj.weight", "model.embedding_norm.weight"]
-    assert err.unexpected == ["lm_head.weight", "model.layers.9.surprise.weight"]
+    assert err.unexpected == ["model.layers.9.surprise.weight"]   # a tied head's copy is ignored
     assert len(err.wrong_shape) == 1 and "[100, 64]" in err.wrong_shape[0] and "[192, 64]" in err.wrong_shape[0]
     assert err.wrong_dtype == ["model.layers.1.ffn_norm.weight: F64"]
     text = str(err)
-    for piece in ("missing (2)", "unexpected (2)", "wrong shape (1)", "unsupported dtype (1)"):
+    for piece in ("missing (2)", "unexpected (1)", "wrong shape (1)", "unsupported dtype (1)"):
         assert piece in text
 
 

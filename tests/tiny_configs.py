@@ -54,3 +54,14 @@ REAL_2L = {
     "conv_L_cache": 3, "conv_bias": False, "tie_embedding": True,
     "max_position_embeddings": 128000,
 }
+
+# widths that are multiples of neither 8 nor 16: fine in 32-bit, refused in bfloat16
+TINY_E = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 60, "num_hidden_layers": 2, "num_attention_heads": 3,
+    "num_key_value_heads": 3, "head_dim": 16, "vocab_size": 131,
+    "layer_types": ["conv", "full_attention"],
+    "intermediate_size": 100,
+    "rope_theta": 10000.0, "norm_eps": 1e-5, "conv_L_cache": 5, "conv_bias": False,
+    "tie_embedding": True, "max_position_embeddings": 512,
+}

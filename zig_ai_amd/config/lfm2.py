@@ -42,6 +42,17 @@ def feed_forward_width(block_ff_dim: int, auto_adjust: bool, multiple_of: Option
     return width
 
 
+def _with_nested_rope(data: Mapping[str, Any]) -> Mapping[str, Any]:
+    """Some writers put the rotary base under ``rope_parameters`` / ``rope_scaling``."""
+    if "rope_theta" in data and data["rope_theta"] is not None:
+        return data
+    for key in ("rope_parameters", "rope_scaling"):
+        nested = data.get(key)
+        if isinstance(nested, Mapping) and nested.get("rope_theta") is not None:
+            return {**data, "rope_theta": nested["rope_theta"]}
+    return data
+
+
 @dataclass(frozen=True)
 class Lfm2Config:
     architecture: str
@@ -111,9 +122,12 @@ class Lfm2Config:
                 f"layer_types has {len(kinds)} entries but num_hidden_layers is {n_layers}")
 
         block_ff = read_int(data, ["block_ff_dim", "intermediate_size"], minimum=1)
-        # Absent means on: the key only ever switches the adjustment off.
-        auto = read_bool(data, ["block_auto_adjust_ff_dim"], default=True)
-        multiple_of = read_int(data, ["block_multiple_of", "multiple_of"], default=None, minimum=1)
+        # ``block_ff_dim`` is the width before the adjustment, which is on unless the
+        # key switches it off; a config that gives only ``intermediate_size`` and says
+        # nothing about adjusting means that width itself.
+        auto = read_bool(data, ["block_auto_adjust_ff_dim"], default=has_any(data, ["block_ff_dim"]))
+        multiple_of = read_int(data, ["block_multiple_of", "multiple_of"],
+                               default=256 if auto else None, minimum=1)
         multiplier = read_float(data, ["block_ffn_dim_multiplier"], default=None, positive=True)
         width = feed_forward_width(block_ff, auto, multiple_of, multiplier)
 
@@ -126,7 +140,7 @@ class Lfm2Config:
             head_dim=head_dim, vocab_size=vocab, layer_types=tuple(kinds),
             block_ff_dim=block_ff, auto_adjust_ff_dim=auto, multiple_of=multiple_of,
             ffn_dim_multiplier=multiplier, intermediate_size=width,
-            rope_theta=read_float(data, ["rope_theta"], positive=True),
+            rope_theta=read_float(_with_nested_rope(data), ["rope_theta"], positive=True),
             norm_eps=read_float(data, ["norm_eps", "rms_norm_eps", "block_norm_eps"], positive=True),
             conv_L_cache=read_int(data, ["conv_L_cache"], minimum=1),
             conv_bias=read_bool(data, ["conv_bias"], default=False),
@@ -238,5 +252,7 @@ class Lfm2Config:
                            {} if self.tie_embedding else
                            {"weight": ("lm_head.weight", "output.weight")})
         schedule = tuple(LayerCall(i) for i in range(self.num_layers))
+        # a tied checkpoint may still carry a copy of the head; it is not read
+        ignored = ("lm_head.weight", "output.weight") if self.tie_embedding else ()
         return ModelSpec(self.architecture, H, self.vocab_size, embedding, tuple(layers),
-                         schedule, final_norm, lm_head, self.max_position_embeddings)
+                         schedule, final_norm, lm_head, self.max_position_embeddings, ignored)

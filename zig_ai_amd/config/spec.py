@@ -75,6 +75,7 @@ class ModelSpec:
     final_norm: PartSpec
     lm_head: PartSpec
     max_position: int = 0
+    ignored_tensors: Tuple[str, ...] = ()    # checkpoint names that may be there and are not read
 
     def __post_init__(self) -> None:
         if not self.layers:

@@ -179,6 +179,15 @@ def embed_gather(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
 LIBRARY_GEMM_ROWS = 16
 
 
+def check_projection_weight(weight: torch.Tensor, what: str) -> None:
+    """Refuse, when a part is built, a weight the GEMM kernels cannot take."""
+    if weight.dtype == torch.bfloat16 and weight.shape[1] % 8:
+        raise KernelError(
+            f"{what}: a bfloat16 projection needs an input width that is a multiple of 8 "
+            f"(rows start on 16-byte boundaries), got {weight.shape[1]}; store the weight in "
+            "32-bit or run with float32")
+
+
 def _k_splits(M: int, N: int, K: int) -> int:
     """Into how many ranges the decode kernel cuts K when its consumer accepts
     partial sums: enough to give every compute unit work when N alone is too

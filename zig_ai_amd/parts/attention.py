@@ -120,6 +120,8 @@ class GroupedQueryAttention(Mixer):
         if pos is not None:
             self.position = lookup("position", pos.kind)(pos.params, {}, runtime)
         self.fused_rotation = bool(getattr(self.position, "fused_rotation", False))
+        ops.check_projection_weight(self.w_qkv, "attention w_qkv")
+        ops.check_projection_weight(self.w_out, "attention w_out")
 
     def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
         nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim

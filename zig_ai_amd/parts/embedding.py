@@ -51,6 +51,7 @@ class LinearHead(Part):
         self.weight = tensors.get("weight")   # the model hands a tied head the embedding table
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        ops.check_projection_weight(self.weight, "output head")
         return ops.linear(x, self.weight, out_dtype=torch.float32)
 
 

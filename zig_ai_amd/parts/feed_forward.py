@@ -36,6 +36,8 @@ class SwiGLU(FeedForward):
         super().__init__(params, tensors, runtime)
         self.gate_up = fuse_rows(tensors["gate.weight"], tensors["up.weight"])
         self.down = tensors["down.weight"]
+        ops.check_projection_weight(self.gate_up, "feed_forward gate_up")
+        ops.check_projection_weight(self.down, "feed_forward down")
 
     def forward(self, x: torch.Tensor, step=None) -> torch.Tensor:
         if x.shape[0] <= 16 and x.dtype == torch.bfloat16 and self.gate_up.dtype == torch.bfloat16 \

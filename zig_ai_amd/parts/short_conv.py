@@ -56,6 +56,8 @@ class ShortConv(Mixer):
         self.b_in = tensors.get("in_proj.bias")
         self.b_conv = tensors.get("conv.bias")
         self.b_out = tensors.get("out_proj.bias")
+        ops.check_projection_weight(self.w_in, "short_conv w_in")
+        ops.check_projection_weight(self.w_out, "short_conv w_out")
 
     def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
         z = ops.linear(x, self.w_in, self.b_in)

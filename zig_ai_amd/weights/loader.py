@@ -130,7 +130,8 @@ def load_tensors(model_dir: str, spec: ModelSpec, run_dtype: torch.dtype,
             wrong_dtype.append(f"{found}: {dname}")
             continue
         chosen.append((exp, found))
-    unexpected = sorted(n for n in ckpt.names() if n not in consumed)
+    unexpected = sorted(n for n in ckpt.names()
+                        if n not in consumed and n not in spec.ignored_tensors)
     if missing or unexpected or wrong_shape or wrong_dtype:
         lines = [f"the tensors in {model_dir} do not fit the model:"]
         if missing:
