@@ -246,13 +246,15 @@ def test_qk_norm_rope_kv_write(dtype, nh, nkv, d, rot, pairing):
     assert rel_err(q, qe) < tol
     c = cache.cpu()
     got_k = torch.stack([c[s // page_size, 0, :, s % page_size, :] for s in slots.tolist()])
-    got_v = torch.stack([c[s // page_size, 1, :, s % page_size, :] for s in slots.tolist()])
+    cv = c[:, 1].reshape(pages, nkv, d, page_size)        # values: [kv_head][head_dim][offset]
+    got_v = torch.stack([cv[s // page_size, :, :, s % page_size] for s in slots.tolist()])
     assert rel_err(got_k, ke) < tol
     assert torch.equal(got_v.double(), ve)                 # values are stored as they are
     written = torch.zeros(pages * page_size, dtype=torch.bool)
     written[slots.long()] = True
-    untouched = c.permute(0, 3, 1, 2, 4).reshape(pages * page_size, -1)[~written]
-    assert (untouched == 0).all()                          # and nothing else was touched
+    untouched_k = c[:, 0].permute(0, 2, 1, 3).reshape(pages * page_size, -1)[~written]
+    untouched_v = cv.permute(0, 3, 1, 2).reshape(pages * page_size, -1)[~written]
+    assert (untouched_k == 0).all() and (untouched_v == 0).all()   # nothing else was touched
 
 
 def test_rope_position_zero_is_identity_and_norm_is_kept():
@@ -274,7 +276,8 @@ def test_rope_position_zero_is_identity_and_norm_is_kept():
 
 # ------------------------------------------------------------------ attention
 def paged_from_dense(k, v, page_size, dtype, extra_pages=3, seed=0):
-    """Scatter dense per-request K/V ``[len, nkv, d]`` into a shuffled paged cache.
+    """Scatter dense per-request K/V ``[len, nkv, d]`` into a shuffled paged cache
+    (per page: keys [kv_head][offset][head_dim], then values [kv_head][head_dim][offset]).
     Returns cache, block table [S, max_pages]."""
     nkv, d = k[0].shape[1], k[0].shape[2]
     need = [(x.shape[0] + page_size - 1) // page_size for x in k]
@@ -291,7 +294,8 @@ def paged_from_dense(k, v, page_size, dtype, extra_pages=3, seed=0):
             table[s, p] = page
             lo, hi = p * page_size, min((p + 1) * page_size, ks.shape[0])
             cache[page, 0, :, : hi - lo] = ks[lo:hi].transpose(0, 1).to(dtype)
-            cache[page, 1, :, : hi - lo] = vs[lo:hi].transpose(0, 1).to(dtype)
+            # values are stored turned round: [kv_head][head_dim][offset]
+            cache[page, 1].view(nkv, d, page_size)[:, :, : hi - lo] = vs[lo:hi].permute(1, 2, 0).to(dtype)
     for page in order[nxt:]:
         cache[page] = 1e4
     return cache, table
@@ -330,7 +334,7 @@ def run_attention(dtype, nh, nkv, d, page_size, ctx, new, window=0, keys_per_spl
                                                 1.0 / math.sqrt(d), window, keys_per_split, nsplit)
     elif mfma:
         out = ops().paged_attention_mfma(q_all, cache.to(dev()), table.to(dev()), positions,
-                                         *items_for(new, max(1, 64 // G)), 1.0 / math.sqrt(d),
+                                         *items_for(new, max(1, 128 // G)), 1.0 / math.sqrt(d),
                                          window)
     else:
         out = ops().paged_attention(q_all, cache.to(dev()), table.to(dev()), positions,
@@ -370,7 +374,8 @@ def test_paged_attention_reference_shapes(dtype):
 
 
 @pytest.mark.parametrize("nh,nkv,d,page_size", [
-    (32, 8, 64, 16), (4, 4, 64, 4), (8, 4, 128, 16), (16, 2, 64, 8), (16, 1, 128, 32), (2, 1, 64, 16)])
+    (32, 8, 64, 16), (4, 4, 64, 4), (8, 4, 128, 16), (16, 2, 64, 8), (16, 1, 128, 32), (2, 1, 64, 16),
+    (6, 2, 64, 12), (5, 1, 128, 20), (7, 7, 64, 64)])
 @pytest.mark.parametrize("window", [0, 70])
 def test_paged_attention_matrix_cores(nh, nkv, d, page_size, window):
     """The matrix-core kernel on mixed steps: long portions, portions that do not fill
@@ -386,8 +391,19 @@ def test_paged_attention_matrix_cores(nh, nkv, d, page_size, window):
     assert float(expect.abs().max()) > 0.5
 
 
+def test_paged_attention_matrix_cores_paired_items():
+    """So many work items that a workgroup takes two of them, a late and an early
+    one, with an odd number of items so that the middle one stays alone."""
+    out, expect = run_attention(torch.bfloat16, 64, 64, 64, 16, [0, 90], [1000, 37], mfma=True)
+    assert rel_err(out, expect) < BF16_TOL
+    out, expect = run_attention(torch.bfloat16, 64, 64, 64, 16, [0, 90, 3], [1000, 37, 130],
+                                window=200, mfma=True)
+    assert rel_err(out, expect) < BF16_TOL
+
+
 @pytest.mark.parametrize("nh,nkv,d,page_size", [
-    (32, 8, 64, 16), (4, 4, 64, 4), (8, 4, 128, 16), (16, 1, 64, 8), (2, 1, 128, 32)])
+    (32, 8, 64, 16), (4, 4, 64, 4), (8, 4, 128, 16), (16, 1, 64, 8), (2, 1, 128, 32),
+    (6, 2, 64, 12), (5, 1, 128, 20)])
 @pytest.mark.parametrize("keys,nsplit", [(0, 1), (64, 12), (256, 3)])
 @pytest.mark.parametrize("window", [0, 70])
 def test_paged_attention_decode_matrix_cores(nh, nkv, d, page_size, keys, nsplit, window):

@@ -17,7 +17,9 @@ Life of a request: ``admit`` (takes a slot, zeroes its state), then per step
 tokens are in the cache; pages wholly behind a group's window go back to the
 pool), finally ``release`` (every page and the slot go back).
 
-Device memory: per group ``kv[layer, page, 2, kv_head, offset, head_dim]``;
+Device memory: per group ``kv[layer, page, 2, kv_head, page_size * head_dim]``,
+where a page's keys lie as ``[offset][head_dim]`` and its values turned round as
+``[head_dim][offset]`` (the order the attention kernels' second product reads);
 state ``slots[slot, floats]`` in 32-bit with one view per state entry.
 """
 

@@ -20,7 +20,10 @@
 // merged by `attention_combine_kernel`; the cut points depend on key positions
 // only.
 //
-// Cache layout: kv[page][0 = keys, 1 = values][kv_head][offset][head_dim].
+// Cache layout, per page: keys as [kv_head][offset][head_dim], then values turned
+// round as [kv_head][head_dim][offset].  The second product wants, for one
+// head-dimension element, consecutive keys side by side; stored this way the
+// matrix-core kernels fetch their value operands with plain 8-byte loads.
 #include <math.h>
 
 #include "common.h"
@@ -90,7 +93,7 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
     for (int idx = tid; idx < KT * vec_per_row; idx += 256) {
       const int j = idx / vec_per_row, c = (idx % vec_per_row) * 8;
       const int kp = tile0 + j;
-      float kx[8], vx[8];
+      float kx[8];
       bool ok = kp >= lo && kp <= range_hi;
       int page = -1;
       if (ok) {
@@ -98,19 +101,27 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
         ok = page >= 0;
       }
       if (ok) {
-        const size_t base = ((((size_t)page * 2) * nkv + g) * page_size + kp % page_size) * d + c;
-        const size_t vofs = (size_t)nkv * page_size * d;
-        load8<T>(kv + base, kx);
-        load8<T>(kv + base + vofs, vx);
+        load8<T>(kv + ((((size_t)page * 2) * nkv + g) * page_size + kp % page_size) * d + c, kx);
       } else {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) { kx[i] = 0.f; vx[i] = 0.f; }
+        for (int i = 0; i < 8; ++i) kx[i] = 0.f;
       }
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        Ks[j * ldk + c + i] = kx[i];
-        Vs[j * ldk + c + i] = vx[i];
+      for (int i = 0; i < 8; ++i) Ks[j * ldk + c + i] = kx[i];
+    }
+    {
+      // values: a thread keeps one key of the tile (256 is a multiple of KT) and walks
+      // the head dimension, so the lanes of a wave read consecutive offsets of a page
+      const int j = tid % KT;
+      const int kp = tile0 + j;
+      const T* vsrc = nullptr;
+      if (kp >= lo && kp <= range_hi) {
+        const int page = table[kp / page_size];
+        if (page >= 0)
+          vsrc = kv + (((size_t)page * 2 + 1) * nkv + g) * page_size * d + kp % page_size;
       }
+      for (int dd = tid / KT; dd < d; dd += 256 / KT)
+        Vs[j * ldk + dd] = vsrc ? to_f32<T>(vsrc[(size_t)dd * page_size]) : 0.f;
     }
     __syncthreads();
 
@@ -222,192 +233,331 @@ attention_combine_kernel(const float* __restrict__ part_acc, const float* __rest
 }
 
 // ------------------------------------------------------------ matrix-core path
-// bfloat16, head_dim 64 or 128, query heads per key/value head dividing 16: the
-// same streaming softmax with both products on the matrix cores.
+// bfloat16, head_dim 64 or 128, page sizes that are multiples of 4: the same
+// streaming softmax with both products on the matrix cores.
 //
-// A workgroup serves up to 64 rows (token, head) of one work item and one
-// key/value head; each of its four waves owns 16 rows.  Per tile of 64 keys:
-//   S^T = K Q^T   (keys as the rows of the first operand, the wave's 16 query rows as
-//                  columns; a lane ends up with the scores of ONE query row for 16 keys)
-//   p   = exp(S^T * scale - m)  in 32-bit, running maximum and sum kept per lane
+// A workgroup serves up to 128 rows (token, head) of one work item and one
+// key/value head; each of its eight waves owns 16 rows.  (Waves of 32 rows would read
+// LDS half as often, but need so many registers that a SIMD holds one wave only, and
+// the kernel is bound by vector instructions and their waits, not by LDS: measured,
+// eight light waves are faster.)  Per tile of 64 keys:
+//   S^T = K Q^T   (keys as the rows of the first operand, 16 query rows as columns; a
+//                  lane ends up with the scores of ONE query row for 16 keys)
+//   p   = 2^(S^T * scale * log2(e) - m)  in 32-bit, running maximum and sum per lane
 //   O^T += V^T P^T  (P^T goes from the accumulator registers straight into the second
 //                  operand: the matrix core does not care in which order the 32 keys of
 //                  a step are numbered as long as both operands agree, so V^T is stored
 //                  in LDS with its keys in the order the accumulator yields them)
+// The tiles go through two LDS buffers: while a tile is being computed the next one is
+// on its way from memory into registers, and the page numbers of the one after that
+// are being read.  Every tile issues the same loads, unconditionally.
 // Operand layout of v_mfma_f32_16x16x32_bf16: lane l supplies row (l % 16), k-slots
 // (l / 16) * 8 .. + 7 of either operand and receives rows (l / 16) * 4 .. + 3, column
 // (l % 16) of the product.
 #define AM_KT 64
+#define AM_ROWS 128
 
-template <int D>
-__global__ void __launch_bounds__(256)
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+
+// A query row's scores for a tile are spread over the four lanes l, l ^ 16, l ^ 32,
+// l ^ 48.  The swap instructions exchange 16-lane rows (odd rows of the first operand
+// with even rows of the second) and 32-lane halves between two registers; fed the
+// same value twice they leave in each lane its own value and its partner's, in one
+// vector instruction each and without a trip through LDS.
+__device__ __forceinline__ float quad_max(float x) {
+  const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false,
+                                                  false);
+  const float y = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(y), __float_as_uint(y), false,
+                                                  false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float quad_sum(float x) {
+  const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false,
+                                                  false);
+  const float y = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(y), __float_as_uint(y), false,
+                                                  false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+// Key position -> block-table entry and offset in the page.  Page sizes are powers of
+// two nearly always: `shift` is then log2(page_size) and the division (some thirty
+// instructions, several times per tile) becomes a shift; otherwise `shift` is -1.
+__device__ __forceinline__ int page_shift_of(int page_size) {
+  return (page_size & (page_size - 1)) == 0 ? __ffs(page_size) - 1 : -1;
+}
+__device__ __forceinline__ int page_entry(int kp, int page_size, int shift) {
+  return shift >= 0 ? kp >> shift : kp / page_size;
+}
+__device__ __forceinline__ int page_offset(int kp, int page_size, int shift) {
+  return shift >= 0 ? kp & (page_size - 1) : kp % page_size;
+}
+
+template <int D, int NW, int NS>
+__global__ void __launch_bounds__(NW * 64)
 paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                             const bf16_t* __restrict__ kv, const int* __restrict__ block_table,
                             int bt_stride, const int* __restrict__ positions,
                             const int* __restrict__ wi_seq, const int* __restrict__ wi_row0,
-                            const int* __restrict__ wi_count, int nh, int nkv, int page_size,
-                            float scale, int window) {
+                            const int* __restrict__ wi_count, int n_items, int nh, int nkv,
+                            int page_size, float scale_log2e, int window) {
   constexpr int LDK = D + 8;        // padded rows, in elements
   constexpr int LDV = AM_KT + 8;
   constexpr int KSTEPS = D / 32;    // matrix-core steps over the head dimension
   constexpr int DBLK = D / 16;      // 16-wide blocks of the head dimension
   constexpr int VEC_PER_ROW = D / 8;
-  __shared__ __attribute__((aligned(16))) bf16_t Ks[AM_KT * LDK];   // [key][dim]
-  __shared__ __attribute__((aligned(16))) bf16_t Vt[D * LDV];       // [dim][key slot]
+  constexpr int NT = NW * 64;                      // threads
+  constexpr int KVEC = AM_KT * VEC_PER_ROW / NT;   // 16-byte pieces of a key tile per thread
+  constexpr int VVEC = D * (AM_KT / 4) / NT;       // 8-byte pieces of a value tile per thread
+  constexpr int KROWS = NT / VEC_PER_ROW;          // keys between a thread's pieces
+  static_assert(NW * NS * 16 == AM_ROWS && KVEC >= 1 && VVEC >= 1, "tile shape");
+  extern __shared__ __attribute__((aligned(16))) unsigned char am_smem[];
+  bf16_t* Ks = reinterpret_cast<bf16_t*>(am_smem);   // [2][key][dim]
+  bf16_t* Vt = Ks + 2 * AM_KT * LDK;                 // [2][dim][key slot]
 
-  const int item = blockIdx.x, gkv = blockIdx.y;
+  const int gkv = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, grp = lane >> 4;
   const int G = nh / nkv;
+  const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int last_entry = bt_stride - 1;
+  const int ps_shift = page_shift_of(page_size);
+
+  // The work of an item grows with its place in a prompt.  The second half of the grid
+  // takes its items in descending order, so that workgroups that start together (and
+  // share a compute unit) weigh about the same in pairs.
+  int item = blockIdx.y;
+  {
+    const int half = n_items / 2;
+    if (item >= half) item = n_items - 1 - (item - half);
+  }
   const int seq = wi_seq[item];
   const int row0 = wi_row0[item];
   int count = wi_count[item];
-  if (count * G > 64) count = 64 / G;   // the host never asks for more
+  if (count * G > AM_ROWS) count = AM_ROWS / G;   // the host never asks for more
   const int rows = count * G;
   const int* table = block_table + (size_t)seq * bt_stride;
 
-  const int rr = wave * 16 + r16;
-  const bool row_valid = rr < rows;
-  const int tok = row0 + (row_valid ? rr / G : 0);
-  const int head = gkv * G + (row_valid ? rr % G : 0);
-  const int pos_row = row_valid ? positions[tok] : -1;
-  const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-
-  bf16x8_t qf[KSTEPS];
+  int tok[NS], head[NS], pos_row[NS];
+  bool row_valid[NS];
+  bf16x8_t qf[NS][KSTEPS];
 #pragma unroll
-  for (int ks = 0; ks < KSTEPS; ++ks)
-    qf[ks] = row_valid ? *reinterpret_cast<const bf16x8_t*>(
-                             q + ((size_t)tok * nh + head) * D + ks * 32 + grp * 8)
-                       : zero8;
+  for (int c = 0; c < NS; ++c) {
+    const int rr = wave * (NS * 16) + c * 16 + r16;
+    row_valid[c] = rr < rows;
+    tok[c] = row0 + (row_valid[c] ? rr / G : 0);
+    head[c] = gkv * G + (row_valid[c] ? rr % G : 0);
+    pos_row[c] = row_valid[c] ? positions[tok[c]] : -1;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks)
+      qf[c][ks] = row_valid[c] ? *reinterpret_cast<const bf16x8_t*>(
+                                     q + ((size_t)tok[c] * nh + head[c]) * D + ks * 32 + grp * 8)
+                               : zero8;
+  }
 
   const int pos_first = positions[row0];
   const int pos_last = positions[row0 + count - 1];
   const int lo = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
   const int hi = pos_last;
-  // what this wave's rows can see at most
-  const int wave_first_row = wave * 16;
+  // what this wave's rows can see
+  const int wave_first_row = wave * (NS * 16);
   const bool wave_active = wave_first_row < rows;
-  int wave_last_tok = (wave_first_row + 15) / G;
+  const bool wave_full = wave_first_row + NS * 16 <= rows;
+  int wave_last_tok = (wave_first_row + NS * 16 - 1) / G;
   if (wave_last_tok > count - 1) wave_last_tok = count - 1;
   const int wave_hi = wave_active ? positions[row0 + wave_last_tok] : -1;
+  const int wave_lo = wave_active ? positions[row0 + wave_first_row / G] : 0;
 
-  f32x4_t o[DBLK];
+  f32x4_t o[NS][DBLK];
+  float m[NS], l[NS];
 #pragma unroll
-  for (int db = 0; db < DBLK; ++db) o[db] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, l = 0.f;
+  for (int c = 0; c < NS; ++c) {
+    m[c] = -INFINITY;
+    l[c] = 0.f;
+#pragma unroll
+    for (int db = 0; db < DBLK; ++db) o[c][db] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  }
 
-  const size_t vofs = (size_t)nkv * page_size * D;
-  for (int tile0 = (lo / AM_KT) * AM_KT; tile0 <= hi; tile0 += AM_KT) {
-    __syncthreads();
-    // keys: lanes run along the head dimension (coalesced rows)
+  // This thread's pieces of a tile: KVEC 16-byte runs along the head dimension of keys
+  // krow0 + v * KROWS, and VVEC 8-byte runs of 4 consecutive keys (run vkr of the
+  // tile) for head-dimension elements vdd0 + v * (NT / 16).  What does not change from
+  // tile to tile is folded into two base pointers.
+  const int krow0 = tid / VEC_PER_ROW, vkr = tid & 15, vdd0 = tid >> 4;
+  const size_t page_stride = (size_t)2 * nkv * page_size * D;
+  const bf16_t* kbase = kv + (size_t)gkv * page_size * D + (tid % VEC_PER_ROW) * 8;
+  const bf16_t* vbase = kv + ((size_t)nkv + gkv) * page_size * D + (size_t)vdd0 * page_size;
+  const int vstep = (NT / 16) * page_size;   // elements between a thread's value pieces
+
+  int kpg[KVEC], vpg;
+  bf16x8_t kreg[KVEC];
+  bf16x4_t vreg[VVEC];
+  auto load_pages = [&](int tile0) {
 #pragma unroll
-    for (int v = 0; v < AM_KT * VEC_PER_ROW / 256; ++v) {
-      const int idx = tid + v * 256;
-      const int j = idx / VEC_PER_ROW, c = (idx % VEC_PER_ROW) * 8;
-      const int kp = tile0 + j;
-      bf16x8_t kx = zero8;
-      if (kp >= lo && kp <= hi) {
-        const int page = table[kp / page_size];
-        if (page >= 0)
-          kx = *reinterpret_cast<const bf16x8_t*>(
-              kv + ((((size_t)page * 2) * nkv + gkv) * page_size + kp % page_size) * D + c);
-      }
-      *reinterpret_cast<bf16x8_t*>(Ks + j * LDK + c) = kx;
+    for (int v = 0; v < KVEC; ++v) {
+      const int e = page_entry(tile0 + krow0 + v * KROWS, page_size, ps_shift);
+      kpg[v] = table[e < last_entry ? e : last_entry];
     }
-    // values, transposed: lanes run along the keys so that the 2-byte stores of one
-    // instruction fall side by side
+    const int e = page_entry(tile0 + vkr * 4, page_size, ps_shift);
+    vpg = table[e < last_entry ? e : last_entry];
+  };
+  // Loads never leave the pool: an unused table entry (-1) reads page 0 instead, and
+  // tiles beyond the last one are fetched like any other.  A key that must not count is
+  // masked in the scores, whatever its row holds; its values are cleared on their way
+  // into LDS, since 0 * (not a number) would not be 0.
+  auto load_data = [&](int tile0) {
 #pragma unroll
-    for (int v = 0; v < AM_KT * VEC_PER_ROW / 256; ++v) {
-      const int idx = tid + v * 256;
-      const int j = idx % AM_KT, c = (idx / AM_KT) * 8;
-      const int kp = tile0 + j;
-      bf16x8_t vx = zero8;
-      if (kp >= lo && kp <= hi) {
-        const int page = table[kp / page_size];
-        if (page >= 0)
-          vx = *reinterpret_cast<const bf16x8_t*>(
-              kv + ((((size_t)page * 2) * nkv + gkv) * page_size + kp % page_size) * D + vofs + c);
-      }
-      // key j of the tile sits in slot: 32-key step, then lane group, then block, then i
-      const int slot = (j & 32) + ((j & 15) >> 2) * 8 + ((j >> 4) & 1) * 4 + (j & 3);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) Vt[(c + e) * LDV + slot] = vx[e];
+    for (int v = 0; v < KVEC; ++v) {
+      const int off = page_offset(tile0 + krow0 + v * KROWS, page_size, ps_shift);
+      const int page = kpg[v] < 0 ? 0 : kpg[v];
+      kreg[v] = *reinterpret_cast<const bf16x8_t*>(kbase + (size_t)page * page_stride + off * D);
     }
-    __syncthreads();
+    const int off = page_offset(tile0 + vkr * 4, page_size, ps_shift);
+    const int page = vpg < 0 ? 0 : vpg;
+    const bf16_t* src = vbase + (size_t)page * page_stride + off;
+#pragma unroll
+    for (int v = 0; v < VVEC; ++v)
+      vreg[v] = *reinterpret_cast<const bf16x4_t*>(src + v * vstep);
+  };
+  // keys jb * 16 + g4 * 4 .. + 3 of the tile sit in slots: 32-key step, then lane group,
+  // then block
+  const int vslot = ((vkr >> 3) & 1) * 32 + (vkr & 3) * 8 + ((vkr >> 2) & 1) * 4;
+  auto store_tile = [&](int buf, int tile0) {
+    bf16_t* ks = Ks + buf * AM_KT * LDK;
+    bf16_t* vt = Vt + buf * D * LDV;
+#pragma unroll
+    for (int v = 0; v < KVEC; ++v)
+      *reinterpret_cast<bf16x8_t*>(ks + (krow0 + v * KROWS) * LDK + (tid % VEC_PER_ROW) * 8) =
+          kreg[v];
+    const int kp = tile0 + vkr * 4;
+    const bool edge_tile = tile0 < lo || tile0 + AM_KT - 1 > hi;   // the same for all threads
+#pragma unroll
+    for (int v = 0; v < VVEC; ++v) {
+      bf16x4_t x = vreg[v];
+      if (edge_tile) {
+        // keys outside [lo, hi] (pages that are not there lie outside it too)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (kp + e < lo || kp + e > hi) x[e] = (bf16_t)0.f;
+      }
+      *reinterpret_cast<bf16x4_t*>(vt + (vdd0 + v * (NT / 16)) * LDV + vslot) = x;
+    }
+  };
 
-    if (wave_active && tile0 <= wave_hi) {
-      f32x4_t s[4];
+  const int tile_first = (lo / AM_KT) * AM_KT;
+  const int n_tiles = (hi - tile_first) / AM_KT + 1;
+  load_pages(tile_first);
+  load_data(tile_first);
+  load_pages(tile_first + AM_KT);
+  store_tile(0, tile_first);
+  __syncthreads();
+
+  for (int t = 0; t < n_tiles; ++t) {
+    const int tile0 = tile_first + t * AM_KT;
+    const int buf = t & 1;
+    load_data(tile0 + AM_KT);
+    load_pages(tile0 + 2 * AM_KT);
+
+    bool wave_sees = wave_active && tile0 <= wave_hi;
+    if (window > 0 && tile0 + AM_KT - 1 <= wave_lo - window) wave_sees = false;
+    if (wave_sees) {
+      const bf16_t* ks = Ks + buf * AM_KT * LDK;
+      const bf16_t* vt = Vt + buf * D * LDV;
+      f32x4_t s[NS][4];
 #pragma unroll
       for (int jb = 0; jb < 4; ++jb) {
-        s[jb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
+        for (int c = 0; c < NS; ++c) s[c][jb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks_ = 0; ks_ < KSTEPS; ++ks_) {
           const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(
-              Ks + (jb * 16 + r16) * LDK + ks * 32 + grp * 8);
-          s[jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], s[jb], 0, 0, 0);
+              ks + (jb * 16 + r16) * LDK + ks_ * 32 + grp * 8);
+#pragma unroll
+          for (int c = 0; c < NS; ++c)
+            s[c][jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c][ks_], s[c][jb], 0, 0, 0);
         }
       }
-      float tmax = -INFINITY;
+      // a tile every key of which counts for every row of the wave needs no mask
+      const bool needs_mask = !wave_full || tile0 + AM_KT - 1 > wave_lo || tile0 < lo ||
+                              (window > 0 && tile0 <= wave_hi - window);
+      bf16x8_t pf[NS][2];
 #pragma unroll
-      for (int jb = 0; jb < 4; ++jb)
+      for (int c = 0; c < NS; ++c) {
+        if (needs_mask) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int kp = tile0 + jb * 16 + grp * 4 + i;
-          bool valid = kp <= pos_row && kp >= lo;
-          if (window > 0 && kp <= pos_row - window) valid = false;
-          const float v = valid ? s[jb][i] * scale : -INFINITY;
-          s[jb][i] = v;
-          tmax = fmaxf(tmax, v);
+          for (int jb = 0; jb < 4; ++jb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int kp = tile0 + jb * 16 + grp * 4 + i;
+              bool valid = kp <= pos_row[c] && kp >= lo;
+              if (window > 0 && kp <= pos_row[c] - window) valid = false;
+              if (!valid) s[c][jb][i] = -INFINITY;
+            }
         }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-      const float m_new = fmaxf(m, tmax);
-      const float m_use = m_new > -INFINITY ? m_new : 0.f;
-      const float alpha = expf(m - m_use);          // m = -inf gives 0
-      float psum = 0.f;
+        float tmax = -INFINITY;
 #pragma unroll
-      for (int jb = 0; jb < 4; ++jb)
+        for (int jb = 0; jb < 4; ++jb)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float p = expf(s[jb][i] - m_use);   // masked scores give 0
-          s[jb][i] = p;
-          psum += p;
+          for (int i = 0; i < 4; ++i) tmax = fmaxf(tmax, s[c][jb][i]);
+        tmax = quad_max(tmax);
+        const float m_new = fmaxf(m[c], tmax * scale_log2e);   // the factor is positive
+        const float m_use = m_new > -INFINITY ? m_new : 0.f;
+        const float alpha = __builtin_amdgcn_exp2f(m[c] - m_use);   // m = -inf gives 0
+        float psum = 0.f;
+#pragma unroll
+        for (int jb = 0; jb < 4; ++jb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            // masked scores (-inf) give 0
+            const float p = __builtin_amdgcn_exp2f(fmaf(s[c][jb][i], scale_log2e, -m_use));
+            s[c][jb][i] = p;
+            psum += p;
+          }
+        psum = quad_sum(psum);
+        l[c] = l[c] * alpha + psum;
+        m[c] = m_new;
+        if (__any(alpha != 1.0f)) {
+#pragma unroll
+          for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[c][db][i] *= alpha;
         }
-      psum += __shfl_xor(psum, 16, 64);
-      psum += __shfl_xor(psum, 32, 64);
-      l = l * alpha + psum;
-      m = m_new;
 #pragma unroll
-      for (int db = 0; db < DBLK; ++db)
+        for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[db][i] *= alpha;
-      bf16x8_t pf[2];
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          pf[kk][i] = (bf16_t)s[2 * kk][i];
-          pf[kk][4 + i] = (bf16_t)s[2 * kk + 1][i];
-        }
+          for (int i = 0; i < 4; ++i) {
+            pf[c][kk][i] = (bf16_t)s[c][2 * kk][i];
+            pf[c][kk][4 + i] = (bf16_t)s[c][2 * kk + 1][i];
+          }
+      }
 #pragma unroll
       for (int db = 0; db < DBLK; ++db)
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
           const bf16x8_t vf = *reinterpret_cast<const bf16x8_t*>(
-              Vt + (db * 16 + r16) * LDV + kk * 32 + grp * 8);
-          o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[kk], o[db], 0, 0, 0);
+              vt + (db * 16 + r16) * LDV + kk * 32 + grp * 8);
+#pragma unroll
+          for (int c = 0; c < NS; ++c)
+            o[c][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[c][kk], o[c][db], 0, 0, 0);
         }
     }
+    if (t + 1 < n_tiles) store_tile(buf ^ 1, tile0 + AM_KT);
+    __syncthreads();
   }
 
-  if (row_valid) {
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
-    bf16_t* dst = out + ((size_t)tok * nh + head) * D;
 #pragma unroll
-    for (int db = 0; db < DBLK; ++db)
+  for (int c = 0; c < NS; ++c)
+    if (row_valid[c]) {
+      const float inv = l[c] > 0.f ? 1.0f / l[c] : 0.f;
+      bf16_t* dst = out + ((size_t)tok[c] * nh + head[c]) * D;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) dst[db * 16 + grp * 4 + i] = (bf16_t)(o[db][i] * inv);
-  }
+      for (int db = 0; db < DBLK; ++db) {
+        bf16x4_t ov;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ov[i] = (bf16_t)(o[c][db][i] * inv);
+        *reinterpret_cast<bf16x4_t*>(dst + db * 16 + grp * 4) = ov;
+      }
+    }
 }
 
 // Decoding on the matrix cores: work items of at most 16 rows (one or a few
@@ -415,10 +565,11 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
 // second operand.  The four waves of a workgroup take the key tiles of the
 // workgroup's key range in turn and never wait for each other inside the loop:
 // keys go from global memory straight into first-operand registers (a lane needs
-// 8 consecutive head-dim elements of one key), values are turned through a
-// wave-private LDS tile into the key-major order the second product needs.  At the
-// end the four partial (m, l, O) are merged in LDS; with `nsplit` > 1 the merged
-// partial goes to `attention_combine_kernel` like those of the plain kernel.
+// 8 consecutive head-dim elements of one key), and so do the values (a lane needs,
+// for one head-dim element, two runs of 4 consecutive keys, which the cache holds
+// side by side).  At the end the four partial (m, l, O) are merged in LDS; with
+// `nsplit` > 1 the merged partial goes to `attention_combine_kernel` like those of
+// the plain kernel.
 template <int D>
 __global__ void __launch_bounds__(256)
 paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
@@ -429,11 +580,8 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
                                    const int* __restrict__ wi_count, float* __restrict__ part_acc,
                                    float* __restrict__ part_ml, int nh, int nkv, int page_size,
                                    float scale, int window, int keys_per_split, int nsplit) {
-  constexpr int LDV = AM_KT + 8;
   constexpr int KSTEPS = D / 32;
   constexpr int DBLK = D / 16;
-  constexpr int VEC_PER_ROW = D / 8;
-  __shared__ __attribute__((aligned(16))) bf16_t Vt_all[4 * D * LDV];   // [wave][dim][key slot]
   __shared__ float mg_m[4][16], mg_l[4][16];
   __shared__ float mg_o[4][DBLK][64][4];
 
@@ -448,7 +596,6 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
   if (count * G > 16) count = 16 / G;   // the host never asks for more
   const int rows = count * G;
   const int* table = block_table + (size_t)seq * bt_stride;
-  bf16_t* Vt = Vt_all + wave * D * LDV;
 
   const bool row_valid = r16 < rows;
   const int tok = row0 + (row_valid ? r16 / G : 0);
@@ -478,50 +625,66 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
 #pragma unroll
   for (int db = 0; db < DBLK; ++db) o[db] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
-  const size_t vofs = (size_t)nkv * page_size * D;
 
-  // One tile's keys (first-operand fragments) and values (rows along the head
-  // dimension, lane = key) in registers; the next tile is fetched while this one is
-  // being computed.
-  bf16x8_t kf[4][KSTEPS], vx[VEC_PER_ROW];
+  // One tile's keys and values as first-operand fragments in registers; the next tile
+  // is fetched while this one is being computed.  vf[db][jb] holds, for head-dim
+  // element db * 16 + r16, keys jb * 16 + grp * 4 .. + 3 of the tile.
+  bf16x8_t kf[4][KSTEPS];
+  bf16x4_t vf[DBLK][4];
   // The block-table entries are read whether or not the key turns out to be in
-  // range (unused entries hold -1), so that these loads do not wait for the
-  // positions the range is computed from.
+  // range (unused entries hold -1 and read page 0 instead), so that these loads do
+  // not wait for the positions the range is computed from.  A key that must not
+  // count is masked in the scores, whatever its row holds; its values are cleared,
+  // since 0 * (not a number) would not be 0.
   const int last_entry = bt_stride - 1;
-  auto fetch = [&](int tile0, bf16x8_t (&kfr)[4][KSTEPS], bf16x8_t (&vxr)[VEC_PER_ROW]) {
-    int kpage[4];
+  const int ps_shift = page_shift_of(page_size);
+  auto fetch = [&](int tile0, bf16x8_t (&kfr)[4][KSTEPS], bf16x4_t (&vfr)[DBLK][4]) {
+    int kpage[4], vpage[4];
 #pragma unroll
     for (int jb = 0; jb < 4; ++jb) {
-      const int e = (tile0 + jb * 16 + r16) / page_size;
+      const int e = page_entry(tile0 + jb * 16 + r16, page_size, ps_shift);
       kpage[jb] = table[e < last_entry ? e : last_entry];
+      const int ev = page_entry(tile0 + jb * 16 + grp * 4, page_size, ps_shift);
+      vpage[jb] = table[ev < last_entry ? ev : last_entry];
     }
-    const int ve = (tile0 + lane) / page_size;
-    const int vpage = table[ve < last_entry ? ve : last_entry];
 #pragma unroll
     for (int jb = 0; jb < 4; ++jb) {
       const int kp = tile0 + jb * 16 + r16;
-      const bf16_t* krow = nullptr;
-      if (kp >= lo && kp <= range_hi && kpage[jb] >= 0)
-        krow = kv + ((((size_t)kpage[jb] * 2) * nkv + gkv) * page_size + kp % page_size) * D;
+      const int page = kpage[jb] < 0 ? 0 : kpage[jb];
+      const bf16_t* krow = kv + ((((size_t)page * 2) * nkv + gkv) * page_size +
+                                 page_offset(kp, page_size, ps_shift)) * D;
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks)
-        kfr[jb][ks] = krow ? *reinterpret_cast<const bf16x8_t*>(krow + ks * 32 + grp * 8) : zero8;
+        kfr[jb][ks] = *reinterpret_cast<const bf16x8_t*>(krow + ks * 32 + grp * 8);
     }
-    const int kp = tile0 + lane;
-    const bf16_t* vrow = nullptr;
-    if (kp >= lo && kp <= range_hi && vpage >= 0)
-      vrow = kv + ((((size_t)vpage * 2) * nkv + gkv) * page_size + kp % page_size) * D + vofs;
+    const bool inner = tile0 >= lo && tile0 + AM_KT - 1 <= range_hi;
 #pragma unroll
-    for (int v = 0; v < VEC_PER_ROW; ++v)
-      vxr[v] = vrow ? *reinterpret_cast<const bf16x8_t*>(vrow + v * 8) : zero8;
+    for (int jb = 0; jb < 4; ++jb) {
+      const int kp = tile0 + jb * 16 + grp * 4;
+      const int page = vpage[jb] < 0 ? 0 : vpage[jb];
+      const bf16_t* vbase = kv + (((size_t)page * 2 + 1) * nkv + gkv) * page_size * D +
+                            page_offset(kp, page_size, ps_shift);
+#pragma unroll
+      for (int db = 0; db < DBLK; ++db) {
+        bf16x4_t x =
+            *reinterpret_cast<const bf16x4_t*>(vbase + (size_t)(db * 16 + r16) * page_size);
+        if (!inner) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (vpage[jb] < 0 || kp + e < lo || kp + e > range_hi) x[e] = (bf16_t)0.f;
+        }
+        vfr[db][jb] = x;
+      }
+    }
   };
 
   int tile0 = tile_first + wave * AM_KT;
-  if (tile0 <= range_hi) fetch(tile0, kf, vx);
+  if (tile0 <= range_hi) fetch(tile0, kf, vf);
   for (; tile0 <= range_hi; tile0 += 4 * AM_KT) {
-    bf16x8_t kfn[4][KSTEPS], vxn[VEC_PER_ROW];
+    bf16x8_t kfn[4][KSTEPS];
+    bf16x4_t vfn[DBLK][4];
     const int next = tile0 + 4 * AM_KT;
-    if (next <= range_hi) fetch(next, kfn, vxn);
+    if (next <= range_hi) fetch(next, kfn, vfn);
 
     f32x4_t s[4];
 #pragma unroll
@@ -530,15 +693,6 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks)
         s[jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[jb][ks], qf[ks], s[jb], 0, 0, 0);
-    }
-    // values into this wave's LDS tile, key-major (lane = key j of the tile)
-    {
-      const int j = lane;
-      const int slot = (j & 32) + ((j & 15) >> 2) * 8 + ((j >> 4) & 1) * 4 + (j & 3);
-#pragma unroll
-      for (int v = 0; v < VEC_PER_ROW; ++v)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) Vt[(v * 8 + e) * LDV + slot] = vx[v][e];
     }
     float tmax = -INFINITY;
 #pragma unroll
@@ -552,8 +706,7 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
         s[jb][i] = v;
         tmax = fmaxf(tmax, v);
       }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    tmax = quad_max(tmax);
     const float m_new = fmaxf(m, tmax);
     const float m_use = m_new > -INFINITY ? m_new : 0.f;
     const float alpha = expf(m - m_use);
@@ -566,8 +719,7 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
         s[jb][i] = p;
         psum += p;
       }
-    psum += __shfl_xor(psum, 16, 64);
-    psum += __shfl_xor(psum, 32, 64);
+    psum = quad_sum(psum);
     l = l * alpha + psum;
     m = m_new;
 #pragma unroll
@@ -582,23 +734,22 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
         pf[kk][i] = (bf16_t)s[2 * kk][i];
         pf[kk][4 + i] = (bf16_t)s[2 * kk + 1][i];
       }
-    __builtin_amdgcn_wave_barrier();   // this wave's stores to Vt precede its loads below
 #pragma unroll
     for (int db = 0; db < DBLK; ++db)
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk) {
-        const bf16x8_t vf = *reinterpret_cast<const bf16x8_t*>(
-            Vt + (db * 16 + r16) * LDV + kk * 32 + grp * 8);
-        o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[kk], o[db], 0, 0, 0);
+        const bf16x8_t vv = __builtin_shufflevector(vf[db][2 * kk], vf[db][2 * kk + 1], 0, 1, 2,
+                                                    3, 4, 5, 6, 7);
+        o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, pf[kk], o[db], 0, 0, 0);
       }
-    __builtin_amdgcn_wave_barrier();   // and those loads precede the next tile's stores
     if (next <= range_hi) {
 #pragma unroll
-      for (int jb = 0; jb < 4; ++jb)
+      for (int jb = 0; jb < 4; ++jb) {
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) kf[jb][ks] = kfn[jb][ks];
 #pragma unroll
-      for (int v = 0; v < VEC_PER_ROW; ++v) vx[v] = vxn[v];
+        for (int db = 0; db < DBLK; ++db) vf[db][jb] = vfn[db][jb];
+      }
     }
   }
 
@@ -704,8 +855,35 @@ extern "C" int za_paged_attention(const void* q, void* out, const void* kv, cons
   return za_launch_status();
 }
 
-// Matrix-core variant: bfloat16 only, head_dim 64 or 128, (nh / nkv) dividing 16, work
-// items of at most 64 / (nh / nkv) query rows.  Returns ZA_ERR_UNSUPPORTED otherwise.
+template <int D>
+static int launch_attention_mfma(const void* q, void* out, const void* kv, const int* block_table,
+                                 int bt_stride, const int* positions, const int* wi_seq,
+                                 const int* wi_row0, const int* wi_count, int n_items, int nh,
+                                 int nkv, int page_size, float scale, int window,
+                                 hipStream_t stream) {
+  constexpr int NW = 8, NS = AM_ROWS / (NW * 16);
+  const size_t shmem = ((size_t)2 * AM_KT * (D + 8) + (size_t)2 * D * (AM_KT + 8)) * sizeof(bf16_t);
+  auto kernel = paged_attention_mfma_kernel<D, NW, NS>;
+  static bool allowed = false;
+  if (!allowed) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+    if (e != hipSuccess) return (int)e;
+    allowed = true;
+  }
+  if (n_items > 65535) return ZA_ERR_UNSUPPORTED;
+  // the key/value head runs fastest, so that workgroups that follow each other (and
+  // are dealt to the chip's eight dies in turn) read different heads' keys and values
+  dim3 grid(nkv, n_items), block(NW * 64);
+  hipLaunchKernelGGL(kernel, grid, block, shmem, stream, (const bf16_t*)q, (bf16_t*)out,
+                     (const bf16_t*)kv, block_table, bt_stride, positions, wi_seq, wi_row0,
+                     wi_count, n_items, nh, nkv, page_size, scale * 1.44269504088896341f, window);
+  return za_launch_status();
+}
+
+// Matrix-core variant: bfloat16 only, head_dim 64 or 128, page sizes that are
+// multiples of 4, a positive scale, work items of at most 128 / (nh / nkv) query
+// tokens.  Returns ZA_ERR_UNSUPPORTED otherwise.
 extern "C" int za_paged_attention_mfma(const void* q, void* out, const void* kv,
                                        const int* block_table, int bt_stride,
                                        const int* positions, const int* wi_seq,
@@ -717,21 +895,21 @@ extern "C" int za_paged_attention_mfma(const void* q, void* out, const void* kv,
       !q || !out || !kv || !block_table || !positions || !wi_seq || !wi_row0 || !wi_count)
     return ZA_ERR_ARG;
   const int G = nh / nkv;
-  if ((d != 64 && d != 128) || G > 16 || 16 % G != 0 || nkv > 65535) return ZA_ERR_UNSUPPORTED;
-  dim3 grid(n_items, nkv), block(256);
+  if ((d != 64 && d != 128) || G > AM_ROWS || page_size % 4 != 0 || !(scale > 0.f) ||
+      nkv > 65535)
+    return ZA_ERR_UNSUPPORTED;
   if (d == 64)
-    hipLaunchKernelGGL((paged_attention_mfma_kernel<64>), grid, block, 0, stream,
-                       (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
-                       positions, wi_seq, wi_row0, wi_count, nh, nkv, page_size, scale, window);
-  else
-    hipLaunchKernelGGL((paged_attention_mfma_kernel<128>), grid, block, 0, stream,
-                       (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
-                       positions, wi_seq, wi_row0, wi_count, nh, nkv, page_size, scale, window);
-  return za_launch_status();
+    return launch_attention_mfma<64>(q, out, kv, block_table, bt_stride, positions, wi_seq,
+                                     wi_row0, wi_count, n_items, nh, nkv, page_size, scale,
+                                     window, stream);
+  return launch_attention_mfma<128>(q, out, kv, block_table, bt_stride, positions, wi_seq,
+                                    wi_row0, wi_count, n_items, nh, nkv, page_size, scale, window,
+                                    stream);
 }
 
-// Matrix-core decode variant: bfloat16, head_dim 64 or 128, work items of at most
-// 16 / (nh / nkv) query rows (nh / nkv dividing 16), contexts optionally cut as in
+// Matrix-core decode variant: bfloat16, head_dim 64 or 128, page sizes that are
+// multiples of 4, work items of at most 16 / (nh / nkv) query tokens, contexts
+// optionally cut as in
 // za_paged_attention (the partial results are merged by the same combine kernel).
 extern "C" int za_paged_attention_decode_mfma(const void* q, void* out, const void* kv,
                                               const int* block_table, int bt_stride,
@@ -749,7 +927,7 @@ extern "C" int za_paged_attention_decode_mfma(const void* q, void* out, const vo
   if (wi_seq && (!wi_row0 || !wi_count)) return ZA_ERR_ARG;
   if (!wi_seq && n_items != n_tokens) return ZA_ERR_ARG;   // identity items: one token each
   const int G = nh / nkv;
-  if ((d != 64 && d != 128) || G > 16 || 16 % G != 0 || nkv > 65535 || nsplit > 65535)
+  if ((d != 64 && d != 128) || G > 16 || page_size % 4 != 0 || nkv > 65535 || nsplit > 65535)
     return ZA_ERR_UNSUPPORTED;
   if (nsplit > 1 && (!part_acc || !part_ml || keys_per_split <= 0 || keys_per_split % 64 != 0))
     return ZA_ERR_ARG;

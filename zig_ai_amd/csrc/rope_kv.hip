@@ -11,7 +11,9 @@
 //          for "half" pairing (the reference's device kernel,
 //          /root/reference/src/cuda/layer_kernels.cu:353-365) or (2p, 2p+1) for "adjacent"
 //          pairing (rope.zig:46-53).  Elements beyond rotary_dim pass through.
-//   k, v -> cache[page][0 or 1][kv_head][offset][head_dim],  slot = page * page_size + offset
+//   k -> cache[page][0][kv_head][offset][head_dim],  slot = page * page_size + offset
+//   v -> cache[page][1][kv_head][head_dim][offset]   (turned round: the attention kernels
+//        read, for one head-dimension element, consecutive keys side by side)
 //   q    -> q_out[token][head][head_dim]
 #include "common.h"
 
@@ -75,9 +77,13 @@ qk_norm_rope_kv_write_kernel(const T* __restrict__ qkv, const int* __restrict__ 
     if (slot < 0) return;
     const int page = slot / page_size, off = slot % page_size;
     const int kvh = is_k ? head - nh : head - nh - nkv;
-    const int which = is_k ? 0 : 1;
-    T* dst = kv_cache + ((((size_t)page * 2 + which) * nkv + kvh) * page_size + off) * d;
-    for (int i = lane; i < d; i += 64) dst[i] = from_f32<T>(s[i]);
+    if (is_k) {
+      T* dst = kv_cache + ((((size_t)page * 2) * nkv + kvh) * page_size + off) * d;
+      for (int i = lane; i < d; i += 64) dst[i] = from_f32<T>(s[i]);
+    } else {
+      T* dst = kv_cache + (((size_t)page * 2 + 1) * nkv + kvh) * page_size * d + off;
+      for (int i = lane; i < d; i += 64) dst[(size_t)i * page_size] = from_f32<T>(s[i]);
+    }
   }
 }
 

@@ -46,8 +46,8 @@ _SIGNATURES = {
                                                       c_int, c_int, c_int, c_int, c_float, c_int,
                                                       c_int, c_int, c_void_p],
     ("shortconv", "za_short_conv"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                     c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_longlong,
-                                     c_void_p],
+                                     c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                     c_longlong, c_void_p],
     ("activation", "za_swiglu"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     ("activation", "za_cast"): [c_void_p, c_int, c_void_p, c_int, c_longlong, c_void_p],
     ("sampling", "za_argmax"): [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int,
@@ -284,7 +284,9 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor,
                           head_dim: int, rotary_dim: int, adjacent_pairs: bool, eps: float,
                           write_kv: bool = True) -> torch.Tensor:
     """Returns the normalised, rotated queries ``[T, num_heads, head_dim]`` and
-    scatters keys/values into ``kv_cache [pages, 2, kv_heads, page_size, head_dim]``."""
+    scatters keys/values into ``kv_cache [pages, 2, kv_heads, page_size, head_dim]``
+    (keys as ``[offset][head_dim]``; the values' half of a page holds
+    ``[head_dim][offset]``)."""
     T = qkv.shape[0]
     total = num_heads + 2 * num_kv_heads
     _need(qkv, "qkv", (torch.float32, torch.bfloat16), (T, total * head_dim))
@@ -380,24 +382,26 @@ def paged_attention(q: torch.Tensor, kv_cache: torch.Tensor, block_table: torch.
     return out
 
 
-ATTENTION_MFMA_ROWS = 64
+ATTENTION_MFMA_ROWS = 128
 
 
 def attention_mfma_supported(dtype: torch.dtype, num_heads: int, num_kv_heads: int,
-                             head_dim: int) -> bool:
-    """Whether the matrix-core attention kernel takes these sizes."""
+                             head_dim: int, page_size: int = 4, scale: float = 1.0) -> bool:
+    """Whether the matrix-core attention kernels (the one for prompt portions and
+    the one for decoding) take these sizes."""
     group = num_heads // num_kv_heads
     return (dtype == torch.bfloat16 and head_dim in (64, 128) and group <= 16
-            and 16 % group == 0)
+            and page_size % 4 == 0 and scale > 0.0)
 
 
 def paged_attention_mfma(q: torch.Tensor, kv_cache: torch.Tensor, block_table: torch.Tensor,
                          positions: torch.Tensor, item_seq: torch.Tensor,
                          item_row0: torch.Tensor, item_count: torch.Tensor, n_items: int,
                          scale: float, window: int = 0) -> torch.Tensor:
-    """The same attention on the matrix cores (bfloat16, head_dim 64 or 128, query
-    heads per key/value head dividing 16).  Work items hold at most
-    ``ATTENTION_MFMA_ROWS // (heads // kv_heads)`` query rows; contexts are not cut."""
+    """The same attention on the matrix cores (bfloat16, head_dim 64 or 128, at most
+    16 query heads per key/value head, a page size that is a multiple of 4, a
+    positive scale).  Work items hold at most
+    ``ATTENTION_MFMA_ROWS // (heads // kv_heads)`` query tokens; contexts are not cut."""
     if q.dim() != 3:
         raise KernelError(f"q must be [T, heads, head_dim], got {tuple(q.shape)}")
     T, nh, d = q.shape
@@ -407,9 +411,9 @@ def paged_attention_mfma(q: torch.Tensor, kv_cache: torch.Tensor, block_table: t
         raise KernelError(f"kv_cache has shape {tuple(kv_cache.shape)}, expected "
                           f"[pages, 2, kv_heads, page_size, {d}]")
     nkv, page_size = kv_cache.shape[2], kv_cache.shape[3]
-    if nh % nkv or not attention_mfma_supported(q.dtype, nh, nkv, d):
+    if nh % nkv or not attention_mfma_supported(q.dtype, nh, nkv, d, page_size, scale):
         raise KernelError(f"the matrix-core attention kernel does not take {nh} heads, {nkv} "
-                          f"key/value heads, head_dim {d}")
+                          f"key/value heads, head_dim {d}, page size {page_size}, scale {scale}")
     _need(block_table, "block_table", torch.int32)
     if block_table.dim() != 2:
         raise KernelError("block_table must be [requests, max_pages]")
@@ -438,7 +442,7 @@ def paged_attention_decode_mfma(q: torch.Tensor, kv_cache: torch.Tensor,
                                 window: int = 0, keys_per_split: int = 0,
                                 nsplit: int = 1) -> torch.Tensor:
     """The matrix-core kernel for decoding: work items of at most
-    ``ATTENTION_MFMA_DECODE_ROWS // (heads // kv_heads)`` query rows, long contexts
+    ``ATTENTION_MFMA_DECODE_ROWS // (heads // kv_heads)`` query tokens, long contexts
     optionally cut into ``nsplit`` ranges of ``keys_per_split`` keys.  With
     ``item_seq=None`` row ``i`` of ``q`` is the single token of request ``i``."""
     if q.dim() != 3:
@@ -450,9 +454,9 @@ def paged_attention_decode_mfma(q: torch.Tensor, kv_cache: torch.Tensor,
         raise KernelError(f"kv_cache has shape {tuple(kv_cache.shape)}, expected "
                           f"[pages, 2, kv_heads, page_size, {d}]")
     nkv, page_size = kv_cache.shape[2], kv_cache.shape[3]
-    if nh % nkv or not attention_mfma_supported(q.dtype, nh, nkv, d):
+    if nh % nkv or not attention_mfma_supported(q.dtype, nh, nkv, d, page_size, scale):
         raise KernelError(f"the matrix-core attention kernel does not take {nh} heads, {nkv} "
-                          f"key/value heads, head_dim {d}")
+                          f"key/value heads, head_dim {d}, page size {page_size}, scale {scale}")
     _need(block_table, "block_table", torch.int32)
     if block_table.dim() != 2:
         raise KernelError("block_table must be [requests, max_pages]")
@@ -511,7 +515,8 @@ def short_conv(z: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tenso
     y = torch.empty((T, width), dtype=z.dtype, device=z.device)
     rc = _fn("shortconv", "za_short_conv")(_ptr(z), _ptr(weight), _ptr(bias), _ptr(state),
                                            _ptr(token_seq), _ptr(seq_start), _ptr(slot_id), _ptr(y),
-                                           _code(z.dtype), T, width, L, state.stride(0), _stream())
+                                           _code(z.dtype), T, slot_id.numel(), width, L,
+                                           state.stride(0), _stream())
     _check(rc, "short_conv")
     return y
 

@@ -95,15 +95,17 @@ class GroupedQueryAttention(Mixer):
             raise ValueError(f"head_dim {self.head_dim} must be a multiple of 16, at most 256")
         # tokens per work item of the two attention kernels
         self.rows_per_item = max(1, ops.ATTENTION_MAX_ROWS // self.group)
-        self.mfma = ops.attention_mfma_supported(runtime.dtype, self.num_heads,
-                                                 self.num_kv_heads, self.head_dim)
         self.mfma_rows_per_item = max(1, ops.ATTENTION_MFMA_ROWS // self.group)
         self.mfma_decode_rows_per_item = max(1, ops.ATTENTION_MFMA_DECODE_ROWS // self.group)
-        self.item_granularities = [self.rows_per_item] + (
-            [self.mfma_rows_per_item, self.mfma_decode_rows_per_item] if self.mfma else [])
         self.window = int(params.get("window") or 0)
         scale = params.get("softmax_scale")
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
+        # whether the matrix-core kernels take these sizes (the page size is checked per step)
+        self.mfma = ops.attention_mfma_supported(runtime.dtype, self.num_heads,
+                                                 self.num_kv_heads, self.head_dim,
+                                                 scale=self.scale)
+        self.item_granularities = [self.rows_per_item] + (
+            [self.mfma_rows_per_item, self.mfma_decode_rows_per_item] if self.mfma else [])
         self.eps = float(params.get("norm_eps", 0.0))
         self.w_qkv = fuse_rows(tensors["q_proj.weight"], tensors["k_proj.weight"],
                                tensors["v_proj.weight"])
@@ -150,13 +152,14 @@ class GroupedQueryAttention(Mixer):
             q = ops.qk_norm_rope_kv_write(packed.contiguous(), step.positions, slots, None, None,
                                           None, cache.kv, nh, nkv, d, 0, False, self.eps,
                                           write_kv=cache.writes)
-        if self.mfma and step.n_tokens > step.n_seqs:
+        mfma = self.mfma and cache.kv.shape[3] % 4 == 0
+        if mfma and step.n_tokens > step.n_seqs:
             # prompt portions in the step: both products on the matrix cores
             o = ops.paged_attention_mfma(q, cache.kv, step.block_tables[cache.group],
                                          step.positions,
                                          *step.attention_items(self.mfma_rows_per_item),
                                          self.scale, self.window)
-        elif self.mfma:
+        elif mfma:
             # single tokens only: the matrix-core kernel whose waves split the keys
             # (every request brings one token: row i is request i, no work-item arrays)
             item_seq = item_row0 = item_count = None
