@@ -221,7 +221,8 @@ def test_gemm_bf16_refuses_odd_k():
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("nh,nkv,d,rot,pairing", [
     (4, 2, 16, 16, "half"), (3, 1, 32, 32, "half"), (5, 5, 48, 48, "adjacent"),
-    (8, 2, 64, 32, "half"), (2, 2, 256, 256, "half"), (6, 3, 128, 64, "adjacent")])
+    (8, 2, 64, 32, "half"), (2, 2, 256, 256, "half"), (6, 3, 128, 64, "adjacent"),
+    (4, 2, 64, 24, "half"), (8, 2, 64, 64, "adjacent"), (7, 7, 32, 16, "half"), (32, 8, 64, 64, "half")])
 def test_qk_norm_rope_kv_write(dtype, nh, nkv, d, rot, pairing):
     T, page_size, pages = 11, 4, 9
     theta, eps = 10000.0, 1e-5

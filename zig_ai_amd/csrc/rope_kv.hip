@@ -87,6 +87,118 @@ qk_norm_rope_kv_write_kernel(const T* __restrict__ qkv, const int* __restrict__ 
   }
 }
 
+// The same for head sizes that are powers of two: a block per token, D / 8 lanes per
+// head with 16-byte accesses, the token's cosines and sines computed once for all its
+// heads, the mean square summed over the head's lanes with lane shuffles.  Half
+// pairing needs rotary_dim / 2 to be a multiple of 8, so that a lane's partner
+// elements all sit in one other lane.
+template <typename T, int D>
+__global__ void __launch_bounds__(256)
+qk_norm_rope_kv_write_pow2_kernel(const T* __restrict__ qkv, const int* __restrict__ positions,
+                                  const int* __restrict__ slots,
+                                  const float* __restrict__ q_norm_w,
+                                  const float* __restrict__ k_norm_w,
+                                  const float* __restrict__ inv_freq, T* __restrict__ q_out,
+                                  T* __restrict__ kv_cache, int nh, int nkv, int rot, int adjacent,
+                                  float eps, int page_size, int write_kv) {
+  constexpr int LPH = D / 8;   // lanes per head
+  __shared__ float cs_tab[D / 2], sn_tab[D / 2];
+  const int t = blockIdx.x;
+  const int half = rot / 2;
+  if ((int)threadIdx.x < half) {
+    const float angle = (float)positions[t] * inv_freq[threadIdx.x];
+    float sn, cs;
+    sincosf(angle, &sn, &cs);
+    cs_tab[threadIdx.x] = cs;
+    sn_tab[threadIdx.x] = sn;
+  }
+  __syncthreads();
+  const int total = nh + 2 * nkv;
+  const int li = threadIdx.x % LPH;
+  const int e0 = li * 8;        // this lane's first element of the head
+  for (int head = threadIdx.x / LPH; head < total; head += 256 / LPH) {
+    const bool is_q = head < nh;
+    const bool is_k = !is_q && head < nh + nkv;
+    float x[8];
+    load8<T>(qkv + ((size_t)t * total + head) * D + e0, x);
+    const float* nw = is_q ? q_norm_w : (is_k ? k_norm_w : nullptr);
+    if (nw) {
+      float ss = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) ss += x[i] * x[i];
+#pragma unroll
+      for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+      const float scale = 1.0f / sqrtf(ss / (float)D + eps);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] = x[i] * scale * nw[e0 + i];
+    }
+    if ((is_q || is_k) && rot > 0) {
+      if (adjacent) {
+#pragma unroll
+        for (int i = 0; i < 8; i += 2)
+          if (e0 + i + 1 < rot) {
+            const int p = (e0 + i) / 2;
+            const float a = x[i], b = x[i + 1], cs = cs_tab[p], sn = sn_tab[p];
+            x[i] = a * cs - b * sn;
+            x[i + 1] = a * sn + b * cs;
+          }
+      } else {
+        const bool low = e0 < half, in_rot = e0 < rot;
+        const int lane = threadIdx.x & 63;
+        const int partner = in_rot ? (low ? lane + half / 8 : lane - half / 8) : lane;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float other = __shfl(x[i], partner, 64);
+          if (in_rot) {
+            const int p = low ? e0 + i : e0 + i - half;
+            const float cs = cs_tab[p], sn = sn_tab[p];
+            x[i] = low ? x[i] * cs - other * sn : other * sn + x[i] * cs;
+          }
+        }
+      }
+    }
+    if (is_q) {
+      store8<T>(q_out + ((size_t)t * nh + head) * D + e0, x);
+    } else if (write_kv) {
+      const int slot = slots[t];
+      if (slot >= 0) {
+        const int page = slot / page_size, off = slot % page_size;
+        if (is_k) {
+          store8<T>(kv_cache + ((((size_t)page * 2) * nkv + (head - nh)) * page_size + off) * D + e0,
+                    x);
+        } else {
+          T* dst = kv_cache + (((size_t)page * 2 + 1) * nkv + (head - nh - nkv)) * page_size * D +
+                   (size_t)e0 * page_size + off;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) dst[(size_t)i * page_size] = from_f32<T>(x[i]);
+        }
+      }
+    }
+  }
+}
+
+template <typename T>
+static bool launch_pow2(const void* qkv, const int* positions, const int* slots,
+                        const float* q_norm_w, const float* k_norm_w, const float* inv_freq,
+                        void* q_out, void* kv_cache, int n_tokens, int nh, int nkv, int d, int rot,
+                        int adjacent, float eps, int page_size, int write_kv,
+                        hipStream_t stream) {
+  if (!adjacent && (rot / 2) % 8 != 0) return false;
+#define ZA_RK_LAUNCH(DD)                                                                        \
+  hipLaunchKernelGGL((qk_norm_rope_kv_write_pow2_kernel<T, DD>), dim3(n_tokens), dim3(256), 0,   \
+                     stream, (const T*)qkv, positions, slots, q_norm_w, k_norm_w, inv_freq,      \
+                     (T*)q_out, (T*)kv_cache, nh, nkv, rot, adjacent, eps, page_size, write_kv)
+  switch (d) {
+    case 16: ZA_RK_LAUNCH(16); return true;
+    case 32: ZA_RK_LAUNCH(32); return true;
+    case 64: ZA_RK_LAUNCH(64); return true;
+    case 128: ZA_RK_LAUNCH(128); return true;
+    case 256: ZA_RK_LAUNCH(256); return true;
+    default: return false;
+  }
+#undef ZA_RK_LAUNCH
+}
+
 extern "C" int za_qk_norm_rope_kv_write(const void* qkv, const int* positions, const int* slots,
                                         const float* q_norm_w, const float* k_norm_w,
                                         const float* inv_freq, void* q_out, void* kv_cache,
@@ -99,6 +211,15 @@ extern "C" int za_qk_norm_rope_kv_write(const void* qkv, const int* positions, c
   if (d > RK_MAX_D || rot < 0 || rot > d || (rot % 2) != 0) return ZA_ERR_UNSUPPORTED;
   if (rot > 0 && !inv_freq) return ZA_ERR_ARG;
   if (write_kv && (!kv_cache || !slots || page_size <= 0)) return ZA_ERR_ARG;
+  if (dtype != 0 && dtype != 1) return ZA_ERR_UNSUPPORTED;
+  const bool fast =
+      dtype == 0 ? launch_pow2<float>(qkv, positions, slots, q_norm_w, k_norm_w, inv_freq, q_out,
+                                      kv_cache, n_tokens, nh, nkv, d, rot, adjacent, eps,
+                                      page_size, write_kv, stream)
+                 : launch_pow2<bf16_t>(qkv, positions, slots, q_norm_w, k_norm_w, inv_freq, q_out,
+                                       kv_cache, n_tokens, nh, nkv, d, rot, adjacent, eps,
+                                       page_size, write_kv, stream);
+  if (fast) return za_launch_status();
   dim3 grid(n_tokens, (nh + 2 * nkv + 3) / 4), block(256);
   if (dtype == 0) {
     hipLaunchKernelGGL((qk_norm_rope_kv_write_kernel<float>), grid, block, 0, stream,
