@@ -25,13 +25,17 @@ state ``slots[slot, floats]`` in 32-bit with one view per state entry.
 
 from __future__ import annotations
 
-from dataclasses import dataclass, field
-from typing import Dict, Hashable, List, Mapping, Optional, Tuple
+from dataclasses import dataclass
+from typing import Dict, Hashable, List, Mapping, Optional, Sequence, Tuple
 
+import ctypes
+
+import numpy as np
 import torch
 
+from ..kernels import host
 from ..parts.base import PagedNeed, StateNeed
-from .pages import OutOfPages, OutOfSlots, Pool, PoolError
+from .pages import OutOfPages, OutOfSlots, Pool, PoolError, raise_for
 
 FREED = -1   # block-table entry of a page that was given back (behind the window)
 
@@ -54,15 +58,6 @@ class PagedGroup:
 
 
 @dataclass
-class RequestCache:
-    slot: int
-    num_tokens: int = 0
-    tables: Dict[int, List[int]] = field(default_factory=dict)   # group index -> page ids
-    reserved: int = 0                                            # tokens the tables cover
-    serial: int = 0                                              # number of this admission
-
-
-@dataclass
 class CacheView:
     """What a mixer sees of the cache for one entry of the run order."""
     kind: str                      # "paged" | "state" | "none"
@@ -73,6 +68,9 @@ class CacheView:
 
 
 class CacheManager:
+    """Groups, tables and slots are kept by the host library; this class owns the
+    device memory, names the requests and translates failures into exceptions."""
+
     def __init__(self, needs: Mapping[int, object], page_size: int, num_pages, num_slots: int,
                  device: Optional[torch.device] = None, dtype: torch.dtype = torch.bfloat16,
                  allocate: bool = True):
@@ -84,9 +82,14 @@ class CacheManager:
         self.page_size = page_size
         self.device = device
         self.dtype = dtype
-        self.groups: List[PagedGroup] = []
+        self._lib = host.lib()
+        self.handles = host.Handles()
+        self._pinned: set = set()      # names a scheduler still knows: their handles are kept
         self._group_of: Dict[int, int] = {}
-        by_key: Dict[Tuple[int, int, int], PagedGroup] = {}
+        by_key: Dict[Tuple[int, int, int], int] = {}
+        group_needs: List[PagedNeed] = []
+        group_ids: List[List[int]] = []
+        group_pages: List[int] = []
         state_entries: List[Tuple[int, StateNeed]] = []
         for cid in sorted(needs):
             need = needs[cid]
@@ -96,16 +99,32 @@ class CacheManager:
                 key = (need.num_kv_heads, need.head_dim, need.window)
                 if key not in by_key:
                     count = num_pages[key] if isinstance(num_pages, Mapping) else int(num_pages)
-                    grp = PagedGroup(len(self.groups), need, [], Pool(count, "page"), page_size)
-                    by_key[key] = grp
-                    self.groups.append(grp)
-                by_key[key].cache_ids.append(cid)
-                self._group_of[cid] = by_key[key].index
+                    if count < 0:
+                        raise ValueError(f"a pool cannot have {count} pages")
+                    by_key[key] = len(group_needs)
+                    group_needs.append(need)
+                    group_ids.append([])
+                    group_pages.append(count)
+                group_ids[by_key[key]].append(cid)
+                self._group_of[cid] = by_key[key]
             elif isinstance(need, StateNeed):
                 state_entries.append((cid, need))
             else:
                 raise TypeError(f"cache need of entry {cid} is {need!r}")
-        self.slots = Pool(num_slots, "slot")
+        if num_slots < 0:
+            raise ValueError(f"a pool cannot have {num_slots} slots")
+        G = len(group_needs)
+        windows = (ctypes.c_int * max(G, 1))(*[n.window for n in group_needs])
+        pages = (ctypes.c_int * max(G, 1))(*group_pages)
+        self._ptr = self._lib.za_cache_new(G, windows, pages, int(page_size), int(num_slots))
+        if not self._ptr:
+            raise ValueError("the host library refused the cache's sizes")
+        self.groups: List[PagedGroup] = [
+            PagedGroup(g, group_needs[g], group_ids[g],
+                       Pool(0, "page", _attach=(self._lib.za_cache_pool(self._ptr, g), self.handles)),
+                       page_size)
+            for g in range(G)]
+        self.slots = Pool(0, "slot", _attach=(self._lib.za_cache_pool(self._ptr, -1), self.handles))
         self._state_layout: Dict[int, Tuple[int, Tuple[int, ...]]] = {}
         offset = 0
         for cid, need in state_entries:
@@ -126,10 +145,18 @@ class CacheManager:
             if self.floats_per_slot:
                 self.slot_memory = torch.zeros((num_slots, self.floats_per_slot),
                                                dtype=torch.float32, device=device)
-        self.requests: Dict[Hashable, RequestCache] = {}
-        self.pages_reused = 0
-        self._admissions = 0
-        self._ever_used: List[set] = [set() for _ in self.groups]
+        self._n_groups = G
+        self._scratch = (ctypes.c_int * max(G, 1))()
+
+    def __del__(self):
+        ptr, self._ptr = getattr(self, "_ptr", None), None
+        if ptr:
+            self._lib.za_cache_free(ptr)
+
+    @property
+    def native(self) -> int:
+        """The host library's object, for the scheduler and the step builder."""
+        return self._ptr
 
     # ------------------------------------------------------------------ views
     def view(self, cache_id: int, writes: bool = True) -> CacheView:
@@ -151,134 +178,141 @@ class CacheManager:
         return CacheView("none", writes=writes)
 
     # --------------------------------------------------------------- requests
+    def _info(self, req: Hashable):
+        h = self.handles.known(req)
+        out = (ctypes.c_longlong * 4)()
+        if h is None or not self._lib.za_cache_request(self._ptr, h, out):
+            raise KeyError(req)
+        return out
+
+    def __contains__(self, req: Hashable) -> bool:
+        h = self.handles.known(req)
+        out = (ctypes.c_longlong * 4)()
+        return h is not None and bool(self._lib.za_cache_request(self._ptr, h, out))
+
+    @property
+    def requests(self):
+        """The admitted requests' names (a container: ``in``, ``len``)."""
+        return _Admitted(self)
+
+    def pin(self, req: Hashable) -> int:
+        """Keep the request's handle until ``unpin`` (for a scheduler that knows the
+        request also while it is not admitted)."""
+        self._pinned.add(req)
+        return self.handles.of(req)
+
+    def unpin(self, req: Hashable) -> None:
+        self._pinned.discard(req)
+        if req not in self:
+            self.handles.drop(req)
+
     def admit(self, req: Hashable) -> int:
-        if req in self.requests:
-            raise PoolError(f"request {req!r} is already admitted")
-        slot = self.slots.take(req)
-        self._admissions += 1
-        self.requests[req] = RequestCache(slot, 0, {g.index: [] for g in self.groups}, 0,
-                                          self._admissions)
+        slot = ctypes.c_int()
+        raise_for(self._lib.za_cache_admit(self._ptr, self.handles.of(req), ctypes.byref(slot)))
         if self.slot_memory is not None:
-            self.slot_memory[slot].zero_()
-        return slot
+            self.slot_memory[slot.value].zero_()
+        return slot.value
+
+    def admitted_by_scheduler(self, req: Hashable) -> None:
+        """The host library's scheduler admitted ``req`` itself: clear its state."""
+        if self.slot_memory is not None:
+            self.slot_memory[self.slot_of(req)].zero_()
 
     def pages_needed(self, req: Hashable, n_new: int) -> Dict[int, int]:
-        rc = self.requests[req]
-        total = rc.num_tokens + n_new
-        want = (total + self.page_size - 1) // self.page_size
-        return {g.index: max(0, want - len(rc.tables[g.index])) for g in self.groups}
+        if req not in self:
+            raise KeyError(req)
+        raise_for(self._lib.za_cache_pages_needed(self._ptr, self.handles.of(req), int(n_new),
+                                                  self._scratch))
+        return {g: self._scratch[g] for g in range(self._n_groups)}
 
     def can_reserve(self, req: Hashable, n_new: int, spare: Optional[Dict[int, int]] = None) -> bool:
         """Whether ``reserve`` would succeed; ``spare`` (group -> pages) is
         subtracted from the free counts first (pages promised to others)."""
-        for gi, n in self.pages_needed(req, n_new).items():
-            free = self.groups[gi].pool.free_count - (spare or {}).get(gi, 0)
-            if n > free:
-                return False
-        return True
+        if req not in self:
+            raise KeyError(req)
+        sp = None
+        if spare:
+            sp = (ctypes.c_int * max(self._n_groups, 1))(
+                *[int(spare.get(g, 0)) for g in range(self._n_groups)])
+        ok = ctypes.c_int()
+        raise_for(self._lib.za_cache_can_reserve(self._ptr, self.handles.of(req), int(n_new), sp,
+                                                 ctypes.byref(ok)))
+        return bool(ok.value)
 
     def reserve(self, req: Hashable, n_new: int) -> None:
         """Make the request's tables cover ``n_new`` more tokens; all groups or none."""
-        rc = self.requests[req]
-        needed = self.pages_needed(req, n_new)
-        for gi, n in needed.items():
-            if n > self.groups[gi].pool.free_count:
-                raise OutOfPages(
-                    f"request {req!r} needs {n} pages of group {gi}, "
-                    f"{self.groups[gi].pool.free_count} of {self.groups[gi].pool.size} free")
-        for gi, n in needed.items():
-            pool = self.groups[gi].pool
-            for _ in range(n):
-                page = pool.take(req)
-                if page in self._ever_used[gi]:
-                    self.pages_reused += 1
-                self._ever_used[gi].add(page)
-                rc.tables[gi].append(page)
-        rc.reserved = max(rc.reserved, rc.num_tokens + n_new)
+        if req not in self:
+            raise KeyError(req)
+        raise_for(self._lib.za_cache_reserve(self._ptr, self.handles.of(req), int(n_new)))
 
     def commit(self, req: Hashable, n_new: int) -> None:
         """``n_new`` tokens were written; give back pages no later query can read."""
-        rc = self.requests[req]
-        if rc.num_tokens + n_new > rc.reserved:
-            raise PoolError(f"request {req!r} commits {n_new} tokens beyond its reservation")
-        rc.num_tokens += n_new
-        for grp in self.groups:
-            w = grp.need.window
-            if w <= 0:
-                continue
-            # The next query sits at position >= num_tokens and reads keys > position - w.
-            first_needed = rc.num_tokens - w + 1
-            if first_needed <= 0:
-                continue
-            table = rc.tables[grp.index]
-            for p in range(min(first_needed // self.page_size, len(table))):
-                if table[p] != FREED:
-                    grp.pool.give(table[p], req)
-                    table[p] = FREED
+        if req not in self:
+            raise KeyError(req)
+        raise_for(self._lib.za_cache_commit(self._ptr, self.handles.of(req), int(n_new)))
+
+    def reserve_many(self, reqs: Sequence[Hashable], counts: Sequence[int]) -> None:
+        """Pages for every entry of a step, all of them or none.  Raises ``KeyError``
+        for a request that is not admitted."""
+        h = np.empty((len(reqs),), dtype=np.int64)
+        for i, r in enumerate(reqs):
+            known = self.handles.known(r)
+            if known is None:
+                raise KeyError(r)
+            h[i] = known
+        c = np.asarray(counts, dtype=np.int32)
+        rc = self._lib.za_cache_reserve_many(self._ptr, len(reqs), h.ctypes.data, c.ctypes.data)
+        if rc == host.STEP:
+            raise KeyError(reqs[int(host.last_error().split()[1].rstrip(":"))])
+        raise_for(rc)
+
+    def commit_many(self, reqs: Sequence[Hashable], counts: Sequence[int]) -> None:
+        h = np.fromiter((self.handles.of(r) for r in reqs), dtype=np.int64, count=len(reqs))
+        c = np.asarray(counts, dtype=np.int32)
+        raise_for(self._lib.za_cache_commit_many(self._ptr, len(reqs), h.ctypes.data, c.ctypes.data))
 
     def release(self, req: Hashable) -> None:
-        rc = self.requests.pop(req)
-        for grp in self.groups:
-            for page in rc.tables[grp.index]:
-                if page != FREED:
-                    grp.pool.give(page, req)
-        self.slots.give(rc.slot, req)
+        if req not in self:
+            raise KeyError(req)
+        raise_for(self._lib.za_cache_release(self._ptr, self.handles.of(req)))
+        if req not in self._pinned:
+            self.handles.drop(req)
 
     # ------------------------------------------------------------- step inputs
     def slot_of(self, req: Hashable) -> int:
-        return self.requests[req].slot
+        return int(self._info(req)[0])
 
     def num_tokens(self, req: Hashable) -> int:
-        return self.requests[req].num_tokens
+        return int(self._info(req)[1])
 
     def serial_of(self, req: Hashable) -> int:
         """A number that differs between two admissions, also of the same id."""
-        return self.requests[req].serial
+        return int(self._info(req)[3])
 
     def table(self, req: Hashable, group: int) -> List[int]:
-        return self.requests[req].tables[group]
+        if req not in self:
+            raise KeyError(req)
+        h = self.handles.of(req)
+        n = self._lib.za_cache_table(self._ptr, h, int(group), None, 0)
+        if n < 0:
+            raise KeyError((req, group))
+        out = np.empty((max(n, 1),), dtype=np.int32)
+        self._lib.za_cache_table(self._ptr, h, int(group), out.ctypes.data, n)
+        return out[:n].tolist()
 
     def token_slots(self, req: Hashable, group: int, start: int, n: int) -> List[int]:
         """Physical places ``page * page_size + offset`` of positions start..start+n-1."""
-        table = self.requests[req].tables[group]
-        ps = self.page_size
-        out = []
-        for pos in range(start, start + n):
-            page = table[pos // ps]
-            if page == FREED:
-                raise PoolError(f"position {pos} of request {req!r} lies in a page given back")
-            out.append(page * ps + pos % ps)
-        return out
+        if req not in self:
+            raise KeyError(req)
+        out = np.empty((max(n, 1),), dtype=np.int32)
+        raise_for(self._lib.za_cache_token_slots(self._ptr, self.handles.of(req), int(group),
+                                                 int(start), int(n), out.ctypes.data))
+        return out[:n].tolist()
 
     # ------------------------------------------------------------------ checks
     def check(self) -> None:
         """No page lost, held twice or freed twice; tables agree with the pools."""
-        self.slots.check()
-        seen_slots = set()
-        for req, rc in self.requests.items():
-            if rc.slot in seen_slots:
-                raise PoolError(f"slot {rc.slot} held twice")
-            seen_slots.add(rc.slot)
-            if self.slots.owner_of(rc.slot) != req:
-                raise PoolError(f"slot {rc.slot} of {req!r} is owned by {self.slots.owner_of(rc.slot)!r}")
-        if len(seen_slots) != self.slots.used_count:
-            raise PoolError("slots in use do not match the admitted requests")
-        for grp in self.groups:
-            grp.pool.check()
-            held = set()
-            for req, rc in self.requests.items():
-                for page in rc.tables[grp.index]:
-                    if page == FREED:
-                        continue
-                    if page in held:
-                        raise PoolError(f"page {page} of group {grp.index} held twice")
-                    held.add(page)
-                    if grp.pool.owner_of(page) != req:
-                        raise PoolError(f"page {page} of {req!r} is owned by "
-                                        f"{grp.pool.owner_of(page)!r}")
-            if len(held) != grp.pool.used_count:
-                raise PoolError(f"group {grp.index}: {grp.pool.used_count} pages in use but "
-                                f"{len(held)} in tables (page lost)")
+        raise_for(self._lib.za_cache_check(self._ptr))
 
     def stats(self) -> dict:
         return {
@@ -290,3 +324,20 @@ class CacheManager:
             "slots_high_water": self.slots.high_water,
             "pages_reused": self.pages_reused, "requests": len(self.requests),
         }
+
+    @property
+    def pages_reused(self) -> int:
+        return int(self._lib.za_cache_pages_reused(self._ptr))
+
+
+class _Admitted:
+    """``cache.requests``: which names are admitted."""
+
+    def __init__(self, cache: "CacheManager"):
+        self._cache = cache
+
+    def __contains__(self, req: Hashable) -> bool:
+        return req in self._cache
+
+    def __len__(self) -> int:
+        return int(self._cache._lib.za_cache_num_requests(self._cache._ptr))

@@ -1,5 +1,6 @@
 """Pools of fixed-size things handed out and taken back: cache pages and state
-slots.  Pure bookkeeping, no device memory.
+slots.  Pure bookkeeping, no device memory; the free list and the owners live in
+the host library (``csrc/host.cpp``), this class is its Python face.
 
 The reference's allocator is a LIFO free list with reference counts, copy on
 write and a CPU swap (/root/reference/src/paged_attention/allocator.zig:19-118);
@@ -10,7 +11,10 @@ which makes "held twice" and "freed twice" detectable.
 
 from __future__ import annotations
 
+import ctypes
 from typing import Hashable, List, Optional
+
+from ..kernels import host
 
 
 class OutOfPages(RuntimeError):
@@ -25,72 +29,93 @@ class PoolError(RuntimeError):
     """A bookkeeping invariant was violated (double free, foreign page, ...)."""
 
 
+def raise_for(code: int) -> None:
+    """Turn a failure code of the host library into this package's exception."""
+    if code == host.OK:
+        return
+    msg = host.last_error()
+    if code == host.OUT_OF_PAGES:
+        raise OutOfPages(msg)
+    if code == host.OUT_OF_SLOTS:
+        raise OutOfSlots(msg)
+    if code == host.POOL:
+        raise PoolError(msg)
+    if code == host.ARG:
+        raise ValueError(msg)
+    raise RuntimeError(f"host library error {code}: {msg}")
+
+
 class Pool:
     """``size`` numbered items; ``take(owner)`` pops the most recently returned
     one, ``give(item, owner)`` returns it."""
 
-    def __init__(self, size: int, what: str = "page"):
-        if size < 0:
-            raise ValueError(f"a pool cannot have {size} {what}s")
-        self.size = size
+    def __init__(self, size: int, what: str = "page", _attach=None):
+        """``_attach``: ``(pointer, handles)`` of a pool that a cache owns."""
         self.what = what
-        self._free: List[int] = list(range(size - 1, -1, -1))   # pop() yields 0 first
-        self._owner: List[Optional[Hashable]] = [None] * size
-        self.high_water = 0
-        self.total_taken = 0
+        self._lib = host.lib()
+        if _attach is not None:
+            self._ptr, self._handles = _attach
+            self._own = False
+        else:
+            if size < 0:
+                raise ValueError(f"a pool cannot have {size} {what}s")
+            self._ptr = self._lib.za_pool_new(int(size), 1 if what == "page" else 0)
+            self._handles = host.Handles()
+            self._own = True
+        self.size = self._stats()[0]
+
+    def __del__(self):
+        if getattr(self, "_own", False) and self._ptr:
+            self._lib.za_pool_free(self._ptr)
+            self._ptr = None
+
+    def _stats(self):
+        out = (ctypes.c_longlong * 4)()
+        self._lib.za_pool_stats(self._ptr, out)
+        return list(out)
 
     @property
     def free_count(self) -> int:
-        return len(self._free)
+        return self._stats()[1]
 
     @property
     def used_count(self) -> int:
-        return self.size - len(self._free)
+        s = self._stats()
+        return s[0] - s[1]
+
+    @property
+    def high_water(self) -> int:
+        return self._stats()[2]
+
+    @property
+    def total_taken(self) -> int:
+        return self._stats()[3]
 
     def take(self, owner: Hashable) -> int:
         if owner is None:
             raise PoolError("an owner is needed")
-        if not self._free:
-            raise (OutOfPages if self.what == "page" else OutOfSlots)(
-                f"no free {self.what} (all {self.size} in use)")
-        item = self._free.pop()
-        if self._owner[item] is not None:
-            raise PoolError(f"{self.what} {item} was on the free list while owned by "
-                            f"{self._owner[item]!r}")
-        self._owner[item] = owner
-        self.total_taken += 1
-        self.high_water = max(self.high_water, self.used_count)
-        return item
+        item = ctypes.c_int()
+        raise_for(self._lib.za_pool_take(self._ptr, self._handles.of(owner), ctypes.byref(item)))
+        return item.value
 
     def take_many(self, owner: Hashable, n: int) -> List[int]:
         """All ``n`` or none."""
-        if n > len(self._free):
-            raise (OutOfPages if self.what == "page" else OutOfSlots)(
-                f"{n} {self.what}s wanted, {len(self._free)} of {self.size} free")
-        return [self.take(owner) for _ in range(n)]
+        if owner is None:
+            raise PoolError("an owner is needed")
+        items = (ctypes.c_int * max(n, 1))()
+        raise_for(self._lib.za_pool_take_many(self._ptr, self._handles.of(owner), int(n), items))
+        return list(items[:n])
 
     def give(self, item: int, owner: Hashable) -> None:
-        if not 0 <= item < self.size:
-            raise PoolError(f"{self.what} {item} does not exist")
-        if self._owner[item] is None:
-            raise PoolError(f"{self.what} {item} freed twice")
-        if self._owner[item] != owner:
-            raise PoolError(f"{self.what} {item} belongs to {self._owner[item]!r}, not {owner!r}")
-        self._owner[item] = None
-        self._free.append(item)
+        known = self._handles.known(owner)
+        raise_for(self._lib.za_pool_give(self._ptr, int(item), known if known is not None else 0))
 
     def owner_of(self, item: int) -> Optional[Hashable]:
-        return self._owner[item]
+        owner = ctypes.c_int64()
+        if self._lib.za_pool_owner(self._ptr, int(item), ctypes.byref(owner)) == 1:
+            return self._handles.name(owner.value)
+        return None
 
     def check(self) -> None:
         """Every item is either free exactly once or owned, never both."""
-        seen = set()
-        for item in self._free:
-            if item in seen:
-                raise PoolError(f"{self.what} {item} is on the free list twice")
-            seen.add(item)
-            if self._owner[item] is not None:
-                raise PoolError(f"{self.what} {item} is free and owned")
-        owned = sum(1 for o in self._owner if o is not None)
-        if owned + len(self._free) != self.size:
-            raise PoolError(f"{owned} owned + {len(self._free)} free != {self.size} {self.what}s")
+        raise_for(self._lib.za_pool_check(self._ptr))

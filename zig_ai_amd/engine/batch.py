@@ -5,7 +5,8 @@ A step packs the new tokens of all its requests into one row sequence
 ``[T]``: request 0's tokens, then request 1's, and so on.  A request contributes
 a portion of its prompt (one token or many) or one decoded token; the model does
 not distinguish the two.  Every integer array the kernels need is laid out in
-ONE host buffer and copied to the device in one transfer.
+ONE host buffer (filled by the host library, ``csrc/host.cpp``) and copied to the
+device in one transfer.
 """
 
 from __future__ import annotations
@@ -17,6 +18,8 @@ import numpy as np
 import torch
 
 from ..cache.manager import FREED, CacheManager
+from ..cache.pages import raise_for
+from ..kernels import host as hostlib
 
 
 class StepError(ValueError):
@@ -83,10 +86,73 @@ def _make_items(seq_lens: Sequence[int], rows_per_item: int):
     return seq, row0, cnt
 
 
+class PreparedEntries:
+    """The entries of a step as the arrays the host library reads."""
+
+    def __init__(self, entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int):
+        if not entries:
+            raise StepError("a step needs at least one entry")
+        S = len(entries)
+        self.entries = entries
+        self.reqs = np.empty((S,), dtype=np.int64)
+        self.counts = np.empty((S,), dtype=np.int32)
+        self.want_counts = np.empty((S,), dtype=np.int32)
+        handles = cache.handles
+        for s, e in enumerate(entries):
+            h = handles.known(e.request)
+            if h is None:
+                raise StepError(f"request {e.request!r} is not admitted")
+            self.reqs[s] = h
+            self.counts[s] = len(e.tokens)
+            self.want_counts[s] = len(e.want)
+        try:
+            tokens = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64,
+                                 count=int(self.counts.sum()))
+            wants = np.fromiter((w for e in entries for w in e.want), dtype=np.int64,
+                                count=int(self.want_counts.sum()))
+        except (TypeError, ValueError, OverflowError) as err:
+            raise StepError(f"token ids and wanted places must be integers: {err}") from err
+        if tokens.size and (tokens.min() < 0 or tokens.max() >= vocab_size):
+            bad = int(tokens[(tokens < 0) | (tokens >= vocab_size)][0])
+            raise StepError(f"token id {bad} is outside the vocabulary of {vocab_size}")
+        self.tokens = tokens.astype(np.int32)
+        self.wants = np.clip(wants, -1, 2 ** 31 - 1).astype(np.int32)
+        self.vocab_size = int(vocab_size)
+        self.ctx = np.empty((S,), dtype=np.int32)
+        self.slots = np.empty((S,), dtype=np.int32)
+        self.meta = np.zeros((6,), dtype=np.int64)
+
+    def build(self, cache: CacheManager, grans: np.ndarray, max_position: int, min_pages: int,
+              sections: np.ndarray, out_ptr, cap: int) -> None:
+        """One call of the host library: with ``out_ptr`` None only the sizes."""
+        rc = hostlib.lib().za_step_build(
+            cache.native, len(self.entries), self.reqs.ctypes.data, self.counts.ctypes.data,
+            self.tokens.ctypes.data, self.want_counts.ctypes.data, self.wants.ctypes.data,
+            self.vocab_size, len(grans), grans.ctypes.data, int(max_position), int(min_pages),
+            out_ptr, cap, sections.ctypes.data, self.meta.ctypes.data, self.ctx.ctypes.data,
+            self.slots.ctypes.data)
+        if rc == hostlib.STEP:
+            msg = hostlib.last_error()
+            if msg.startswith("entry "):        # name the request instead of its place
+                place = int(msg.split()[1].rstrip(":"))
+                msg = f"request {self.entries[place].request!r}: " + msg.split(" ", 2)[2]
+            raise StepError(msg)
+        raise_for(rc)
+
+    def extent(self, cache: CacheManager) -> Tuple[int, int]:
+        """(pages of the longest block table, longest context including the new
+        tokens) among the entries."""
+        self.build(cache, np.zeros((0,), dtype=np.int32), 0, 0,
+                   np.zeros((2 * (7 + 2 * len(cache.groups)),), dtype=np.int64), None, 0)
+        return int(self.meta[3]), int(self.meta[4])
+
+
 def build_step(entries: Sequence[StepEntry], cache: CacheManager, device: torch.device,
                vocab_size: int, item_granularities: Sequence[int] = (),
                max_position: int = 0, min_pages: int = 0, max_keys: int = 0,
-               into: Optional[torch.Tensor] = None) -> StepContext:
+               into: Optional[torch.Tensor] = None,
+               staging: Optional[torch.Tensor] = None,
+               prepared: Optional[PreparedEntries] = None) -> StepContext:
     """Lay out the step.  Every request must be admitted and its pages for this
     step reserved beforehand; nothing is committed here.
 
@@ -94,89 +160,40 @@ def build_step(entries: Sequence[StepEntry], cache: CacheManager, device: torch.
     the block tables) only.  ``min_pages`` widens the block tables, ``max_keys``
     overrides the context length used for planning, and ``into`` is a device
     buffer to fill instead of a new one: together they let a replayed HIP graph
-    find every array at the address it was captured with."""
-    if not entries:
-        raise StepError("a step needs at least one entry")
-    seen = set()
-    seq_lens, ctx_lens, slots = [], [], []
-    for e in entries:
-        if e.request in seen:
-            raise StepError(f"request {e.request!r} appears twice in one step")
-        seen.add(e.request)
-        n = len(e.tokens)
-        if n == 0:
-            raise StepError(f"request {e.request!r} brings no tokens")
-        for t in e.tokens:
-            if not 0 <= int(t) < vocab_size:
-                raise StepError(f"token id {t} of request {e.request!r} is outside the "
-                                f"vocabulary of {vocab_size}")
-        for w in e.want:
-            if not 0 <= int(w) < n:
-                raise StepError(f"request {e.request!r} wants logits at place {w} of {n} tokens")
-        ctx = cache.num_tokens(e.request)
-        if max_position and ctx + n > max_position:
-            raise StepError(f"request {e.request!r} would reach position {ctx + n - 1}, beyond "
-                            f"max_position_embeddings {max_position}")
-        seq_lens.append(n)
-        ctx_lens.append(ctx)
-        slots.append(cache.slot_of(e.request))
-    T, S = sum(seq_lens), len(entries)
-    R = sum(len(e.want) for e in entries)
+    find every array at the address it was captured with.  ``staging`` is a pinned
+    host buffer to lay the step out in, from which ``into`` is filled by a copy
+    that does not block; the caller waits for that copy before it lays out the
+    next step there.  ``prepared``: the same entries, already turned into arrays."""
+    prep = prepared if prepared is not None else PreparedEntries(entries, cache, vocab_size)
+    S = len(entries)
+    counts, meta = prep.counts, prep.meta
+    grans = np.asarray(sorted(set(int(g) for g in item_granularities)), dtype=np.int32)
     groups = cache.groups
-    max_pages = 1
-    for e in entries:
-        for g in groups:
-            max_pages = max(max_pages, len(cache.table(e.request, g.index)))
-    max_pages = max(max_pages, min_pages)
+    n_sections = 7 + 2 * len(groups) + 3 * len(grans)
+    sections = np.zeros((2 * n_sections,), dtype=np.int64)
+    ctx_arr, slot_arr = prep.ctx, prep.slots
 
-    sections: List[Tuple[str, int]] = [
-        ("token_ids", T), ("positions", T), ("token_seq", T), ("seq_start", S + 1),
-        ("ctx_len", S), ("slot_id", S), ("logit_rows", R)]
+    def call(out_ptr, cap):
+        prep.build(cache, grans, max_position, min_pages, sections, out_ptr, cap)
+
+    call(None, 0)                               # sizes first, then the buffer itself
+    if staging is not None:
+        if staging.numel() < int(meta[5]) or staging.dtype != torch.int32:
+            raise StepError(f"the step needs {int(meta[5])} int32 entries, the staging buffer "
+                            f"holds {staging.numel()}")
+        host = staging.numpy()[:int(meta[5])]
+    else:
+        host = np.empty((int(meta[5]),), dtype=np.int32)
+    call(host.ctypes.data, host.size)
+    T, R, max_pages = int(meta[0]), int(meta[2]), int(meta[3])
+    names = ["token_ids", "positions", "token_seq", "seq_start", "ctx_len", "slot_id", "logit_rows"]
     for g in groups:
-        sections.append((f"slots{g.index}", T))
-        sections.append((f"table{g.index}", S * max_pages))
-    item_lists = {}
-    for gran in sorted(set(item_granularities)):
-        item_lists[gran] = _make_items(seq_lens, gran)
-        w = len(item_lists[gran][0])
-        sections += [(f"iseq{gran}", w), (f"irow{gran}", w), (f"icnt{gran}", w)]
-    offsets, total = {}, 0
-    for name, n in sections:
-        offsets[name] = (total, n)
-        total += (n + 3) // 4 * 4          # keep every section 16-byte aligned
-    host = np.full((max(total, 4),), FREED, dtype=np.int32)
-
-    def put(name: str, values) -> None:
-        off, n = offsets[name]
-        host[off:off + n] = values
-
-    row = 0
-    starts, logit_rows = [0], []
-    for s, e in enumerate(entries):
-        n = seq_lens[s]
-        a, b = offsets["token_ids"][0] + row, offsets["token_ids"][0] + row + n
-        host[a:b] = np.asarray(e.tokens, dtype=np.int32)
-        a = offsets["positions"][0] + row
-        host[a:a + n] = np.arange(ctx_lens[s], ctx_lens[s] + n, dtype=np.int32)
-        a = offsets["token_seq"][0] + row
-        host[a:a + n] = s
-        logit_rows += [row + int(w) for w in e.want]
-        for g in groups:
-            a = offsets[f"slots{g.index}"][0] + row
-            host[a:a + n] = cache.token_slots(e.request, g.index, ctx_lens[s], n)
-            table = cache.table(e.request, g.index)
-            a = offsets[f"table{g.index}"][0] + s * max_pages
-            host[a:a + len(table)] = table
-        row += n
-        starts.append(row)
-    put("seq_start", starts)
-    put("ctx_len", ctx_lens)
-    put("slot_id", slots)
-    put("logit_rows", logit_rows)
-    for gran, (seq, row0, cnt) in item_lists.items():
-        put(f"iseq{gran}", seq)
-        put(f"irow{gran}", row0)
-        put(f"icnt{gran}", cnt)
+        names += [f"slots{g.index}", f"table{g.index}"]
+    for gran in grans.tolist():
+        names += [f"iseq{gran}", f"irow{gran}", f"icnt{gran}"]
+    offsets = {name: (int(sections[2 * i]), int(sections[2 * i + 1])) for i, name in enumerate(names)}
+    seq_lens, ctx_lens, slots = counts.tolist(), ctx_arr.tolist(), slot_arr.tolist()
+    item_lists = {gran: offsets[f"iseq{gran}"][1] for gran in grans.tolist()}
 
     if into is None:
         dev = torch.from_numpy(host).to(device)
@@ -185,7 +202,10 @@ def build_step(entries: Sequence[StepEntry], cache: CacheManager, device: torch.
             raise StepError(f"the step needs {host.size} int32 entries, the buffer holds "
                             f"{into.numel()}")
         dev = into
-        dev[:host.size].copy_(torch.from_numpy(host))
+        if staging is not None:
+            dev[:host.size].copy_(staging[:host.size], non_blocking=True)
+        else:
+            dev[:host.size].copy_(torch.from_numpy(host))
 
     def view(name: str) -> torch.Tensor:
         off, n = offsets[name]
@@ -193,7 +213,7 @@ def build_step(entries: Sequence[StepEntry], cache: CacheManager, device: torch.
 
     ctx = StepContext(
         n_tokens=T, n_seqs=S, n_logit_rows=R,
-        max_keys=max(max_keys, max(c + n for c, n in zip(ctx_lens, seq_lens))),
+        max_keys=max(max_keys, int(meta[4])),
         token_ids=view("token_ids"), positions=view("positions"), token_seq=view("token_seq"),
         seq_start=view("seq_start"), ctx_len=view("ctx_len"), slot_id=view("slot_id"),
         logit_rows=view("logit_rows"),
@@ -202,6 +222,6 @@ def build_step(entries: Sequence[StepEntry], cache: CacheManager, device: torch.
     for g in groups:
         ctx.slot_mapping[g.index] = view(f"slots{g.index}")
         ctx.block_tables[g.index] = view(f"table{g.index}").view(S, max_pages)
-    for gran, (seq, _, _) in item_lists.items():
-        ctx.items[gran] = (view(f"iseq{gran}"), view(f"irow{gran}"), view(f"icnt{gran}"), len(seq))
+    for gran, n_items in item_lists.items():
+        ctx.items[gran] = (view(f"iseq{gran}"), view(f"irow{gran}"), view(f"icnt{gran}"), n_items)
     return ctx

@@ -13,7 +13,7 @@ from typing import Dict, Hashable, List, Optional, Sequence
 
 import torch
 
-from ..sampling.sampler import SamplingParams, UniformStream, sample_rows
+from ..sampling.sampler import SamplingParams, sample_rows, uniforms
 from .batch import StepEntry
 from .model import DecoderModel
 from .runner import ModelRunner
@@ -38,7 +38,6 @@ class Engine:
         self.runner = ModelRunner(self.model, page_size, num_pages, max_num_seqs)
         self.scheduler = Scheduler(self.runner.cache, max_num_seqs, max_num_batched_tokens,
                                    chunk_size, limit)
-        self._streams: Dict[Hashable, UniformStream] = {}
         self._next_id = 0
         self.timings = {"steps": 0, "step_seconds": 0.0, "tokens_run": 0, "tokens_generated": 0}
 
@@ -60,7 +59,6 @@ class Engine:
         req = Request(request_id, prompt, max_new_tokens, sampling or SamplingParams(),
                       eos_token_id)
         self.scheduler.add(req)
-        self._streams[req.id] = UniformStream(req.sampling.seed, req.number)
         return req
 
     def step(self) -> List[Request]:
@@ -71,17 +69,17 @@ class Engine:
         start = time.perf_counter()
         entries = []
         for e in plan:
-            tokens = e.request.tokens[e.start:e.start + e.count]
-            entries.append(StepEntry(e.request.id, tokens, [e.count - 1] if e.samples else []))
+            entries.append(StepEntry(e.request.id, e.request.span(e.start, e.count),
+                                     [e.count - 1] if e.samples else []))
         logits = self.runner.step(entries)
         sampling = [e for e in plan if e.samples]
         drawn = sample_rows(
             logits, [e.request.sampling for e in sampling],
-            [self._streams[e.request.id].at(len(e.request.output)) for e in sampling],
+            uniforms([e.request.sampling.seed for e in sampling],
+                     [e.request.number for e in sampling],
+                     [len(e.request.output) for e in sampling]),
             [e.request.output for e in sampling])
         done = self.scheduler.update(plan, {e.request.id: t for e, t in zip(sampling, drawn)})
-        for req in done:
-            self._streams.pop(req.id, None)
         self.timings["steps"] += 1
         self.timings["step_seconds"] += time.perf_counter() - start
         self.timings["tokens_run"] += sum(e.count for e in plan)

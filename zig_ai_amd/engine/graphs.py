@@ -22,9 +22,12 @@ from __future__ import annotations
 import gc
 from typing import Dict, Sequence, Tuple
 
+import numpy as np
 import torch
 
-from .batch import StepEntry, StepError, build_step
+from ..cache.pages import raise_for
+from ..kernels import host as hostlib
+from .batch import PreparedEntries, StepEntry, StepError, build_step
 
 PAGE_BUCKET = 64        # block-table width is rounded up to a multiple of this
 KEYS_BUCKET = 1024      # and the longest context to a multiple of this
@@ -45,44 +48,108 @@ class DecodeGraphs:
         self._granularities = tuple(item_granularities)
         self._max_position = max_position
         self.entries: Dict[Tuple[int, int, int], dict] = {}
+        self._arrays: Dict[int, dict] = {}       # per number of entries: arrays for the library
+        self._lib = hostlib.lib()
         self.captures = 0
         self.replays = 0
 
+    def _scratch(self, S: int) -> dict:
+        sc = self._arrays.get(S)
+        if sc is None:
+            sc = {"reqs": np.empty((S,), dtype=np.int64), "toks": np.empty((S,), dtype=np.int32),
+                  "ones": np.ones((S,), dtype=np.int32), "zeros": np.zeros((S,), dtype=np.int32),
+                  "ctx": np.empty((S,), dtype=np.int32), "slots": np.empty((S,), dtype=np.int32),
+                  "meta": np.zeros((6,), dtype=np.int64), "extent": np.zeros((2,), dtype=np.int64)}
+            sc["ptr"] = {k: v.ctypes.data for k, v in sc.items()}
+            self._arrays[S] = sc
+        return sc
+
+    @staticmethod
+    def _raise(rc: int, entries: Sequence[StepEntry]) -> None:
+        if rc == hostlib.STEP:
+            msg = hostlib.last_error()
+            if msg.startswith("entry "):        # name the request instead of its place
+                place = int(msg.split()[1].rstrip(":"))
+                msg = f"request {entries[place].request!r}: " + msg.split(" ", 2)[2]
+            raise StepError(msg)
+        raise_for(rc)
+
     def run(self, runner, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Logits ``[len(entries), vocab]`` of a step of single tokens (one row per
-        entry, whatever the entries want).  Pages must be reserved already."""
-        cache, model = runner.cache, runner.model
+        entry, whatever the entries want).  Takes the pages the new tokens need (all
+        or none: ``OutOfPages`` leaves everything as it was)."""
+        cache = runner.cache
         S = len(entries)
-        widest = max((len(cache.table(e.request, g.index)) for e in entries for g in cache.groups),
-                     default=1)
-        longest = max(cache.num_tokens(e.request) + 1 for e in entries)
+        sc = self._scratch(S)
+        ptr = sc["ptr"]
+        known = cache.handles.known
+        reqs, toks = sc["reqs"], sc["toks"]
+        for i, e in enumerate(entries):
+            h = known(e.request)
+            if h is None:
+                raise StepError(f"request {e.request!r} was not admitted")
+            reqs[i] = h
+            try:
+                toks[i] = e.tokens[0]
+            except (OverflowError, TypeError, ValueError):
+                raise StepError(f"token id {e.tokens[0]!r} of request {e.request!r} is outside "
+                                f"the vocabulary of {self._vocab}") from None
+        lib = self._lib
+        rc = lib.za_decode_prepare(cache.native, S, ptr["reqs"], ptr["toks"], self._vocab,
+                                   self._max_position, ptr["extent"])
+        if rc:
+            self._raise(rc, entries)
+        widest, longest = int(sc["extent"][0]), int(sc["extent"][1])
         key = (S, _round_up(widest, PAGE_BUCKET), _round_up(longest, KEYS_BUCKET))
         slot = self.entries.get(key)
         if slot is not None and slot["graph"] is not None:
-            self._refill(slot, cache, entries, key)
+            # Bring the persistent integer buffer up to date: the host library lays the
+            # step out in the pinned staging buffer, and one copy that does not block
+            # takes it to the device.  The layout equals the captured one because it
+            # depends only on the number of entries and the table width.
+            if slot["copied"] is not None:
+                slot["copied"].synchronize()    # the last transfer out of the staging buffer
+            pinned = slot["pinned"]
+            rc = lib.za_step_build(cache.native, S, ptr["reqs"], ptr["ones"], ptr["toks"],
+                                   ptr["ones"], ptr["zeros"], self._vocab, len(slot["grans"]),
+                                   slot["grans_ptr"], self._max_position, key[1], slot["pinned_ptr"],
+                                   slot["words"], slot["sections_ptr"], ptr["meta"], ptr["ctx"],
+                                   ptr["slots"])
+            if rc:
+                self._raise(rc, entries)
+            if int(sc["meta"][5]) != slot["words"]:
+                raise StepError(f"the step's layout has {int(sc['meta'][5])} entries, the "
+                                f"recorded one {slot['words']}")
+            slot["buffer"].copy_(pinned, non_blocking=True)
+            if slot["copied"] is None:
+                slot["copied"] = torch.cuda.Event()
+            slot["copied"].record()
             slot["graph"].replay()
             self.replays += 1
             return slot["logits"]
+        model = runner.model
         asked = [StepEntry(e.request, e.tokens, [0]) for e in entries]
+        prepared = PreparedEntries(asked, cache, self._vocab)
         if slot is None:
             # size the persistent buffer with a dry layout on the host
-            probe = build_step(asked, cache, torch.device("cpu"), model.spec.vocab_size,
-                               model.item_granularities, model.spec.max_position,
-                               min_pages=key[1], max_keys=key[2])
+            probe = build_step(asked, cache, torch.device("cpu"), self._vocab,
+                               self._granularities, self._max_position,
+                               min_pages=key[1], max_keys=key[2], prepared=prepared)
             words = probe.host.size
+            grans = np.asarray(sorted(set(int(g) for g in self._granularities)), dtype=np.int32)
             slot = {"buffer": torch.full((words,), -1, dtype=torch.int32, device=runner.device),
                     "pinned": torch.empty((words,), dtype=torch.int32, pin_memory=True),
-                    "graph": None, "logits": None, "requests": None}
+                    "graph": None, "logits": None, "copied": None, "words": words,
+                    "grans": grans,
+                    "sections": np.zeros((2 * (7 + 2 * len(cache.groups) + 3 * len(grans)),),
+                                         dtype=np.int64)}
+            slot["grans_ptr"] = grans.ctypes.data
+            slot["sections_ptr"] = slot["sections"].ctypes.data
+            slot["pinned_ptr"] = slot["pinned"].data_ptr()
             self.entries[key] = slot
-        ctx = build_step(asked, cache, runner.device, model.spec.vocab_size,
-                         model.item_granularities, model.spec.max_position,
-                         min_pages=key[1], max_keys=key[2], into=slot["buffer"])
-        # keep the host image: later steps of the same requests only patch it
-        slot["pinned"].numpy()[:] = ctx.host
-        slot["offsets"] = ctx.offsets
-        slot["requests"] = tuple(cache.serial_of(e.request) for e in entries)
-        slot["table_lens"] = [[len(cache.table(e.request, g.index)) for g in cache.groups]
-                              for e in entries]
+        ctx = build_step(asked, cache, runner.device, self._vocab, self._granularities,
+                         self._max_position, min_pages=key[1], max_keys=key[2],
+                         into=slot["buffer"], prepared=prepared)
         logits = model.forward(ctx, runner.views)          # this step, eagerly
         graph = torch.cuda.CUDAGraph()
         # No collection while the capture is open: a collector run could free
@@ -98,63 +165,3 @@ class DecodeGraphs:
         slot["graph"] = graph
         self.captures += 1
         return logits
-
-    def _refill(self, slot: dict, cache, entries: Sequence[StepEntry], key) -> None:
-        """Bring the persistent integer buffer up to date for this step.  When the
-        step holds the same requests in the same order as the last one that used
-        this graph, only what a decoded token changes is patched: token ids,
-        positions, the new tokens' places, and block-table entries that were added."""
-        if slot.get("copied") is not None:
-            slot["copied"].synchronize()        # the last transfer out of the staging buffer
-        host = slot["pinned"].numpy()
-        off = slot["offsets"]
-        admissions = tuple(cache.serial_of(e.request) for e in entries)
-        requests = tuple(e.request for e in entries)
-        S = len(entries)
-        vocab = self._vocab
-        for e in entries:
-            t = int(e.tokens[0])
-            if not 0 <= t < vocab:
-                raise StepError(f"token id {t} of request {e.request!r} is outside the "
-                                f"vocabulary of {vocab}")
-        if admissions != slot["requests"]:
-            asked = [StepEntry(e.request, e.tokens, [0]) for e in entries]
-            fresh = build_step(asked, cache, torch.device("cpu"), vocab, self._granularities,
-                               self._max_position, min_pages=key[1], max_keys=key[2])
-            host[:] = fresh.host
-            slot["requests"] = admissions
-            slot["table_lens"] = [[len(cache.table(e.request, g.index)) for g in cache.groups]
-                                  for e in entries]
-        else:
-            ctxs = [cache.num_tokens(r) for r in requests]
-            if self._max_position and max(ctxs) + 1 > self._max_position:
-                raise StepError(f"a request would reach position {max(ctxs)}, beyond "
-                                f"max_position_embeddings {self._max_position}")
-            a = off["token_ids"][0]
-            host[a:a + S] = [int(e.tokens[0]) for e in entries]
-            a = off["positions"][0]
-            host[a:a + S] = ctxs
-            a = off["ctx_len"][0]
-            host[a:a + S] = ctxs
-            ps = cache.page_size
-            width = key[1]
-            for gi, g in enumerate(cache.groups):
-                sa = off[f"slots{g.index}"][0]
-                ta = off[f"table{g.index}"][0]
-                for s, r in enumerate(requests):
-                    table = cache.table(r, g.index)
-                    c = ctxs[s]
-                    host[sa + s] = table[c // ps] * ps + c % ps
-                    known = slot["table_lens"][s][gi]
-                    if len(table) != known:
-                        host[ta + s * width + known: ta + s * width + len(table)] = table[known:]
-                        slot["table_lens"][s][gi] = len(table)
-                    if g.need.window > 0:
-                        # pages behind the window were given back: mark them
-                        first = max(0, (c - g.need.window + 1) // ps)
-                        if first:
-                            host[ta + s * width: ta + s * width + first] = table[:first]
-        slot["buffer"].copy_(slot["pinned"], non_blocking=True)
-        if slot.get("copied") is None:
-            slot["copied"] = torch.cuda.Event()
-        slot["copied"].record()

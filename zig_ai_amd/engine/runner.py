@@ -51,19 +51,10 @@ class ModelRunner:
     # --------------------------------------------------------------------- step
     def reserve(self, entries: Sequence[StepEntry]) -> None:
         """Pages for every entry of the step, all of them or none."""
-        wanted = {}
-        for e in entries:
-            if e.request not in self.cache.requests:
-                raise StepError(f"request {e.request!r} was not admitted")
-            for gi, n in self.cache.pages_needed(e.request, len(e.tokens)).items():
-                wanted[gi] = wanted.get(gi, 0) + n
-        for gi, n in wanted.items():
-            pool = self.cache.groups[gi].pool
-            if n > pool.free_count:
-                raise OutOfPages(f"the step needs {n} pages of group {gi}, "
-                                 f"{pool.free_count} of {pool.size} are free")
-        for e in entries:
-            self.cache.reserve(e.request, len(e.tokens))
+        try:
+            self.cache.reserve_many([e.request for e in entries], [len(e.tokens) for e in entries])
+        except KeyError as err:
+            raise StepError(f"request {err.args[0]!r} was not admitted") from None
 
     def prepare(self, entries: Sequence[StepEntry]) -> StepContext:
         """Reserve pages for the entries and lay out the step."""
@@ -79,13 +70,11 @@ class ModelRunner:
         else:
             ctx = self.prepare(entries)
             logits = self.model.forward(ctx, self.views)
-        for e in entries:
-            self.cache.commit(e.request, len(e.tokens))
+        self.cache.commit_many([e.request for e in entries], [len(e.tokens) for e in entries])
         self.steps_run += 1
         return logits
 
     def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        self.reserve(entries)
         for e in entries:
             for w in e.want:
                 if int(w) != 0:

@@ -27,12 +27,15 @@ Different by design:
 
 from __future__ import annotations
 
-from collections import deque
+import ctypes
 from dataclasses import dataclass, field
-from typing import Deque, Dict, Hashable, List, Optional, Sequence
+from typing import Dict, Hashable, List, Optional, Sequence
+
+import numpy as np
 
 from ..cache.manager import CacheManager
-from ..cache.pages import OutOfPages
+from ..cache.pages import OutOfPages, raise_for  # noqa: F401  (OutOfPages: what schedule() raises)
+from ..kernels import host as hostlib
 from ..sampling.sampler import SamplingParams
 
 WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
@@ -56,6 +59,15 @@ class Request:
     def tokens(self) -> List[int]:
         return self.prompt + self.output
 
+    def span(self, start: int, count: int) -> List[int]:
+        """``tokens[start:start + count]`` without joining the two lists."""
+        n = len(self.prompt)
+        if start >= n:
+            return self.output[start - n:start - n + count]
+        if start + count <= n:
+            return self.prompt[start:start + count]
+        return self.prompt[start:] + self.output[:start + count - n]
+
     @property
     def remaining(self) -> int:
         return len(self.prompt) + len(self.output) - self.num_computed
@@ -70,6 +82,13 @@ class ScheduledEntry:
 
 
 class Scheduler:
+    """The decisions are taken by the host library (``csrc/host.cpp``), which keeps
+    each request's counters; this class keeps the ``Request`` objects (with their
+    tokens) and mirrors the counters into them after every call."""
+
+    _PHASES = (WAITING, RUNNING, FINISHED)
+    _REASONS = (None, "eos", "length", "max_model_len")
+
     def __init__(self, cache: CacheManager, max_num_seqs: int = 64,
                  max_num_batched_tokens: int = 2048, chunk_size: int = 512,
                  max_model_len: int = 0):
@@ -80,11 +99,28 @@ class Scheduler:
         self.max_num_batched_tokens = max_num_batched_tokens
         self.chunk_size = chunk_size
         self.max_model_len = max_model_len
-        self.waiting: Deque[Request] = deque()
-        self.running: List[Request] = []
+        self._lib = hostlib.lib()
+        self._ptr = self._lib.za_sched_new(cache.native, int(max_num_seqs),
+                                           int(max_num_batched_tokens), int(chunk_size),
+                                           int(max_model_len or 0))
+        if not self._ptr:
+            raise ValueError("the host library refused the scheduler's limits")
+        self._requests: Dict[int, Request] = {}       # handle -> request, until forgotten
         self.finished: List[Request] = []
-        self._arrivals = 0
-        self.preemption_count = 0
+        cap = max(max_num_seqs, 1) + 1
+        self._cap = cap
+        self._ids = np.empty((cap,), dtype=np.int64)
+        self._starts = np.empty((cap,), dtype=np.int32)
+        self._counts = np.empty((cap,), dtype=np.int32)
+        self._samples = np.empty((cap,), dtype=np.int32)
+        self._tokens = np.empty((cap,), dtype=np.int32)
+        self._victims = np.empty((cap,), dtype=np.int64)
+        self._reasons = np.empty((cap,), dtype=np.int32)
+
+    def __del__(self):
+        ptr, self._ptr = getattr(self, "_ptr", None), None
+        if ptr:
+            self._lib.za_sched_free(ptr)
 
     # ----------------------------------------------------------------- intake
     def add(self, request: Request) -> None:
@@ -92,118 +128,105 @@ class Scheduler:
             raise ValueError(f"request {request.id!r} has an empty prompt")
         if request.max_new_tokens < 0:
             raise ValueError("max_new_tokens must be >= 0")
-        request.number = self._arrivals
-        self._arrivals += 1
+        handle = self.cache.pin(request.id)
+        number = ctypes.c_longlong()
+        eos = request.eos_token_id
+        has_eos = eos is not None and -2 ** 31 <= int(eos) < 2 ** 31
+        rc = self._lib.za_sched_add(self._ptr, handle, len(request.prompt),
+                                    int(request.max_new_tokens), 1 if has_eos else 0,
+                                    int(eos) if has_eos else 0, ctypes.byref(number))
+        if rc:
+            self.cache.unpin(request.id)
+            raise_for(rc)
+        request.number = number.value
         request.phase = WAITING
+        self._requests[handle] = request
         if request.max_new_tokens == 0:
-            self._finish(request, "length")
-            return
-        self.waiting.append(request)
+            self._finished(request, "length")
 
     def has_work(self) -> bool:
-        return bool(self.waiting or self.running)
+        return bool(self._lib.za_sched_has_work(self._ptr))
+
+    def _queue(self, which: int) -> List[Request]:
+        n = self._lib.za_sched_queue(self._ptr, which, None, 0)
+        out = np.empty((max(n, 1),), dtype=np.int64)
+        self._lib.za_sched_queue(self._ptr, which, out.ctypes.data, n)
+        return [self._requests[int(h)] for h in out[:n]]
+
+    @property
+    def waiting(self) -> List[Request]:
+        return self._queue(0)
+
+    @property
+    def running(self) -> List[Request]:
+        return self._queue(1)
+
+    @property
+    def preemption_count(self) -> int:
+        return int(self._lib.za_sched_preemptions(self._ptr))
 
     # --------------------------------------------------------------- one step
     def schedule(self) -> List[ScheduledEntry]:
-        budget = self.max_num_batched_tokens
-        plan: List[ScheduledEntry] = []
-        promised: Dict[int, int] = {}
-
-        def fits(req: Request, n: int) -> bool:
-            return self.cache.can_reserve(req.id, n, promised)
-
-        def promise(req: Request, n: int) -> None:
-            for gi, pages in self.cache.pages_needed(req.id, n).items():
-                promised[gi] = promised.get(gi, 0) + pages
-
-        # Decoding requests first (one token each), then running prompts, in arrival order.
-        order = sorted(self.running, key=lambda r: (r.remaining != 1, r.number))
-        for req in order:
-            if req.phase != RUNNING:          # preempted while serving an earlier one
-                continue
-            if budget == 0:
-                break
-            n = min(req.remaining, budget, self.chunk_size)
-            while not fits(req, n):
-                victim = max((r for r in self.running if r.phase == RUNNING),
-                             key=lambda r: r.number)
-                if victim is req and len([r for r in self.running if r.phase == RUNNING]) == 1 \
-                        and not plan:
-                    raise OutOfPages(
-                        f"request {req.id!r} needs more pages for {req.num_computed + n} tokens "
-                        "than the whole pool holds")
-                planned = next((e for e in plan if e.request is victim), None)
-                if planned is not None:
-                    # its pages for this step were only promised, not taken
-                    for gi, pages in self.cache.pages_needed(victim.id, planned.count).items():
-                        promised[gi] -= pages
-                    budget += planned.count
-                    plan.remove(planned)
-                self._preempt(victim)
-                if victim is req:
-                    break
-            if req.phase != RUNNING:
-                continue
-            promise(req, n)
-            plan.append(ScheduledEntry(req, req.num_computed, n,
-                                       req.num_computed + n == len(req.tokens)))
-            budget -= n
-        self.running = [r for r in self.running if r.phase == RUNNING]
-
-        # Admit waiting requests, head of the line first, while everything fits.
-        while self.waiting and budget > 0 and len(self.running) < self.max_num_seqs \
-                and self.cache.slots.free_count > 0:
-            req = self.waiting[0]
-            n = min(req.remaining, budget, self.chunk_size)
-            self.cache.admit(req.id)
-            if not fits(req, n):
-                self.cache.release(req.id)
-                if not self.running:
-                    raise OutOfPages(
-                        f"request {req.id!r} needs more pages for its first {n} tokens than "
-                        "the whole pool holds")
-                break
-            self.waiting.popleft()
-            req.phase = RUNNING
-            self.running.append(req)
-            promise(req, n)
-            plan.append(ScheduledEntry(req, 0, n, n == len(req.tokens)))
-            budget -= n
+        n_plan, n_victims = ctypes.c_int(), ctypes.c_int()
+        rc = self._lib.za_sched_schedule(
+            self._ptr, self._cap, self._ids.ctypes.data, self._starts.ctypes.data,
+            self._counts.ctypes.data, self._samples.ctypes.data, ctypes.byref(n_plan),
+            self._victims.ctypes.data, ctypes.byref(n_victims))
+        for h in self._victims[:min(n_victims.value, self._cap)].tolist():
+            victim = self._requests[h]
+            victim.num_computed = 0
+            victim.phase = WAITING
+            victim.preemptions += 1
+        raise_for(rc)
+        plan = []
+        ids = self._ids[:n_plan.value].tolist()
+        starts = self._starts[:n_plan.value].tolist()
+        counts = self._counts[:n_plan.value].tolist()
+        samples = self._samples[:n_plan.value].tolist()
+        for h, start, count, sample in zip(ids, starts, counts, samples):
+            req = self._requests[h]
+            if req.phase != RUNNING:                  # admitted in this call
+                req.phase = RUNNING
+                self.cache.admitted_by_scheduler(req.id)
+            plan.append(ScheduledEntry(req, start, count, bool(sample)))
         return plan
-
-    def _preempt(self, victim: Request) -> None:
-        self.cache.release(victim.id)
-        victim.num_computed = 0
-        victim.phase = WAITING
-        victim.preemptions += 1
-        self.preemption_count += 1
-        self.waiting.appendleft(victim)
 
     # ---------------------------------------------------------- after the step
     def update(self, plan: Sequence[ScheduledEntry], sampled: Dict[Hashable, int]) -> List[Request]:
         """Record the step: tokens computed, tokens drawn; finish and free what is done."""
-        done = []
-        for entry in plan:
+        n = len(plan)
+        if n > self._cap:
+            raise ValueError("a plan longer than max_num_seqs")
+        handles = self.cache.handles
+        for i, entry in enumerate(plan):
             req = entry.request
+            self._ids[i] = handles.of(req.id)
+            self._counts[i] = entry.count
+            self._samples[i] = 1 if entry.samples else 0
+            token = 0
+            if entry.samples:
+                token = int(sampled[req.id])
+                req.output.append(token)
+            self._tokens[i] = token
             req.num_computed += entry.count
-            if not entry.samples:
-                continue
-            token = int(sampled[req.id])
-            req.output.append(token)
-            if req.eos_token_id is not None and token == req.eos_token_id:
-                self._finish(req, "eos")
-            elif len(req.output) >= req.max_new_tokens:
-                self._finish(req, "length")
-            elif self.max_model_len and len(req.prompt) + len(req.output) >= self.max_model_len:
-                self._finish(req, "max_model_len")
-            if req.phase == FINISHED:
-                done.append(req)
-        self.running = [r for r in self.running if r.phase == RUNNING]
+        n_done = ctypes.c_int()
+        raise_for(self._lib.za_sched_update(
+            self._ptr, n, self._ids.ctypes.data, self._counts.ctypes.data,
+            self._samples.ctypes.data, self._tokens.ctypes.data, self._victims.ctypes.data,
+            self._reasons.ctypes.data, ctypes.byref(n_done)))
+        done = []
+        for h, reason in zip(self._victims[:n_done.value].tolist(),
+                             self._reasons[:n_done.value].tolist()):
+            req = self._requests[h]
+            self._finished(req, self._REASONS[reason])
+            done.append(req)
         return done
 
-    def _finish(self, req: Request, reason: str) -> None:
-        if req.id in self.cache.requests:
-            self.cache.release(req.id)
+    def _finished(self, req: Request, reason: str) -> None:
+        handle = self.cache.handles.of(req.id)
         req.phase = FINISHED
         req.finish_reason = reason
         self.finished.append(req)
+        self._lib.za_sched_forget(self._ptr, handle)
+        self._requests.pop(handle, None)
+        self.cache.unpin(req.id)

@@ -1,6 +1,8 @@
-"""Compiling the HIP sources under ``csrc/`` for gfx950 and loading the result.
+"""Compiling the sources under ``csrc/`` and loading the result: the HIP kernels
+for gfx950 with hipcc, the host-side bookkeeping (``host.cpp``) with the C++
+compiler.
 
-Every ``<name>.hip`` becomes ``lib<name>.so`` in ``zig_ai_amd/_lib`` (or, when
+Every ``<name>.hip`` / ``<name>.cpp`` becomes ``lib<name>.so`` in ``zig_ai_amd/_lib`` (or, when
 the package folder cannot be written, in a per-user folder under the system's
 temporary directory).  A library is compiled the first time something needs it
 and it is not there, or when its sources have changed since it was built;
@@ -26,6 +28,9 @@ PACKAGE_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC_DIR = os.path.join(PACKAGE_DIR, "csrc")
 ARCH = "gfx950"
 SOURCES = ("norm", "gemm", "rope_kv", "attention", "shortconv", "activation", "sampling")
+HOST_SOURCES = ("host",)            # plain C++, no device code: usable without a GPU or ROCm
+ALL_SOURCES = SOURCES + HOST_SOURCES
+CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden"]
 HIPCC_FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -49,6 +54,18 @@ def find_hipcc() -> Optional[str]:
         if cand and os.path.isfile(cand) and os.access(cand, os.X_OK):
             return cand
     return None
+
+
+def find_cxx() -> Optional[str]:
+    for cand in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"),
+                 shutil.which("clang++"), find_hipcc()):
+        if cand and os.path.isfile(cand) and os.access(cand, os.X_OK):
+            return cand
+    return None
+
+
+def _source_of(name: str) -> str:
+    return os.path.join(CSRC_DIR, name + (".cpp" if name in HOST_SOURCES else ".hip"))
 
 
 def _lib_dirs() -> List[str]:
@@ -75,10 +92,11 @@ def _writable_lib_dir() -> str:
 
 def source_digest(name: str) -> str:
     h = hashlib.sha256()
-    for path in (os.path.join(CSRC_DIR, "common.h"), os.path.join(CSRC_DIR, name + ".hip")):
+    host = name in HOST_SOURCES
+    for path in ([] if host else [os.path.join(CSRC_DIR, "common.h")]) + [_source_of(name)]:
         with open(path, "rb") as f:
             h.update(f.read())
-    h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(" ".join(CXX_FLAGS if host else HIPCC_FLAGS).encode())
     return h.hexdigest()
 
 
@@ -107,18 +125,29 @@ def _find_stale(name: str) -> Optional[str]:
 
 
 def compile_one(name: str) -> str:
-    hipcc = find_hipcc()
-    if hipcc is None:
-        raise KernelBuildError(
-            f"kernel library lib{name}.so is not built and hipcc was not found "
-            "(looked at $HIPCC, PATH and /opt/rocm/bin/hipcc)")
-    src = os.path.join(CSRC_DIR, name + ".hip")
+    host = name in HOST_SOURCES
+    src = _source_of(name)
     if not os.path.isfile(src):
         raise KernelBuildError(f"{src} does not exist")
+    if host:
+        cxx = find_cxx()
+        if cxx is None:
+            raise KernelBuildError(
+                f"lib{name}.so is not built and no C++ compiler was found "
+                "(looked at $CXX, g++, c++, clang++ and hipcc)")
+        flags = CXX_FLAGS + (["-x", "c++"] if os.path.basename(cxx).startswith("hipcc") else [])
+    else:
+        cxx = find_hipcc()
+        if cxx is None:
+            raise KernelBuildError(
+                f"kernel library lib{name}.so is not built and hipcc was not found "
+                "(looked at $HIPCC, PATH and /opt/rocm/bin/hipcc)")
+        flags = HIPCC_FLAGS
     out_dir = _writable_lib_dir()
     so = os.path.join(out_dir, f"lib{name}.so")
     tmp = os.path.join(out_dir, f".lib{name}.{os.getpid()}.{threading.get_ident()}.so")
-    cmd = [hipcc] + HIPCC_FLAGS + ["-I", CSRC_DIR, "-o", tmp, src]
+    cmd = [cxx] + flags + ["-I", CSRC_DIR, "-o", tmp, src]
+    what = os.path.basename(src)
     env = dict(os.environ)
     home = env.get("HOME", "")
     if not home or not os.path.isdir(home) or not os.access(home, os.W_OK):
@@ -139,29 +168,29 @@ def compile_one(name: str) -> str:
             proc.wait(timeout=15)
             break
         except subprocess.TimeoutExpired:
-            _say(f"still compiling {name}.hip for {ARCH} ({time.time() - start:.0f} s)")
+            _say(f"still compiling {what} ({time.time() - start:.0f} s)")
     reader.join()
     if proc.returncode != 0:
         if os.path.exists(tmp):
             os.remove(tmp)
         text = "".join(l for l in output if "packed-fp32-ops" not in l)
-        raise KernelBuildError(f"hipcc failed on {name}.hip (exit {proc.returncode}):\n{text}")
+        raise KernelBuildError(f"{os.path.basename(cxx)} failed on {what} (exit {proc.returncode}):\n{text}")
     os.replace(tmp, so)
     with open(so + ".digest.tmp", "w") as f:
         f.write(source_digest(name))
     os.replace(so + ".digest.tmp", so + ".digest")
-    _say(f"compiled {name}.hip in {time.time() - start:.1f} s -> {so}")
+    _say(f"compiled {what} in {time.time() - start:.1f} s -> {so}")
     return so
 
 
-def build_all(names: Iterable[str] = SOURCES, force: bool = False, jobs: int = 4) -> Dict[str, str]:
+def build_all(names: Iterable[str] = ALL_SOURCES, force: bool = False, jobs: int = 4) -> Dict[str, str]:
     """Compile the named sources (all by default); with ``force`` also those
     that are up to date.  Returns ``{name: path}``."""
     names = list(names)
     todo = [n for n in names if force or _find_built(n) is None]
     paths = {n: _find_built(n) for n in names if n not in todo}
     if todo:
-        _say(f"compiling {len(todo)} kernel source(s) for {ARCH}: {', '.join(todo)}")
+        _say(f"compiling {len(todo)} source(s) (kernels for {ARCH}): {', '.join(todo)}")
         with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(todo)))) as pool:
             for n, p in zip(todo, pool.map(compile_one, todo)):
                 paths[n] = p
@@ -169,17 +198,17 @@ def build_all(names: Iterable[str] = SOURCES, force: bool = False, jobs: int = 4
 
 
 def load(name: str) -> ctypes.CDLL:
-    """The library of ``csrc/<name>.hip``, compiled first if need be."""
+    """The library of ``csrc/<name>.hip`` (or ``.cpp``), compiled first if need be."""
     with _lock:
         if name in _loaded:
             return _loaded[name]
         path = _find_built(name)
         if path is None:
             stale = _find_stale(name)
-            if stale is not None and find_hipcc() is None:
+            if stale is not None and (find_cxx() if name in HOST_SOURCES else find_hipcc()) is None:
                 raise KernelBuildError(
-                    f"{stale} was built from other sources than the ones present and hipcc "
-                    "is not available to rebuild it")
+                    f"{stale} was built from other sources than the ones present and no "
+                    "compiler is available to rebuild it")
             path = compile_one(name)
         lib = ctypes.CDLL(path)
         _loaded[name] = lib

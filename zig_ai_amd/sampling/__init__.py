@@ -1,3 +1,3 @@
 """Sampling: greedy, temperature, top-k, top-p, repetition penalty."""
 
-from .sampler import SamplingParams, UniformStream, sample_rows  # noqa: F401
+from .sampler import SamplingParams, UniformStream, sample_rows, uniforms  # noqa: F401

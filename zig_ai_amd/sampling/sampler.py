@@ -24,7 +24,7 @@ from typing import List, Optional, Sequence
 import numpy as np
 import torch
 
-from ..kernels import ops
+from ..kernels import host, ops
 
 
 @dataclass(frozen=True)
@@ -48,18 +48,31 @@ class SamplingParams:
         return self.temperature <= 0.0
 
 
+def uniforms(seeds: Sequence[int], request_numbers: Sequence[int],
+             indices: Sequence[int]) -> List[float]:
+    """Number ``indices[i]`` of the stream of ``(seeds[i], request_numbers[i])`` for
+    every ``i``: 32-bit floats in [0, 1) from a counter-based generator in the host
+    library (``csrc/host.cpp``), each a pure function of its three keys."""
+    n = len(seeds)
+    mask = 0xFFFFFFFFFFFFFFFF
+    s = np.fromiter((int(v) & mask for v in seeds), dtype=np.uint64, count=n)
+    r = np.fromiter((int(v) & mask for v in request_numbers), dtype=np.uint64, count=n)
+    k = np.fromiter((int(v) & mask for v in indices), dtype=np.uint64, count=n)
+    out = np.empty((max(n, 1),), dtype=np.float32)
+    host.lib().za_uniforms(n, s.ctypes.data, r.ctypes.data, k.ctypes.data, out.ctypes.data)
+    return out[:n].tolist()
+
+
 class UniformStream:
     """The uniform numbers of one request: number ``k`` is a pure function of
     (seed, request number, k)."""
 
     def __init__(self, seed: int, request_number: int):
-        self._seed = int(seed) & 0xFFFFFFFFFFFFFFFF
-        self._request = int(request_number) & 0xFFFFFFFFFFFFFFFF
+        self.seed = int(seed)
+        self.request = int(request_number)
 
     def at(self, k: int) -> float:
-        bits = np.random.Philox(key=self._seed, counter=[int(k), self._request, 0, 0])
-        u = np.random.Generator(bits).random(dtype=np.float32)
-        return float(u)
+        return uniforms([self.seed], [self.request], [k])[0]
 
 
 def sample_rows(logits: torch.Tensor, params: Sequence[SamplingParams],
