@@ -113,8 +113,10 @@ class PreparedEntries:
         except (TypeError, ValueError, OverflowError) as err:
             raise StepError(f"token ids and wanted places must be integers: {err}") from err
         if tokens.size and (tokens.min() < 0 or tokens.max() >= vocab_size):
-            bad = int(tokens[(tokens < 0) | (tokens >= vocab_size)][0])
-            raise StepError(f"token id {bad} is outside the vocabulary of {vocab_size}")
+            where = int(np.flatnonzero((tokens < 0) | (tokens >= vocab_size))[0])
+            owner = int(np.searchsorted(np.cumsum(self.counts), where, side="right"))
+            raise StepError(f"request {entries[owner].request!r}: token id {int(tokens[where])} "
+                            f"is outside the vocabulary of {vocab_size}")
         self.tokens = tokens.astype(np.int32)
         self.wants = np.clip(wants, -1, 2 ** 31 - 1).astype(np.int32)
         self.vocab_size = int(vocab_size)

@@ -97,9 +97,11 @@ class DecoderModel:
         for b in self.blocks:
             every += [b.mixer_norm, b.mixer, b.feed_forward_norm, b.feed_forward]
         self.graph_safe = all(getattr(p, "graph_safe", False) for p in every)
-        # Compile what this model's parts use, together, before the first step.
+        # Compile what this model's parts use (and the host library), together, before
+        # the first step.
         if self.kernel_sources:
-            kernel_build.build_all(self.kernel_sources, jobs=len(self.kernel_sources))
+            wanted = list(self.kernel_sources) + list(kernel_build.HOST_SOURCES)
+            kernel_build.build_all(wanted, jobs=len(wanted))
 
     # ------------------------------------------------------------- construction
     @classmethod
