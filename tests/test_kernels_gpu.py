@@ -418,6 +418,62 @@ def test_paged_attention_decode_matrix_cores(nh, nkv, d, page_size, keys, nsplit
     assert rel_err(out, expect) < BF16_TOL
 
 
+def light_attention(q, k, v, positions, window=0):
+    """Causal attention for a few query rows against a long context: q [n, nh, d] at
+    ``positions``, k and v [T, nkv, d]; float64, one score row per query."""
+    n, nh, d = q.shape
+    nkv = k.shape[1]
+    out = torch.zeros((n, nh, d), dtype=torch.float64)
+    keys = torch.arange(k.shape[0])
+    for h in range(nh):
+        g = h // (nh // nkv)
+        s = (q[:, h].double() @ k[:, g].double().T) / math.sqrt(d)
+        mask = keys[None, :] > positions[:, None]
+        if window > 0:
+            mask = mask | (keys[None, :] <= positions[:, None] - window)
+        p = torch.softmax(s.masked_fill(mask, float("-inf")), dim=-1)
+        out[:, h] = p @ v[:, g].double()
+    return out
+
+
+@pytest.mark.parametrize("window", [0, 3000])
+def test_attention_over_long_contexts(window):
+    """Tens of thousands of keys: a portion of a prompt far into its request, and
+    single tokens whose context is cut into many ranges; one key far back is made to
+    dominate the last query."""
+    nh, nkv, d, ps = 8, 2, 64, 16
+    ctx, n = 20000, 150
+    k = rand((ctx + n, nkv, d), torch.bfloat16, 91)
+    v = rand((ctx + n, nkv, d), torch.bfloat16, 92)
+    q = rand((n, nh, d), torch.bfloat16, 93)
+    far = ctx + n - 2500                    # inside the window when there is one
+    k[far] = 0
+    k[far, :, 3] = 16.0
+    q[-1] = 0
+    q[-1, :, 3] = 16.0                      # score 32 against N(0, 4) for the other keys
+    cache, table = paged_from_dense([k], [v], ps, torch.bfloat16, seed=9)
+    positions = torch.arange(ctx, ctx + n, dtype=torch.int32)
+    expect = light_attention(q, k, v, positions.long(), window)
+    assert float((expect[-1] - v[far].double().repeat_interleave(nh // nkv, 0)).abs().max()) < 0.05
+    args = (cache.to(dev()), table.to(dev()), positions.to(dev()))
+    out = ops().paged_attention_mfma(q.to(dev()), *args, *items_for([n], 128 // (nh // nkv)),
+                                     1.0 / math.sqrt(d), window)
+    assert rel_err(out, expect) < BF16_TOL
+    # the last 16 tokens one by one, as a decode step of 16 requests would bring them:
+    # 16 requests that share the pages but stand at different positions
+    m = 16
+    tables = table.repeat(m, 1).to(dev())
+    pos_m = positions[-m:].to(dev())
+    for keys, nsplit in [(0, 1), (1024, (ctx + n + 1023) // 1024), (256, (ctx + n + 255) // 256)]:
+        out = ops().paged_attention_decode_mfma(q[-m:].to(dev()), cache.to(dev()), tables, pos_m,
+                                                None, None, None, m, 1.0 / math.sqrt(d), window,
+                                                keys, nsplit)
+        assert rel_err(out, expect[-m:]) < BF16_TOL, (keys, nsplit)
+        out = ops().paged_attention(q[-m:].to(dev()), cache.to(dev()), tables, pos_m,
+                                    *items_for([1] * m, 1), 1.0 / math.sqrt(d), window, keys, nsplit)
+        assert rel_err(out, expect[-m:]) < BF16_TOL, (keys, nsplit)
+
+
 def test_single_token_attention_returns_value():
     """One key: the softmax is 1 and the output is V (derived, but only checked for
     finiteness, in /root/reference/src/transformer/hybrid_attn.zig:1207-1212)."""
