@@ -125,6 +125,40 @@ def test_command_line_greedy():
     assert result["outputs"] == [oracle.greedy(prompt, 8)]
 
 
+def test_command_line_diagnostics(tmp_path):
+    """--random-weights with --config, --no-graph, --dump-logits, --verbose, --profile:
+    the same tokens with and without graphs; the dumped logits are those of the plain
+    implementation on the random model the same seed writes."""
+    import numpy as np
+    from tiny_configs import TINY_B
+    from zig_ai_amd.config import config_from_dict
+    from zig_ai_amd.weights import write_random_model
+    cfg_path = tmp_path / "config.json"
+    cfg_path.write_text(json.dumps(TINY_B))
+    prompt = eu.random_tokens(9, 512, 78)
+    base = [sys.executable, "-m", "zig_ai_amd", "--random-weights", "--config", str(cfg_path),
+            "--weights-seed", "5", "--prompt-ids", " ".join(map(str, prompt)), "-n", "6",
+            "--temperature", "0", "--dtype", "float32", "--page-size", "8", "--num-pages", "16",
+            "--max-num-seqs", "2", "--eos", "-1", "--json"]
+    dump = tmp_path / "dump"
+    runs = []
+    for extra in (["--no-graph", "--dump-logits", str(dump), "--verbose", "--profile"], []):
+        out = subprocess.run(base + extra, cwd=ROOT, capture_output=True, text=True, timeout=600)
+        assert out.returncode == 0, out.stderr[-2000:]
+        runs.append((json.loads(out.stdout.strip().splitlines()[-1])["outputs"], out.stderr))
+    assert runs[0][0] == runs[1][0]
+    assert "step 0: 1 requests, 9 tokens" in runs[0][1] and "decode:" in runs[0][1]
+    folder = str(tmp_path / "model")
+    write_random_model(config_from_dict(TINY_B), folder, seed=5, dtype=torch.float32)
+    oracle = plain.PlainLfm2(folder)
+    assert runs[0][0] == [oracle.greedy(prompt, 6)]
+    seq = list(prompt)
+    for step in range(6):
+        got = torch.from_numpy(np.fromfile(dump / f"{step}.f32", dtype="<f4"))
+        assert eu.rel_err(got.view(1, -1), oracle.logits(seq)[-1:]) < 1e-4
+        seq.append(runs[0][0][0][step])
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run(dtype, tmp_path):
     """bin/trace_run on a mixed trace with a pool so small that pages are used

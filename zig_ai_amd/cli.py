@@ -24,7 +24,12 @@ from typing import List, Optional
 
 def build_parser() -> argparse.ArgumentParser:
     ap = argparse.ArgumentParser(prog="zig-ai", description="LFM2 inference on one MI355X")
-    ap.add_argument("-m", "--model", required=True, help="model folder (config.json + safetensors)")
+    ap.add_argument("-m", "--model", default=None, help="model folder (config.json + safetensors)")
+    ap.add_argument("--random-weights", action="store_true",
+                    help="no checkpoint: draw weights N(0, 0.02) for --config (or the config.json "
+                         "in --model) into a temporary model folder")
+    ap.add_argument("--config", default=None, help="a config.json, for --random-weights")
+    ap.add_argument("--weights-seed", type=int, default=0, help="seed of --random-weights")
     ap.add_argument("--prompt", default=None, help="prompt text, or token ids without a tokenizer")
     ap.add_argument("--prompt-ids", default=None, help="prompt as token ids: \"5 17 3\" or \"5,17,3\"")
     ap.add_argument("--prompt-file", default=None,
@@ -47,7 +52,19 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--num-pages", type=int, default=None)
     ap.add_argument("--max-num-seqs", type=int, default=64)
+    ap.add_argument("--max-model-len", type=int, default=None,
+                    help="longest prompt + generation (default: the model's, at most 8192)")
     ap.add_argument("--eos", type=int, default=None, help="stop token id (default: the config's)")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="launch decode steps kernel by kernel instead of replaying HIP graphs "
+                         "(the reference's NOGRAPH)")
+    ap.add_argument("--dump-logits", default=None, metavar="DIR",
+                    help="write the logits every token is drawn from to DIR/<step>.f32, "
+                         "[rows, vocab] little-endian 32-bit (the reference's DUMP_LOGITS)")
+    ap.add_argument("--verbose", action="store_true", help="one line per step on standard error")
+    ap.add_argument("--profile", action="store_true",
+                    help="prompt and generation throughput on standard error at the end "
+                         "(the reference's PERF_STAGE)")
     ap.add_argument("--json", action="store_true", help="print one JSON object instead of text")
     return ap
 
@@ -76,6 +93,24 @@ def main(argv: Optional[List[str]] = None) -> int:
     if args.backend == "cpu":
         print("this engine has no CPU path; use --backend gpu", file=sys.stderr)
         return 2
+    scratch = None
+    if args.random_weights:
+        import tempfile
+        from .config import load_config
+        from .weights import write_random_model
+        source = args.config or args.model
+        if source is None:
+            print("--random-weights needs --config FILE (or --model with a config.json)",
+                  file=sys.stderr)
+            return 2
+        import torch
+        scratch = tempfile.TemporaryDirectory(prefix="zigai_random_")
+        store = torch.float32 if args.dtype == "float32" else torch.bfloat16
+        write_random_model(load_config(source), scratch.name, seed=args.weights_seed, dtype=store)
+        args.model = scratch.name
+    if not args.model:
+        print("give -m MODEL_DIR (or --random-weights --config FILE)", file=sys.stderr)
+        return 2
     tokenizer = load_tokenizer(args.model)
     prompts: List[List[int]]
     if args.prompt_file:
@@ -94,10 +129,29 @@ def main(argv: Optional[List[str]] = None) -> int:
     prompts = [p for p in prompts for _ in range(max(1, args.num_parallel))]
 
     from .engine.engine import Engine
+    if args.dump_logits:
+        os.makedirs(args.dump_logits, exist_ok=True)
+    phases = {"prompt_tokens": 0, "prompt_s": 0.0, "decode_tokens": 0, "decode_s": 0.0}
+
+    def on_step(info) -> None:
+        plan = info["plan"]
+        run = sum(e.count for e in plan)
+        decode = all(e.count == 1 and e.start > 0 for e in plan)
+        phases["decode_tokens" if decode else "prompt_tokens"] += run
+        phases["decode_s" if decode else "prompt_s"] += info["seconds"]
+        if args.dump_logits and info["logits"].shape[0]:
+            info["logits"].cpu().numpy().astype("<f4").tofile(
+                os.path.join(args.dump_logits, f"{info['step']}.f32"))
+        if args.verbose:
+            print(f"step {info['step']}: {len(plan)} requests, {run} tokens, "
+                  f"{len(info['tokens'])} drawn, {info['seconds'] * 1e3:.2f} ms", file=sys.stderr)
+
     load_start = time.perf_counter()
     engine = Engine(args.model, dtype=args.dtype, page_size=args.page_size,
                     num_pages=args.num_pages, max_num_seqs=args.max_num_seqs,
-                    max_num_batched_tokens=args.batch_size, chunk_size=args.ubatch_size)
+                    max_num_batched_tokens=args.batch_size, chunk_size=args.ubatch_size,
+                    max_model_len=args.max_model_len, use_graphs=not args.no_graph,
+                    on_step=on_step if (args.dump_logits or args.verbose or args.profile) else None)
     load_s = time.perf_counter() - load_start
     start = time.perf_counter()
     outputs = engine.generate(prompts, max_new_tokens=args.max_tokens,
@@ -108,6 +162,14 @@ def main(argv: Optional[List[str]] = None) -> int:
     torch.cuda.synchronize()
     total_s = time.perf_counter() - start
     n_new = sum(len(o) for o in outputs)
+    if args.profile:
+        for name in ("prompt", "decode"):
+            t, sec = phases[f"{name}_tokens"], phases[f"{name}_s"]
+            if t:
+                print(f"{name}: {t} tokens in {sec * 1e3:.1f} ms ({t / sec:.1f} tok/s)",
+                      file=sys.stderr)
+    if scratch is not None:
+        scratch.cleanup()
     if args.json:
         print(json.dumps({"outputs": outputs, "load_s": load_s, "generate_s": total_s,
                           "tokens_per_s": n_new / total_s if total_s > 0 else 0.0,

@@ -46,8 +46,9 @@ def config_from_dict(data: Mapping[str, Any]):
 
 
 def load_config(model_dir: str):
-    """Read ``model_dir/config.json`` and parse it with the registered class."""
-    path = os.path.join(model_dir, "config.json")
+    """Read ``model_dir/config.json`` (or the JSON file ``model_dir`` itself) and parse
+    it with the registered class."""
+    path = model_dir if os.path.isfile(model_dir) else os.path.join(model_dir, "config.json")
     if not os.path.isfile(path):
         raise ConfigError(f"{path} does not exist")
     with open(path, "r", encoding="utf-8") as f:

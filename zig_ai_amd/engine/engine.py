@@ -24,10 +24,16 @@ class Engine:
     def __init__(self, model_dir: str, dtype: str = "bfloat16", page_size: int = 16,
                  num_pages: Optional[int] = None, max_num_seqs: int = 64,
                  max_num_batched_tokens: int = 2048, chunk_size: int = 512,
-                 max_model_len: Optional[int] = None):
+                 max_model_len: Optional[int] = None, use_graphs: bool = True,
+                 on_step=None):
         """``num_pages``: pages per cache group; by default enough for
         ``max_num_seqs`` requests of ``max_model_len`` tokens (the model's
-        ``max_position_embeddings`` if not given, capped at 8192)."""
+        ``max_position_embeddings`` if not given, capped at 8192).
+        ``use_graphs=False`` launches every decode step kernel by kernel.
+        ``on_step(info)``, if given, is called after every step with a dict:
+        ``step``, ``plan`` (the scheduled entries), ``logits`` (32-bit, one row per
+        entry that samples, on the device), ``tokens`` (what was drawn from them),
+        ``seconds``."""
         self.model = DecoderModel.from_folder(model_dir, dtype)
         limit = max_model_len or self.model.spec.max_position or 8192
         if max_model_len is None:
@@ -35,7 +41,9 @@ class Engine:
         self.max_model_len = limit
         if num_pages is None:
             num_pages = max_num_seqs * ((limit + page_size - 1) // page_size)
-        self.runner = ModelRunner(self.model, page_size, num_pages, max_num_seqs)
+        self.runner = ModelRunner(self.model, page_size, num_pages, max_num_seqs,
+                                  use_graphs=use_graphs)
+        self.on_step = on_step
         self.scheduler = Scheduler(self.runner.cache, max_num_seqs, max_num_batched_tokens,
                                    chunk_size, limit)
         self._next_id = 0
@@ -81,7 +89,11 @@ class Engine:
             [e.request.output for e in sampling])
         done = self.scheduler.update(plan, {e.request.id: t for e, t in zip(sampling, drawn)})
         self.timings["steps"] += 1
-        self.timings["step_seconds"] += time.perf_counter() - start
+        elapsed = time.perf_counter() - start
+        self.timings["step_seconds"] += elapsed
+        if self.on_step is not None:
+            self.on_step({"step": self.timings["steps"] - 1, "plan": plan, "logits": logits,
+                          "tokens": drawn, "seconds": elapsed})
         self.timings["tokens_run"] += sum(e.count for e in plan)
         self.timings["tokens_generated"] += len(sampling)
         return done
