@@ -159,3 +159,101 @@ def test_random_workloads_finish_in_order_of_fairness(seed):
         assert r.output == [1000 + k for k in range(r.max_new_tokens)]   # none lost or doubled
     assert all(g.pool.free_count == g.pool.size for g in cache.groups)
     assert cache.slots.free_count == cache.slots.size
+
+
+SEEDS = range(30)
+
+
+def run_differential(seed):
+    """One random workload through the host library and through the plain statement
+    of the policy (tests/plain_scheduler.py) in lockstep; returns what happened."""
+    from plain_scheduler import FREED, PlainCache, PlainOutOfPages, PlainScheduler
+    seen = {"preemptions": 0, "refused": 0, "freed": 0, "steps": 0, "eos": 0}
+    rng = random.Random(seed)
+    page_size = rng.choice([2, 4, 8])
+    windows = [0] + ([rng.choice([5, 9, 16])] if seed % 2 else [])
+    num_slots = rng.randint(2, 5)
+    num_pages = rng.randint(4, 11)
+    limits = dict(max_num_seqs=rng.randint(1, 5), max_num_batched_tokens=rng.randint(3, 24),
+                  chunk_size=rng.randint(2, 12), max_model_len=rng.choice([0, 0, 30]))
+    needs = {0: StateNeed((4, 3))}
+    for g, w in enumerate(windows):
+        needs[1 + g] = PagedNeed(1, 16, w)
+    cache = CacheManager(needs, page_size, num_pages, num_slots, allocate=False)
+    sched = Scheduler(cache, **limits)
+    pcache = PlainCache(windows, num_pages, page_size, num_slots)
+    psched = PlainScheduler(pcache, limits["max_num_seqs"], limits["max_num_batched_tokens"],
+                            limits["chunk_size"], limits["max_model_len"])
+    biggest = (num_pages * page_size) // 2
+    pending = [(i, rng.randint(1, max(1, biggest)), rng.randint(0, 16),
+                rng.choice([None, None, 7])) for i in range(rng.randint(4, 12))]
+    reqs = {}
+    steps = 0
+    while pending or sched.has_work():
+        # requests arrive over time
+        while pending and (rng.random() < 0.5 or not sched.has_work()):
+            rid, plen, max_new, eos = pending.pop(0)
+            reqs[rid] = Request(rid, [1] * plen, max_new, eos_token_id=eos)
+            sched.add(reqs[rid])
+            psched.add(rid, plen, max_new, eos)
+        assert sched.has_work() == psched.has_work()
+        if not sched.has_work():
+            continue
+        try:
+            want = psched.schedule()
+        except PlainOutOfPages:
+            with pytest.raises(OutOfPages):
+                sched.schedule()
+            seen["refused"] = 1
+            return seen                             # both refuse: a request that cannot fit
+        plan = sched.schedule()
+        assert [(e.request.id, e.start, e.count, e.samples) for e in plan] == want
+        assert sched.preemption_count == psched.preemptions
+        assert [r.id for r in sched.waiting] == psched.waiting
+        assert sorted(r.id for r in sched.running) == sorted(psched.running)
+        for e in plan:
+            cache.reserve(e.request.id, e.count)
+            pcache.reserve(e.request.id, e.count)
+        for e in plan:
+            cache.commit(e.request.id, e.count)
+            pcache.commit(e.request.id, e.count)
+        for rid in psched.running:
+            assert cache.slot_of(rid) == pcache.req[rid]["slot"]
+            assert cache.num_tokens(rid) == pcache.req[rid]["tokens"]
+            for g in range(len(windows)):
+                assert cache.table(rid, g) == pcache.req[rid]["tables"][g]
+                seen["freed"] += pcache.req[rid]["tables"][g].count(FREED)
+        sampled = {e.request.id: rng.choice([7, 11, 12, 13]) for e in plan if e.samples}
+        done = sched.update(plan, sampled)
+        assert [r.id for r in done] == psched.update(want, sampled)
+        for r in done:
+            assert r.finish_reason == psched.info[r.id]["done"]
+            seen["eos"] += r.finish_reason == "eos"
+        for g in range(len(windows)):
+            assert cache.groups[g].pool.free_count == len(pcache.free[g])
+        assert cache.slots.free_count == len(pcache.free_slots)
+        cache.check()
+        steps += 1
+        assert steps < 5000
+    assert all(r.phase == FINISHED for r in reqs.values())
+    assert all(g.pool.free_count == g.pool.size for g in cache.groups)
+    seen["preemptions"] = psched.preemptions
+    seen["steps"] = steps
+    return seen
+
+
+@pytest.mark.parametrize("seed", SEEDS)
+def test_host_library_against_the_plain_scheduler(seed):
+    """Random workloads, pools so small that requests are preempted, windows that
+    give pages back: the host library's plans, block tables and free counts equal
+    those of the plain statement of the policy, step by step."""
+    run_differential(seed)
+
+
+def test_the_random_workloads_reach_the_hard_cases():
+    total = {}
+    for seed in SEEDS:
+        for k, v in run_differential(seed).items():
+            total[k] = total.get(k, 0) + v
+    assert total["preemptions"] >= 10 and total["refused"] >= 1
+    assert total["freed"] >= 10 and total["eos"] >= 3 and total["steps"] >= 300

@@ -158,6 +158,16 @@ class CacheManager:
         """The host library's object, for the scheduler and the step builder."""
         return self._ptr
 
+    @staticmethod
+    def bytes_per_page_index(needs: Mapping[int, object], page_size: int, element_size: int) -> int:
+        """Device bytes that ONE more page in every group costs (all groups are given
+        the same number of pages when ``num_pages`` is a single number)."""
+        total = 0
+        for need in needs.values():
+            if isinstance(need, PagedNeed):
+                total += 2 * need.num_kv_heads * page_size * need.head_dim * element_size
+        return total
+
     # ------------------------------------------------------------------ views
     def view(self, cache_id: int, writes: bool = True) -> CacheView:
         if cache_id in self._group_of:

@@ -14,6 +14,7 @@ from typing import Dict, Hashable, List, Optional, Sequence
 import torch
 
 from ..sampling.sampler import SamplingParams, sample_rows, uniforms
+from ..cache.manager import CacheManager
 from .batch import StepEntry
 from .model import DecoderModel
 from .runner import ModelRunner
@@ -25,10 +26,12 @@ class Engine:
                  num_pages: Optional[int] = None, max_num_seqs: int = 64,
                  max_num_batched_tokens: int = 2048, chunk_size: int = 512,
                  max_model_len: Optional[int] = None, use_graphs: bool = True,
-                 on_step=None):
+                 on_step=None, memory_fraction: float = 0.85):
         """``num_pages``: pages per cache group; by default enough for
         ``max_num_seqs`` requests of ``max_model_len`` tokens (the model's
-        ``max_position_embeddings`` if not given, capped at 8192).
+        ``max_position_embeddings`` if not given, capped at 8192), but no more than
+        fit into ``memory_fraction`` of the device memory that is free once the
+        weights are loaded.
         ``use_graphs=False`` launches every decode step kernel by kernel.
         ``on_step(info)``, if given, is called after every step with a dict:
         ``step``, ``plan`` (the scheduled entries), ``logits`` (32-bit, one row per
@@ -40,7 +43,19 @@ class Engine:
             limit = min(limit, 8192)
         self.max_model_len = limit
         if num_pages is None:
-            num_pages = max_num_seqs * ((limit + page_size - 1) // page_size)
+            per_request = (limit + page_size - 1) // page_size
+            num_pages = max_num_seqs * per_request
+            element = 4 if self.model.runtime.dtype == torch.float32 else 2
+            per_page = CacheManager.bytes_per_page_index(self.model.cache_needs, page_size, element)
+            if per_page:
+                free, _ = torch.cuda.mem_get_info(self.model.runtime.device)
+                fit = int(free * memory_fraction) // per_page
+                if fit < per_request:
+                    raise MemoryError(
+                        f"{free / 2**30:.1f} GiB of device memory are free: not enough for the "
+                        f"cache of one request of {limit} tokens ({per_request * per_page / 2**30:.1f}"
+                        " GiB); lower max_model_len")
+                num_pages = min(num_pages, fit)
         self.runner = ModelRunner(self.model, page_size, num_pages, max_num_seqs,
                                   use_graphs=use_graphs)
         self.on_step = on_step
