@@ -141,13 +141,6 @@ class PreparedEntries:
             raise StepError(msg)
         raise_for(rc)
 
-    def extent(self, cache: CacheManager) -> Tuple[int, int]:
-        """(pages of the longest block table, longest context including the new
-        tokens) among the entries."""
-        self.build(cache, np.zeros((0,), dtype=np.int32), 0, 0,
-                   np.zeros((2 * (7 + 2 * len(cache.groups)),), dtype=np.int64), None, 0)
-        return int(self.meta[3]), int(self.meta[4])
-
 
 def build_step(entries: Sequence[StepEntry], cache: CacheManager, device: torch.device,
                vocab_size: int, item_granularities: Sequence[int] = (),
