@@ -1,6 +1,8 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py --shape 2.6b --prompt-len 6144        # another LFM2 shape, same measurement
+    python bench.py --shape 350m --workload serve         # 64 requests through the scheduler
 
 Default run: the layer sizes of the LFM2-1.2B shape (16 layers, hidden 2048, vocabulary 65,536)
 with random bfloat16 weights N(0, 0.02), a batch of 8 requests, each prefilled
@@ -37,6 +39,59 @@ LFM2_1_2B = {
     "conv_L_cache": 3, "conv_bias": False, "tie_embedding": True,
     "max_position_embeddings": 128000,
 }
+
+
+def _shape(hidden, heads, kv_heads, ff, layers, attention_at):
+    cfg = dict(LFM2_1_2B)
+    cfg.update(hidden_size=hidden, num_attention_heads=heads, num_key_value_heads=kv_heads,
+               block_ff_dim=ff, num_hidden_layers=layers,
+               layer_types=["full_attention" if i in attention_at else "conv"
+                            for i in range(layers)])
+    return cfg
+
+
+# the shapes the engine is measured on; the default is the first
+SHAPES = {
+    "1.2b": LFM2_1_2B,
+    "350m": _shape(1024, 16, 8, 6656, 16, (2, 5, 8, 10, 12, 14)),
+    "2.6b": _shape(2048, 32, 8, 10752, 30, (2, 6, 10, 14, 18, 21, 24, 27)),
+}
+
+
+def serve(cfg, name, n_requests, new_tokens) -> int:
+    """Requests with prompts of 128 to 2,048 tokens through the scheduler, the step
+    function and the sampler (temperature 0.7), all admitted at once."""
+    import random
+    import tempfile
+
+    import torch
+    from zig_ai_amd.config import config_from_dict
+    from zig_ai_amd.engine import Engine
+    from zig_ai_amd.weights import write_random_model
+
+    rng = random.Random(1)
+    prompts = [[rng.randrange(cfg["vocab_size"]) for _ in range(rng.randint(128, 2048))]
+               for _ in range(n_requests)]
+    with tempfile.TemporaryDirectory(prefix="zigai_bench_") as folder:
+        write_random_model(config_from_dict(cfg), folder, seed=0, dtype=torch.bfloat16)
+        engine = Engine(folder, dtype="bfloat16", page_size=16, max_num_seqs=64,
+                        max_num_batched_tokens=4096, chunk_size=2048, max_model_len=4096)
+        engine.generate(prompts[:2], max_new_tokens=4, temperature=0.0, eos_token_id=-1)   # warm-up
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        out = engine.generate(prompts, max_new_tokens=new_tokens, temperature=0.7, seed=3,
+                              eos_token_id=-1)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        stats = engine.stats()
+    prompt_tokens, generated = sum(len(p) for p in prompts), sum(len(o) for o in out)
+    print(json.dumps({
+        "workload": "serve", "model": f"LFM2-{name} shape", "requests": n_requests,
+        "prompt_tokens": prompt_tokens, "generated_tokens": generated, "seconds": dt,
+        "generated_per_s": generated / dt, "tokens_per_s": (prompt_tokens + generated) / dt,
+        "steps": stats["steps"], "preemptions": stats["preemptions"], "dtype": "bf16",
+        "data": "synthetic token ids; random weights N(0, 0.02)"}), flush=True)
+    return 0
 
 
 def count_bytes(model):
@@ -80,6 +135,15 @@ def main() -> int:
     ap.add_argument("--prompt-len", type=int, default=2048)
     ap.add_argument("--layers", type=int, default=None,
                     help="run fewer layers than the configuration has (both numbers are reported)")
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="1.2b",
+                    help="layer sizes: LFM2-1.2B (the default run), 350M or 2.6B")
+    ap.add_argument("--workload", choices=["steps", "serve"], default="steps",
+                    help="steps: decode steps and one prefill (the default run); serve: 64 "
+                         "requests with prompts of 128-2048 tokens and 256 new tokens each "
+                         "through the scheduler")
+    ap.add_argument("--requests", type=int, default=64, help="requests of --workload serve")
+    ap.add_argument("--new-tokens", type=int, default=256, help="new tokens per request of "
+                    "--workload serve")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points")
     ap.add_argument("--phase", choices=["all", "prefill", "decode"], default="all",
                     help="measure only one phase (for profiling); the JSON line then holds "
@@ -94,7 +158,9 @@ def main() -> int:
     from zig_ai_amd.kernels import ops
 
     torch.cuda.set_device(0)
-    cfg = dict(LFM2_1_2B)
+    cfg = dict(SHAPES[args.shape])
+    if args.workload == "serve":
+        return serve(cfg, args.shape.upper(), args.requests, args.new_tokens)
     full_layers = cfg["num_hidden_layers"]
     if args.layers is not None and args.layers < full_layers:
         cfg["num_hidden_layers"] = args.layers
@@ -189,13 +255,15 @@ def main() -> int:
             points[f"decode_b{b}"] = b * steps / d
 
     line = {
-        "metric": "decode tok/s @ batch 8 (LFM2-1.2B shape, context 2048 prompt + decode)",
+        "metric": f"decode tok/s @ batch {args.batch} (LFM2-{args.shape.upper()} shape, context "
+                  f"{args.prompt_len} prompt + decode)",
         "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic token ids uniform over the vocabulary; random weights N(0, 0.02)",
         "config": {
-            "model": "LFM2-1.2B shape", "global_batch": args.batch, "seq_len": 4096,
+            "model": f"LFM2-{args.shape.upper()} shape", "global_batch": args.batch,
+            "seq_len": args.prompt_len + 2048,
             "prompt_len": args.prompt_len, "parallelism": "single GPU",
             "layers": cfg["num_hidden_layers"], "layers_of_config": full_layers,
             "attention_layers": n_attn, "hidden_size": cfg["hidden_size"],
