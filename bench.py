@@ -8,7 +8,8 @@ Default run: the layer sizes of the LFM2-1.2B shape (16 layers, hidden 2048, voc
 with random bfloat16 weights N(0, 0.02), a batch of 8 requests, each prefilled
 with 2,048 synthetic tokens and decoded from there (context 4,096).  A step is
 one decode step of the whole batch through the engine's own step function and
-greedy sampler.  Prints ONE JSON line: decoded tokens per second as ``value``,
+greedy sampler, issued as generation issues them (the tokens of a step reach the
+next one on the device; the host reads them every 8 steps).  Prints ONE JSON line: decoded tokens per second as ``value``,
 a 2,048-token prefill under ``prefill``, the decode step against the HBM
 roofline under ``roofline``, and batch 1 / batch 64 decoding under ``points``.
 """
@@ -183,16 +184,23 @@ def main() -> int:
             logits = runner.step([StepEntry(r, tokens(prompt_len), [prompt_len - 1])])
             last.append(int(ops.argmax(logits)[0]))
 
-        def one(cur):
-            logits = runner.step([StepEntry(r, [cur[r]], [0]) for r in range(batch)])
-            return ops.argmax(logits).tolist()
+        requests = list(range(batch))
 
-        for _ in range(warmup):
-            last = one(last)
+        def run(cur, n):
+            """``n`` decode steps the way generation issues them: greedy tokens handed
+            from step to step on the device, the host reading them every 8 steps."""
+            done = 0
+            while done < n:
+                k = min(8, n - done)
+                drawn = runner.decode_steps(requests, cur, k, lambda logits, i: ops.argmax(logits))
+                cur = drawn[-1].tolist()
+                done += drawn.shape[0]
+            return cur
+
+        last = run(last, warmup)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(steps):
-            last = one(last)
+        last = run(last, steps)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         ctx_mid = prompt_len + warmup + steps / 2.0

@@ -270,3 +270,54 @@ def test_widths_that_are_no_multiple_of_eight():
     narrow = eu.model_folder(TINY_E, 4, torch.bfloat16, **eu.sharp_kwargs())
     with pytest.raises(KernelError, match="multiple of 8"):
         DecoderModel.from_folder(narrow, "bfloat16")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_hand_tokens_over_on_the_device(dtype):
+    """Several decode steps without the host reading the tokens in between: the same
+    tokens as step by step, including across the first step of a new graph shape and
+    when pages run out in the middle."""
+    from zig_ai_amd.engine import StepEntry
+    from zig_ai_amd.kernels import ops
+    model, _, prompts = setup("B", dtype)
+    long_prompt = max(prompts, key=len)
+    greedy = lambda logits, i: ops.argmax(logits)
+    ids = ["a", "b", "c"]
+    lens = [9, 30, 17]
+
+    def start(runner):
+        last = []
+        for r, n in zip(ids, lens):
+            runner.admit(r)
+            logits = runner.step([StepEntry(r, long_prompt[:n], [n - 1])])
+            last.append(int(ops.argmax(logits)[0]))
+        return last
+
+    single = runner_for(model, 8, 64)
+    cur = start(single)
+    want = []
+    for _ in range(20):
+        logits = single.step([StepEntry(r, [t], [0]) for r, t in zip(ids, cur)])
+        cur = ops.argmax(logits).tolist()
+        want.append(cur)
+    many = runner_for(model, 8, 64)
+    cur = start(many)
+    got = []
+    for k in (1, 7, 12):                                  # 12: crosses a page and a graph shape
+        drawn = many.decode_steps(ids, cur, k, greedy)
+        assert drawn.shape == (k, 3) and drawn.dtype == torch.int32
+        got += drawn.tolist()
+        cur = got[-1]
+    if dtype == "float32":
+        assert got == want
+    else:
+        assert sum(g != w for g, w in zip(got, want)) <= 1   # a near-tie may tip in bfloat16
+    # a pool that holds the prompts and little more: the run stops when pages run out
+    tight = runner_for(model, 8, 9)                       # 2 + 4 + 3 pages for the prompts
+    cur = start(tight)
+    drawn = tight.decode_steps(ids, cur, 16, greedy)
+    assert 1 <= drawn.shape[0] < 16
+    tight.cache.check()
+    assert [tight.cache.num_tokens(r) for r in ids] == [n + drawn.shape[0] for n in lens]
+    if dtype == "float32":
+        assert drawn.tolist() == want[:drawn.shape[0]]

@@ -18,7 +18,8 @@ from ..cache.manager import CacheManager
 from .batch import StepEntry
 from .model import DecoderModel
 from .runner import ModelRunner
-from .scheduler import Request, ScheduledEntry, Scheduler
+from ..kernels import ops
+from .scheduler import RUNNING, Request, ScheduledEntry, Scheduler
 
 
 class Engine:
@@ -26,13 +27,18 @@ class Engine:
                  num_pages: Optional[int] = None, max_num_seqs: int = 64,
                  max_num_batched_tokens: int = 2048, chunk_size: int = 512,
                  max_model_len: Optional[int] = None, use_graphs: bool = True,
-                 on_step=None, memory_fraction: float = 0.85):
+                 on_step=None, memory_fraction: float = 0.85, multi_step: int = 8):
         """``num_pages``: pages per cache group; by default enough for
         ``max_num_seqs`` requests of ``max_model_len`` tokens (the model's
         ``max_position_embeddings`` if not given, capped at 8192), but no more than
         fit into ``memory_fraction`` of the device memory that is free once the
         weights are loaded.
         ``use_graphs=False`` launches every decode step kernel by kernel.
+        ``multi_step``: while every running request decodes and none waits, up to this
+        many decode steps are issued without the host waiting for the tokens in
+        between (each step's tokens reach the next on the device); a request that
+        meets its stop token inside such a run wastes the steps after it, nothing
+        else changes.  1 switches it off, and so does ``on_step``.
         ``on_step(info)``, if given, is called after every step with a dict:
         ``step``, ``plan`` (the scheduled entries), ``logits`` (32-bit, one row per
         entry that samples, on the device), ``tokens`` (what was drawn from them),
@@ -59,6 +65,7 @@ class Engine:
         self.runner = ModelRunner(self.model, page_size, num_pages, max_num_seqs,
                                   use_graphs=use_graphs)
         self.on_step = on_step
+        self.multi_step = 1 if on_step is not None else max(1, int(multi_step))
         self.scheduler = Scheduler(self.runner.cache, max_num_seqs, max_num_batched_tokens,
                                    chunk_size, limit)
         self._next_id = 0
@@ -90,6 +97,9 @@ class Engine:
         if not plan:
             return []
         start = time.perf_counter()
+        k = self._steps_ahead(plan)
+        if k > 1:
+            return self._decode_many(plan, k, start)
         entries = []
         for e in plan:
             entries.append(StepEntry(e.request.id, e.request.span(e.start, e.count),
@@ -111,6 +121,56 @@ class Engine:
                           "tokens": drawn, "seconds": elapsed})
         self.timings["tokens_run"] += sum(e.count for e in plan)
         self.timings["tokens_generated"] += len(sampling)
+        return done
+
+    def _steps_ahead(self, plan: Sequence[ScheduledEntry]) -> int:
+        """How many decode steps may be issued in one go after this plan: more than
+        one only if every entry is a decoding request, nobody waits to be admitted,
+        and no request needs its history on the host between steps."""
+        if self.multi_step <= 1 or self.scheduler.has_waiting():
+            return 1
+        k = self.multi_step
+        for e in plan:
+            req = e.request
+            if e.count != 1 or not e.samples or e.start == 0 \
+                    or req.sampling.repetition_penalty != 1.0:
+                return 1
+            k = min(k, req.max_new_tokens - len(req.output),
+                    self.max_model_len - len(req.prompt) - len(req.output))
+        return max(1, k)
+
+    def _decode_many(self, plan: Sequence[ScheduledEntry], k: int, start: float) -> List[Request]:
+        reqs = [e.request for e in plan]
+        params = [r.sampling for r in reqs]
+        device = self.model.runtime.device
+        if all(p.greedy for p in params):
+            def sample(logits: torch.Tensor, i: int) -> torch.Tensor:
+                return ops.argmax(logits)
+        else:
+            S = len(reqs)
+            packed = torch.tensor([[p.temperature for p in params], [p.top_p for p in params]],
+                                  dtype=torch.float32).to(device)
+            top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32).to(device)
+            u = torch.tensor(uniforms([p.seed for p in params] * k,
+                                      [r.number for r in reqs] * k,
+                                      [len(r.output) + i for i in range(k) for r in reqs]),
+                             dtype=torch.float32).view(k, S).to(device)
+
+            def sample(logits: torch.Tensor, i: int) -> torch.Tensor:
+                return ops.sample(logits, packed[0], top_k, packed[1], u[i])
+        drawn = self.runner.decode_steps([r.id for r in reqs],
+                                         [r.span(e.start, 1)[0] for r, e in zip(reqs, plan)],
+                                         k, sample).tolist()        # the one wait of the run
+        done: List[Request] = []
+        alive = list(range(len(reqs)))
+        for j, row in enumerate(drawn):
+            step_plan = [ScheduledEntry(reqs[a], plan[a].start + j, 1, True) for a in alive]
+            done += self.scheduler.update(step_plan, {reqs[a].id: row[a] for a in alive})
+            self.timings["tokens_generated"] += len(alive)
+            self.timings["tokens_run"] += len(alive)
+            alive = [a for a in alive if reqs[a].phase == RUNNING]
+        self.timings["steps"] += len(drawn)
+        self.timings["step_seconds"] += time.perf_counter() - start
         return done
 
     def run(self) -> None:

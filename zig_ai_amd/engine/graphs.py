@@ -20,7 +20,7 @@ they were at capture.  Nothing in the graph clears memory with a memset node.
 from __future__ import annotations
 
 import gc
-from typing import Dict, Sequence, Tuple
+from typing import Dict, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -74,12 +74,22 @@ class DecodeGraphs:
             raise StepError(msg)
         raise_for(rc)
 
-    def run(self, runner, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def run(self, runner, entries: Sequence[StepEntry],
+            device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Logits ``[len(entries), vocab]`` of a step of single tokens (one row per
         entry, whatever the entries want).  Takes the pages the new tokens need (all
-        or none: ``OutOfPages`` leaves everything as it was)."""
+        or none: ``OutOfPages`` leaves everything as it was).
+
+        With ``device_tokens`` (int32 ``[len(entries)]`` on the device, for instance
+        what the sampler drew from the last step's logits) the entries' own tokens are
+        ignored and the step reads its token ids from that tensor, copied on the
+        device: the host never waits for them, so it can lay out this step while the
+        last one is still running."""
         cache = runner.cache
         S = len(entries)
+        if device_tokens is not None and (device_tokens.dtype != torch.int32
+                                          or device_tokens.numel() != S):
+            raise StepError(f"device_tokens must be int32 [{S}]")
         sc = self._scratch(S)
         ptr = sc["ptr"]
         known = cache.handles.known
@@ -89,6 +99,9 @@ class DecodeGraphs:
             if h is None:
                 raise StepError(f"request {e.request!r} was not admitted")
             reqs[i] = h
+            if device_tokens is not None:
+                toks[i] = 0                      # a stand-in; the ids are copied on the device
+                continue
             try:
                 toks[i] = e.tokens[0]
             except (OverflowError, TypeError, ValueError):
@@ -124,10 +137,16 @@ class DecodeGraphs:
             if slot["copied"] is None:
                 slot["copied"] = torch.cuda.Event()
             slot["copied"].record()
+            if device_tokens is not None:
+                first = int(slot["sections"][0])          # where the token ids sit
+                slot["buffer"][first:first + S].copy_(device_tokens.view(-1))
             slot["graph"].replay()
             self.replays += 1
             return slot["logits"]
         model = runner.model
+        if device_tokens is not None:                     # a first step of this shape: on the host
+            entries = [StepEntry(e.request, [t], [0])
+                       for e, t in zip(entries, device_tokens.view(-1).tolist())]
         asked = [StepEntry(e.request, e.tokens, [0]) for e in entries]
         prepared = PreparedEntries(asked, cache, self._vocab)
         if slot is None:

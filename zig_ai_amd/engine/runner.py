@@ -14,7 +14,7 @@ written for several sequences (``num_seqs``, ``block_tables[seq]``:
 
 from __future__ import annotations
 
-from typing import Hashable, List, Optional, Sequence
+from typing import Callable, Hashable, List, Optional, Sequence
 
 import torch
 
@@ -73,6 +73,40 @@ class ModelRunner:
         self.cache.commit_many([e.request for e in entries], [len(e.tokens) for e in entries])
         self.steps_run += 1
         return logits
+
+    def decode_steps(self, requests: Sequence[Hashable], tokens: Sequence[int], n_steps: int,
+                     sample: Callable[[torch.Tensor, int], torch.Tensor]) -> torch.Tensor:
+        """Up to ``n_steps`` decode steps of the same requests without the host waiting
+        in between: ``tokens`` are the requests' next tokens, ``sample(logits, i)``
+        draws the tokens of step ``i`` (int32 ``[len(requests)]`` on the device, without
+        looking at them on the host), and those are the next step's tokens, handed over
+        on the device.  Returns what was drawn, ``[steps done, len(requests)]`` on the
+        device; fewer steps than asked for are done when pages run out after the first
+        (``OutOfPages`` from the first step is raised)."""
+        if len(requests) != len(tokens) or not requests:
+            raise StepError("one next token per request is needed")
+        entries = [StepEntry(r, [t], [0]) for r, t in zip(requests, tokens)]
+        ones = [1] * len(requests)
+        drawn: List[torch.Tensor] = []
+        current = None
+        for i in range(n_steps):
+            try:
+                if self.graphs is not None:
+                    logits = self.graphs.run(self, entries, device_tokens=current)
+                else:
+                    if current is not None:
+                        entries = [StepEntry(r, [t], [0])
+                                   for r, t in zip(requests, current.view(-1).tolist())]
+                    logits = self.model.forward(self.prepare(entries), self.views)
+            except OutOfPages:
+                if i == 0:
+                    raise
+                break
+            current = sample(logits, i)
+            drawn.append(current)
+            self.cache.commit_many(requests, ones)
+            self.steps_run += 1
+        return torch.stack(drawn)
 
     def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         for e in entries:

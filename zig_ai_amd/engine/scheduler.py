@@ -147,6 +147,9 @@ class Scheduler:
     def has_work(self) -> bool:
         return bool(self._lib.za_sched_has_work(self._ptr))
 
+    def has_waiting(self) -> bool:
+        return self._lib.za_sched_queue(self._ptr, 0, None, 0) > 0
+
     def _queue(self, which: int) -> List[Request]:
         n = self._lib.za_sched_queue(self._ptr, which, None, 0)
         out = np.empty((max(n, 1),), dtype=np.int64)
