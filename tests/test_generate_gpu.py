@@ -111,6 +111,28 @@ def test_eos_and_length_stop():
     assert engine.generate([prompt], max_new_tokens=0, temperature=0.0)[0] == []
 
 
+def test_steps_issued_ahead_change_nothing():
+    """Up to 8 decode steps issued without waiting for the tokens in between, against
+    one step at a time: the same tokens, also for a request that meets its stop token
+    in the middle of such a run, with sampling and with a budget that admits late."""
+    from zig_ai_amd.engine import Engine
+    folder = folder_for(TINY_B, 1)
+    prompts = [eu.random_tokens(n, 512, 600 + n) for n in (12, 40, 7, 25)]
+    for kw in (dict(temperature=0.0), dict(temperature=0.9, top_k=30, seed=11)):
+        def one():                                    # a new engine: requests numbered from 0
+            return Engine(folder, dtype="float32", page_size=8, num_pages=64, max_num_seqs=4,
+                          multi_step=1)
+        free_run = one().generate(prompts, max_new_tokens=20, eos_token_id=-1, **kw)
+        stop = free_run[1][9]                         # request 1 stops inside a run of 8
+        want = one().generate(prompts, max_new_tokens=20, eos_token_id=stop, **kw)
+        ahead = Engine(folder, dtype="float32", page_size=8, num_pages=64, max_num_seqs=2,
+                       multi_step=8)                  # two at a time: the others wait, then join
+        got = ahead.generate(prompts, max_new_tokens=20, eos_token_id=stop, **kw)
+        assert got == want and len(want[1]) <= 10
+        stats = ahead.stats()
+        assert stats["requests"] == 0 and all(g["pages_free"] == g["pages"] for g in stats["groups"])
+
+
 def test_command_line_greedy():
     folder = folder_for(TINY_A, 0)
     oracle = plain.PlainLfm2(folder)
