@@ -160,3 +160,25 @@ def test_uniform_streams():
     assert abs(np.corrcoef(x[:-1], x[1:])[0, 1]) < 0.06
     # large keys are taken whole
     assert uniforms([2 ** 63 + 5], [2 ** 40], [2 ** 33]) != uniforms([5], [2 ** 40], [2 ** 33])
+
+
+def test_context_split_plan():
+    """How decode attention cuts long contexts: a function of the batch shape and the
+    longest context only; ranges cover the context, are multiples of the key tile,
+    and there are never more than SPLIT_MAX of them."""
+    from zig_ai_amd.parts.attention import SPLIT_MAX, SPLIT_TARGET, plan_split
+    for items in (1, 2, 8, 33, 64, 200):
+        for kv_heads in (1, 8):
+            for max_keys in (1, 100, 513, 2048, 4096, 33000, 131072, 1 << 20):
+                keys, nsplit = plan_split(items, kv_heads, max_keys)
+                assert (keys, nsplit) == plan_split(items, kv_heads, max_keys)
+                if nsplit == 1:
+                    assert keys == 0
+                    continue
+                assert keys % 64 == 0 and keys & (keys - 1) == 0
+                assert keys * nsplit >= max_keys > keys * (nsplit - 1)
+                assert nsplit <= SPLIT_MAX
+    assert plan_split(64, 8, 100000) == (0, 1)            # enough requests: no cut
+    assert plan_split(8, 8, 2200) == (512, 5)             # the benchmark's decode step
+    keys, nsplit = plan_split(1, 8, 131072)               # one long request: ~SPLIT_TARGET groups
+    assert (keys, nsplit) == (4096, 32) and 8 * nsplit >= SPLIT_TARGET

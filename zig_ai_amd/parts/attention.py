@@ -27,8 +27,10 @@ from .feed_forward import fuse_rows
 
 # Cutting long contexts pays only when the launch would otherwise leave most of the
 # machine idle (decoding few requests).  Measured on one MI355X with 8 key/value
-# heads: from 512 workgroups on nothing is gained; below, the longest range (of
-# 1024, 512 or 256 keys) that still yields SPLIT_TARGET workgroups is best.
+# heads, contexts from 2,048 to 131,072 keys and 1 to 64 requests: from 512
+# workgroups on nothing is gained; below, the longest range (a power of two from
+# 256 to 8,192 keys) that still yields SPLIT_TARGET workgroups is best or within a
+# few percent of it (fewer partial results to merge).
 BUSY_WORKGROUPS = 512
 SPLIT_TARGET = 256
 SPLIT_KEYS_MIN = 256
@@ -42,7 +44,7 @@ def plan_split(n_items: int, num_kv_heads: int, max_keys: int):
     if groups >= BUSY_WORKGROUPS or max_keys <= 2 * SPLIT_KEYS_MIN:
         return 0, 1
     keys = SPLIT_KEYS_MIN
-    for cand in (1024, 512):
+    for cand in (8192, 4096, 2048, 1024, 512):
         if groups * ((max_keys + cand - 1) // cand) >= SPLIT_TARGET:
             keys = cand
             break
