@@ -336,7 +336,7 @@ def run_attention(dtype, nh, nkv, d, page_size, ctx, new, window=0, keys_per_spl
     elif mfma:
         out = ops().paged_attention_mfma(q_all, cache.to(dev()), table.to(dev()), positions,
                                          *items_for(new, max(1, 128 // G)), 1.0 / math.sqrt(d),
-                                         window)
+                                         window, keys_per_split, nsplit)
     else:
         out = ops().paged_attention(q_all, cache.to(dev()), table.to(dev()), positions,
                                     *items_for(new, max(1, 32 // G)), 1.0 / math.sqrt(d), window,
@@ -390,6 +390,19 @@ def test_paged_attention_matrix_cores(nh, nkv, d, page_size, window):
                                 sharpen=True, mfma=True)
     assert rel_err(out, expect) < BF16_TOL
     assert float(expect.abs().max()) > 0.5
+
+
+@pytest.mark.parametrize("keys,nsplit", [(64, 12), (256, 3), (1024, 1)])
+@pytest.mark.parametrize("window", [0, 70])
+def test_paged_attention_matrix_cores_cut_contexts(keys, nsplit, window):
+    """Prompt portions with their contexts cut into ranges: ranges that a row cannot
+    see at all, ranges that end inside a tile's worth of rows, empty ranges."""
+    ctx = [700, 0, 255, 64, 300]
+    new = [40, 150, 3, 70, 1]
+    for nh, nkv, d, ps in [(32, 8, 64, 16), (6, 2, 128, 8)]:
+        out, expect = run_attention(torch.bfloat16, nh, nkv, d, ps, ctx, new, window=window,
+                                    keys_per_split=keys, nsplit=nsplit, sharpen=True, mfma=True)
+        assert rel_err(out, expect) < BF16_TOL
 
 
 def test_paged_attention_matrix_cores_paired_items():
@@ -456,9 +469,10 @@ def test_attention_over_long_contexts(window):
     expect = light_attention(q, k, v, positions.long(), window)
     assert float((expect[-1] - v[far].double().repeat_interleave(nh // nkv, 0)).abs().max()) < 0.05
     args = (cache.to(dev()), table.to(dev()), positions.to(dev()))
-    out = ops().paged_attention_mfma(q.to(dev()), *args, *items_for([n], 128 // (nh // nkv)),
-                                     1.0 / math.sqrt(d), window)
-    assert rel_err(out, expect) < BF16_TOL
+    for keys, nsplit in [(0, 1), (4096, 5), (1024, 20)]:
+        out = ops().paged_attention_mfma(q.to(dev()), *args, *items_for([n], 128 // (nh // nkv)),
+                                         1.0 / math.sqrt(d), window, keys, nsplit)
+        assert rel_err(out, expect) < BF16_TOL, (keys, nsplit)
     # the last 16 tokens one by one, as a decode step of 16 requests would bring them:
     # 16 requests that share the pages but stand at different positions
     m = 16

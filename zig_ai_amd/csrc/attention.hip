@@ -300,8 +300,10 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
                             const bf16_t* __restrict__ kv, const int* __restrict__ block_table,
                             int bt_stride, const int* __restrict__ positions,
                             const int* __restrict__ wi_seq, const int* __restrict__ wi_row0,
-                            const int* __restrict__ wi_count, int n_items, int nh, int nkv,
-                            int page_size, float scale_log2e, int window) {
+                            const int* __restrict__ wi_count, int n_items,
+                            float* __restrict__ part_acc, float* __restrict__ part_ml, int nh,
+                            int nkv, int page_size, float scale_log2e, int window,
+                            int keys_per_split, int nsplit) {
   constexpr int LDK = D + 8;        // padded rows, in elements
   constexpr int LDV = AM_KT + 8;
   constexpr int KSTEPS = D / 32;    // matrix-core steps over the head dimension
@@ -359,7 +361,12 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
   const int pos_first = positions[row0];
   const int pos_last = positions[row0 + count - 1];
   const int lo = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
-  const int hi = pos_last;
+  // with nsplit > 1 this workgroup serves the keys of one range only (ranges are
+  // multiples of the tile, so a tile lies in one range); its partial result is
+  // merged with the others' by attention_combine_kernel
+  const int z = blockIdx.z;
+  int hi = pos_last;
+  if (nsplit > 1 && (z + 1) * keys_per_split - 1 < hi) hi = (z + 1) * keys_per_split - 1;
   // what this wave's rows can see
   const int wave_first_row = wave * (NS * 16);
   const bool wave_active = wave_first_row < rows;
@@ -444,8 +451,9 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
     }
   };
 
-  const int tile_first = (lo / AM_KT) * AM_KT;
-  const int n_tiles = (hi - tile_first) / AM_KT + 1;
+  int tile_first = (lo / AM_KT) * AM_KT;
+  if (nsplit > 1 && z * keys_per_split > tile_first) tile_first = z * keys_per_split;
+  const int n_tiles = hi >= tile_first ? (hi - tile_first) / AM_KT + 1 : 0;   // 0: an empty range
   load_pages(tile_first);
   load_data(tile_first);
   load_pages(tile_first + AM_KT);
@@ -479,7 +487,7 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
       }
       // a tile every key of which counts for every row of the wave needs no mask
       const bool needs_mask = !wave_full || tile0 + AM_KT - 1 > wave_lo || tile0 < lo ||
-                              (window > 0 && tile0 <= wave_hi - window);
+                              tile0 + AM_KT - 1 > hi || (window > 0 && tile0 <= wave_hi - window);
       bf16x8_t pf[NS][2];
 #pragma unroll
       for (int c = 0; c < NS; ++c) {
@@ -489,7 +497,7 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               const int kp = tile0 + jb * 16 + grp * 4 + i;
-              bool valid = kp <= pos_row[c] && kp >= lo;
+              bool valid = kp <= pos_row[c] && kp >= lo && kp <= hi;
               if (window > 0 && kp <= pos_row[c] - window) valid = false;
               if (!valid) s[c][jb][i] = -INFINITY;
             }
@@ -548,8 +556,22 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
 #pragma unroll
   for (int c = 0; c < NS; ++c)
     if (row_valid[c]) {
+      const size_t orow = (size_t)tok[c] * nh + head[c];
+      if (nsplit > 1) {
+        // unnormalised accumulator, and (maximum, sum) with the maximum turned back
+        // from the base-2 scale into the natural one the merge kernel works in
+        float* pa = part_acc + (orow * nsplit + z) * D;
+#pragma unroll
+        for (int db = 0; db < DBLK; ++db)
+          *reinterpret_cast<f32x4_t*>(pa + db * 16 + grp * 4) = o[c][db];
+        if (grp == 0) {
+          part_ml[(orow * nsplit + z) * 2] = m[c] * 0.69314718055994531f;
+          part_ml[(orow * nsplit + z) * 2 + 1] = l[c];
+        }
+        continue;
+      }
       const float inv = l[c] > 0.f ? 1.0f / l[c] : 0.f;
-      bf16_t* dst = out + ((size_t)tok[c] * nh + head[c]) * D;
+      bf16_t* dst = out + orow * D;
 #pragma unroll
       for (int db = 0; db < DBLK; ++db) {
         bf16x4_t ov;
@@ -858,9 +880,10 @@ extern "C" int za_paged_attention(const void* q, void* out, const void* kv, cons
 template <int D>
 static int launch_attention_mfma(const void* q, void* out, const void* kv, const int* block_table,
                                  int bt_stride, const int* positions, const int* wi_seq,
-                                 const int* wi_row0, const int* wi_count, int n_items, int nh,
-                                 int nkv, int page_size, float scale, int window,
-                                 hipStream_t stream) {
+                                 const int* wi_row0, const int* wi_count, int n_items,
+                                 int n_tokens, float* part_acc, float* part_ml, int nh, int nkv,
+                                 int page_size, float scale, int window, int keys_per_split,
+                                 int nsplit, hipStream_t stream) {
   constexpr int NW = 8, NS = AM_ROWS / (NW * 16);
   const size_t shmem = ((size_t)2 * AM_KT * (D + 8) + (size_t)2 * D * (AM_KT + 8)) * sizeof(bf16_t);
   auto kernel = paged_attention_mfma_kernel<D, NW, NS>;
@@ -874,23 +897,34 @@ static int launch_attention_mfma(const void* q, void* out, const void* kv, const
   if (n_items > 65535) return ZA_ERR_UNSUPPORTED;
   // the key/value head runs fastest, so that workgroups that follow each other (and
   // are dealt to the chip's eight dies in turn) read different heads' keys and values
-  dim3 grid(nkv, n_items), block(NW * 64);
+  dim3 grid(nkv, n_items, nsplit), block(NW * 64);
   hipLaunchKernelGGL(kernel, grid, block, shmem, stream, (const bf16_t*)q, (bf16_t*)out,
                      (const bf16_t*)kv, block_table, bt_stride, positions, wi_seq, wi_row0,
-                     wi_count, n_items, nh, nkv, page_size, scale * 1.44269504088896341f, window);
+                     wi_count, n_items, part_acc, part_ml, nh, nkv, page_size,
+                     scale * 1.44269504088896341f, window, keys_per_split, nsplit);
+  int rc = za_launch_status();
+  if (rc != 0 || nsplit == 1) return rc;
+  dim3 cgrid((unsigned)((size_t)n_tokens * nh)), cblock(64);
+  hipLaunchKernelGGL((attention_combine_kernel<bf16_t>), cgrid, cblock, 0, stream, part_acc,
+                     part_ml, (bf16_t*)out, D, nsplit);
   return za_launch_status();
 }
 
 // Matrix-core variant: bfloat16 only, head_dim 64 or 128, page sizes that are
 // multiples of 4, a positive scale, work items of at most 128 / (nh / nkv) query
-// tokens.  Returns ZA_ERR_UNSUPPORTED otherwise.
+// tokens; contexts optionally cut as in za_paged_attention (partial results merged by
+// the same combine kernel).  Returns ZA_ERR_UNSUPPORTED otherwise.
 extern "C" int za_paged_attention_mfma(const void* q, void* out, const void* kv,
                                        const int* block_table, int bt_stride,
                                        const int* positions, const int* wi_seq,
                                        const int* wi_row0, const int* wi_count, int n_items,
-                                       int nh, int nkv, int d, int page_size, float scale,
-                                       int window, hipStream_t stream) {
-  if (n_items == 0) return 0;
+                                       int n_tokens, float* part_acc, float* part_ml, int nh,
+                                       int nkv, int d, int page_size, float scale, int window,
+                                       int keys_per_split, int nsplit, hipStream_t stream) {
+  if (n_items == 0 || n_tokens == 0) return 0;
+  if (nsplit < 1 || nsplit > 65535 ||
+      (nsplit > 1 && (!part_acc || !part_ml || keys_per_split <= 0 || keys_per_split % 64 != 0)))
+    return ZA_ERR_ARG;
   if (n_items < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || page_size <= 0 || bt_stride <= 0 ||
       !q || !out || !kv || !block_table || !positions || !wi_seq || !wi_row0 || !wi_count)
     return ZA_ERR_ARG;
@@ -900,11 +934,11 @@ extern "C" int za_paged_attention_mfma(const void* q, void* out, const void* kv,
     return ZA_ERR_UNSUPPORTED;
   if (d == 64)
     return launch_attention_mfma<64>(q, out, kv, block_table, bt_stride, positions, wi_seq,
-                                     wi_row0, wi_count, n_items, nh, nkv, page_size, scale,
-                                     window, stream);
+                                     wi_row0, wi_count, n_items, n_tokens, part_acc, part_ml, nh,
+                                     nkv, page_size, scale, window, keys_per_split, nsplit, stream);
   return launch_attention_mfma<128>(q, out, kv, block_table, bt_stride, positions, wi_seq,
-                                    wi_row0, wi_count, n_items, nh, nkv, page_size, scale, window,
-                                    stream);
+                                    wi_row0, wi_count, n_items, n_tokens, part_acc, part_ml, nh,
+                                    nkv, page_size, scale, window, keys_per_split, nsplit, stream);
 }
 
 // Matrix-core decode variant: bfloat16, head_dim 64 or 128, page sizes that are

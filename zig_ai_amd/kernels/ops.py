@@ -38,8 +38,8 @@ _SIGNATURES = {
                                           c_int, c_int, c_int, c_void_p],
     ("attention", "za_paged_attention_mfma"): [c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                                c_void_p, c_void_p, c_void_p, c_void_p, c_int,
-                                               c_int, c_int, c_int, c_int, c_float, c_int,
-                                               c_void_p],
+                                               c_int, c_void_p, c_void_p, c_int, c_int, c_int,
+                                               c_int, c_float, c_int, c_int, c_int, c_void_p],
     ("attention", "za_paged_attention_decode_mfma"): [c_void_p, c_void_p, c_void_p, c_void_p,
                                                       c_int, c_void_p, c_void_p, c_void_p,
                                                       c_void_p, c_int, c_int, c_void_p, c_void_p,
@@ -397,11 +397,14 @@ def attention_mfma_supported(dtype: torch.dtype, num_heads: int, num_kv_heads: i
 def paged_attention_mfma(q: torch.Tensor, kv_cache: torch.Tensor, block_table: torch.Tensor,
                          positions: torch.Tensor, item_seq: torch.Tensor,
                          item_row0: torch.Tensor, item_count: torch.Tensor, n_items: int,
-                         scale: float, window: int = 0) -> torch.Tensor:
+                         scale: float, window: int = 0, keys_per_split: int = 0,
+                         nsplit: int = 1) -> torch.Tensor:
     """The same attention on the matrix cores (bfloat16, head_dim 64 or 128, at most
     16 query heads per key/value head, a page size that is a multiple of 4, a
     positive scale).  Work items hold at most
-    ``ATTENTION_MFMA_ROWS // (heads // kv_heads)`` query tokens; contexts are not cut."""
+    ``ATTENTION_MFMA_ROWS // (heads // kv_heads)`` query tokens; long contexts may be
+    cut into ``nsplit`` ranges of ``keys_per_split`` keys (a portion of a prompt far
+    into its request yields few work items)."""
     if q.dim() != 3:
         raise KernelError(f"q must be [T, heads, head_dim], got {tuple(q.shape)}")
     T, nh, d = q.shape
@@ -423,10 +426,17 @@ def paged_attention_mfma(q: torch.Tensor, kv_cache: torch.Tensor, block_table: t
         if t.numel() < n_items:
             raise KernelError(f"{name} holds {t.numel()} entries, fewer than {n_items} items")
     out = torch.empty_like(q)
+    part_acc = part_ml = None
+    if nsplit > 1:
+        if keys_per_split <= 0 or keys_per_split % 64:
+            raise KernelError("keys_per_split must be a positive multiple of 64")
+        part_acc = torch.empty((T, nh, nsplit, d), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((T, nh, nsplit, 2), dtype=torch.float32, device=q.device)
     rc = _fn("attention", "za_paged_attention_mfma")(
         _ptr(q), _ptr(out), _ptr(kv_cache), _ptr(block_table), block_table.shape[1],
-        _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, nh, nkv, d,
-        page_size, float(scale), int(window), _stream())
+        _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
+        _ptr(part_acc), _ptr(part_ml), nh, nkv, d, page_size, float(scale), int(window),
+        int(keys_per_split), int(nsplit), _stream())
     _check(rc, "paged_attention_mfma")
     return out
 

@@ -26,30 +26,29 @@ from .base import (Mixer, PagedNeed, Runtime, TensorRule, lookup, register_mixer
 from .feed_forward import fuse_rows
 
 # Cutting long contexts pays only when the launch would otherwise leave most of the
-# machine idle (decoding few requests).  Measured on one MI355X with 8 key/value
-# heads, contexts from 2,048 to 131,072 keys and 1 to 64 requests: from 512
-# workgroups on nothing is gained; below, the longest range (a power of two from
-# 256 to 8,192 keys) that still yields SPLIT_TARGET workgroups is best or within a
-# few percent of it (fewer partial results to merge).
+# machine idle (decoding few requests, or a portion of a prompt far into a long
+# request).  Measured on one MI355X with 8 key/value heads, contexts from 2,048 to
+# 131,072 keys and 1 to 64 requests: from 512 workgroups on nothing is gained; below,
+# as few ranges as still yield SPLIT_TARGET workgroups are best or within a few
+# percent of it (fewer partial results to merge), all of the same length.
 BUSY_WORKGROUPS = 512
 SPLIT_TARGET = 256
 SPLIT_KEYS_MIN = 256
 SPLIT_MAX = 64
 
 
-def plan_split(n_items: int, num_kv_heads: int, max_keys: int):
+def plan_split(n_items: int, num_kv_heads: int, max_keys: int, target: int = SPLIT_TARGET):
     """(keys per range, number of ranges) for one launch; a function of the batch
-    shape and of the longest context only."""
+    shape and of the longest context only.  ``target``: workgroups to reach (the
+    kernel for prompt portions runs two workgroups per compute unit and wants 512)."""
     groups = n_items * num_kv_heads
     if groups >= BUSY_WORKGROUPS or max_keys <= 2 * SPLIT_KEYS_MIN:
         return 0, 1
-    keys = SPLIT_KEYS_MIN
-    for cand in (8192, 4096, 2048, 1024, 512):
-        if groups * ((max_keys + cand - 1) // cand) >= SPLIT_TARGET:
-            keys = cand
-            break
-    while (max_keys + keys - 1) // keys > SPLIT_MAX:
-        keys *= 2
+    wanted = (target + groups - 1) // groups                # ranges that fill the machine
+    nsplit = min(wanted, max_keys // SPLIT_KEYS_MIN, SPLIT_MAX)
+    if nsplit <= 1:
+        return 0, 1
+    keys = ((max_keys + nsplit - 1) // nsplit + 63) // 64 * 64   # a multiple of the key tile
     nsplit = (max_keys + keys - 1) // keys
     return (keys, nsplit) if nsplit > 1 else (0, 1)
 
@@ -157,10 +156,12 @@ class GroupedQueryAttention(Mixer):
         mfma = self.mfma and cache.kv.shape[3] % 4 == 0
         if mfma and step.n_tokens > step.n_seqs:
             # prompt portions in the step: both products on the matrix cores
+            items = step.attention_items(self.mfma_rows_per_item)
+            # a portion far into a long request yields few work items: cut its context
+            keys, nsplit = plan_split(items[3], nkv, step.max_keys, target=BUSY_WORKGROUPS)
             o = ops.paged_attention_mfma(q, cache.kv, step.block_tables[cache.group],
-                                         step.positions,
-                                         *step.attention_items(self.mfma_rows_per_item),
-                                         self.scale, self.window)
+                                         step.positions, *items, self.scale, self.window,
+                                         keys, nsplit)
         elif mfma:
             # single tokens only: the matrix-core kernel whose waves split the keys
             # (every request brings one token: row i is request i, no work-item arrays)
