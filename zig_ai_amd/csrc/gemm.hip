@@ -3,15 +3,17 @@
 // layout the reference hands to its library GEMM:
 // /root/reference/src/matmul/root.zig:292-313).
 //
-//   gemm_f32_kernel          true 32-bit: LDS-tiled FMA, no matrix-core rounding modes
-//   gemm_bf16_mfma_kernel    bfloat16 operands on the matrix cores (16x16x32), any M
-//   gemm_bf16_skinny_kernel  bfloat16, M <= 64: streams W once, K split over the waves
-//   gemm_bf16_rows16_kernel  bfloat16, M <= 16 (decoding): activations held in registers
+//   gemm_f32_kernel                 true 32-bit: LDS-tiled FMA, no matrix-core rounding modes
+//   gemm_bf16_mfma_kernel           bfloat16 operands on the matrix cores (16x16x32), any M
+//   gemm_bf16_skinny_kernel         bfloat16, M <= 64: streams W once, K split over the waves
+//   gemm_bf16_rows16_kernel         bfloat16, M <= 16 (decoding): activations held in registers
+//   gemm_bf16_rows16_swiglu_kernel  the same for the fused gate/up projection: writes
+//                                   silu(gate) * up instead of the two products
 //
-// In all three every output element is a sum over k in an order that depends
-// only on K, never on M or on the tile it falls in, so a token's result does
-// not depend on which other tokens share the step (the skinny and the tiled
-// bfloat16 kernels differ from each other in rounding only).
+// In every one of them an output element is a sum over k in an order that
+// depends only on K, never on M or on the tile it falls in, so a token's result
+// does not depend on which other tokens share the step (the bfloat16 kernels
+// differ from each other in rounding only).
 #include "common.h"
 
 // ---------------------------------------------------------------- 32-bit FMA
