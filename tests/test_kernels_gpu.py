@@ -147,31 +147,51 @@ def test_gemm_bf16(M, N, K, out_dtype):
 
 @pytest.mark.parametrize("M", [1, 16, 40, 64])
 def test_gemm_bf16_skinny_and_tiled_agree(M):
-    """The two bfloat16 kernels may differ in rounding only."""
-    x, w = rand((M, 512), torch.bfloat16, 16), rand((96, 512), torch.bfloat16, 17)
-    a = ops().linear(x.to(dev()), w.to(dev()), out_dtype=torch.float32)
-    b = ops().linear(x.to(dev()), w.to(dev()), out_dtype=torch.float32, force_tiled=True)
-    assert rel_err(a, b.double()) < F32_TOL
+    """The bfloat16 kernels may differ in rounding only (a bias keeps the product
+    in this package's kernels at every M)."""
+    x, w, b = rand((M, 512), torch.bfloat16, 16), rand((96, 512), torch.bfloat16, 17), rand((96,), torch.float32, 15)
+    a = ops().linear(x.to(dev()), w.to(dev()), b.to(dev()), out_dtype=torch.float32)
+    c = ops().linear(x.to(dev()), w.to(dev()), b.to(dev()), out_dtype=torch.float32, force_tiled=True)
+    assert rel_err(a, c.double()) < F32_TOL
+
+
+@pytest.mark.parametrize("M", [17, 40, 64, 65, 300])
+@pytest.mark.parametrize("N,K", [(50, 96), (257, 1024), (2048, 2048), (1000, 4096)])
+def test_gemm_bf16_library_keeps_32_bits(M, N, K):
+    """More rows than a decode batch, no bias: the library's product.  Asked for a
+    32-bit result it must give the 32-bit sums, not a bfloat16 result widened: the
+    error against 64-bit is that of 32-bit summation."""
+    x, w = rand((M, K), torch.bfloat16, 40), rand((N, K), torch.bfloat16, 41)
+    out = ops().linear(x.to(dev()), w.to(dev()), out_dtype=torch.float32)
+    assert out.dtype == torch.float32 and out.shape == (M, N)
+    assert rel_err(out, x.double() @ w.double().T) < F32_TOL
+    low = ops().linear(x.to(dev()), w.to(dev()))
+    assert low.dtype == torch.bfloat16
+    assert rel_err(low, x.double() @ w.double().T) < BF16_TOL
 
 
 def test_gemm_rows_do_not_depend_on_batch():
     """A token's projection is the same whatever else is in the step: bitwise
-    within one kernel (each sums over k in an order fixed by K alone), within
-    rounding between kernels."""
+    within one of this package's kernels (each sums over k in an order fixed by K
+    alone), within rounding between kernels and in the library."""
     x, w = rand((64, 256), torch.bfloat16, 18), rand((80, 256), torch.bfloat16, 19)
+    bias = rand((80,), torch.float32, 20).to(dev())
 
     def run(m, **kw):
         return ops().linear(x[:m].contiguous().to(dev()), w.to(dev()), out_dtype=torch.float32, **kw).cpu()
 
-    for group in ((1, 5, 16), (17, 33, 64)):              # the kernels' ranges of M
-        full = run(group[-1])
-        for m in group[:-1]:
-            assert torch.equal(run(m), full[:m])
+    full = run(16)
+    for m in (1, 5):
+        assert torch.equal(run(m), full[:m])
+    full = run(64, bias=bias)                            # with a bias: the kernel for 17..64 rows
+    for m in (17, 33):
+        assert torch.equal(run(m, bias=bias), full[:m])
     tiled = run(64, force_tiled=True)
     for m in (3, 40):
         assert torch.equal(run(m, force_tiled=True), tiled[:m])
     assert rel_err(run(16), tiled[:16].double()) < F32_TOL
-    assert rel_err(run(64), tiled.double()) < F32_TOL
+    for m in (17, 33, 64):                               # the library
+        assert rel_err(run(m), tiled[:m].double()) < F32_TOL
     x32, w32 = x.float(), w.float()
     full32 = ops().linear(x32.to(dev()), w32.to(dev())).cpu()
     part32 = ops().linear(x32[:3].contiguous().to(dev()), w32.to(dev())).cpu()
@@ -195,8 +215,45 @@ def test_gemm_bf16_partial_sums(M, N, K):
     stack = ops().linear(x.to(dev()), w.to(dev()), b.to(dev()), partial_ok=True)
     assert stack.dim() == 3 and stack.dtype == torch.float32 and stack.shape[0] in (2, 4)
     assert rel_err(stack.sum(0), x.double() @ w.double().T + b.double()) < F32_TOL
-    big = ops().linear(rand((40, K), torch.bfloat16, 33).to(dev()), w.to(dev()), partial_ok=True)
-    assert big.dim() == 2                                   # only decode batches are split
+    many = ops().linear(rand((600, K), torch.bfloat16, 33).to(dev()), w.to(dev()), partial_ok=True)
+    assert many.dim() == 2                                  # only small batches are split
+
+
+@pytest.mark.parametrize("M", [17, 40, 64, 200])
+@pytest.mark.parametrize("N,K,few_rows,more_rows", [
+    (2048, 8192, 8, 8), (2048, 2048, 8, 1), (300, 4096, 8, 8), (1024, 4608, 4, 4),
+    (2048, 4160, 1, 1), (6144, 2048, 1, 1), (64, 1024, 1, 1)])
+def test_gemm_bf16_library_partial_sums(M, N, K, few_rows, more_rows):
+    """Beyond a decode batch the library is given K in ranges when N is small (up
+    to 64 rows from K = 2048 on, up to LIBRARY_SPLIT_ROWS rows from 4096 on): the
+    stack of 32-bit partial results sums to the product."""
+    x, w = rand((M, K), torch.bfloat16, 42), rand((N, K), torch.bfloat16, 43)
+    out = ops().linear(x.to(dev()), w.to(dev()), partial_ok=True)
+    expect = x.double() @ w.double().T
+    split = few_rows if M <= 64 else more_rows
+    if split > 1:
+        assert out.dim() == 3 and out.dtype == torch.float32 and out.shape == (split, M, N)
+        assert out.is_contiguous()
+        assert rel_err(out.sum(0), expect) < F32_TOL
+        part = x[:, :K // split].double() @ w[:, :K // split].double().T
+        assert rel_err(out[0], part) < F32_TOL
+    else:
+        assert out.shape == (M, N) and out.dtype == torch.bfloat16
+        assert rel_err(out, expect) < BF16_TOL
+
+
+@pytest.mark.parametrize("M,N,K,split", [(8, 2048, 2048, 2), (16, 1024, 3072, 2), (1, 2048, 2080, 1),
+                                         (8, 6144, 2048, 1), (4, 64, 1024, 1)])
+def test_gemm_bf16_decode_rows_split_short_k(M, N, K, split):
+    x, w = rand((M, K), torch.bfloat16, 44), rand((N, K), torch.bfloat16, 45)
+    out = ops().linear(x.to(dev()), w.to(dev()), partial_ok=True)
+    expect = x.double() @ w.double().T
+    if split > 1:
+        assert out.shape == (split, M, N) and out.dtype == torch.float32
+        assert rel_err(out.sum(0), expect) < F32_TOL
+    else:
+        assert out.shape == (M, N) and out.dtype == torch.bfloat16
+        assert rel_err(out, expect) < BF16_TOL
 
 
 @pytest.mark.parametrize("M,I,K", [(1, 48, 64), (8, 8192, 2048), (16, 100, 520), (5, 176, 96),

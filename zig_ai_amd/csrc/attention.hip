@@ -257,7 +257,6 @@ attention_combine_kernel(const float* __restrict__ part_acc, const float* __rest
 #define AM_KT 64
 #define AM_ROWS 128
 
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
 
 // A query row's scores for a tile are spread over the four lanes l, l ^ 16, l ^ 32,
 // l ^ 48.  The swap instructions exchange 16-lane rows (odd rows of the first operand

@@ -10,6 +10,7 @@
 typedef __bf16 bf16_t;
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 // Every launcher returns 0 on success or a hipError_t; bad arguments return one

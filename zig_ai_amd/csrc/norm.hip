@@ -13,12 +13,61 @@
 
 // `delta` may be a stack of `n_partials` partial sums (each `partial_stride`
 // elements apart): the pieces a projection split along K leaves to its consumer.
+// They are added up first, in their order, and the sum is added to the residual.
 template <typename TD>
 __device__ __forceinline__ float delta_at(const TD* dl, size_t i, int n_partials,
                                           size_t partial_stride) {
   float v = to_f32<TD>(dl[i]);
   for (int p = 1; p < n_partials; ++p) v += to_f32<TD>(dl[i + p * partial_stride]);
   return v;
+}
+
+// Four consecutive elements as floats; `p` aligned to four elements.
+template <typename T> __device__ __forceinline__ void load4(const T* p, float out[4]);
+template <> __device__ __forceinline__ void load4<float>(const float* p, float out[4]) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w;
+}
+template <> __device__ __forceinline__ void load4<bf16_t>(const bf16_t* p, float out[4]) {
+  const bf16x4_t v = *reinterpret_cast<const bf16x4_t*>(p);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) out[i] = (float)v[i];
+}
+template <typename T> __device__ __forceinline__ void store4(T* p, const float in[4]);
+template <> __device__ __forceinline__ void store4<float>(float* p, const float in[4]) {
+  *reinterpret_cast<float4*>(p) = make_float4(in[0], in[1], in[2], in[3]);
+}
+template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, const float in[4]) {
+  bf16x4_t v;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v[i] = (bf16_t)in[i];
+  *reinterpret_cast<bf16x4_t*>(p) = v;
+}
+
+// The same sum as delta_at for the four elements at `i`, with the loads of up to
+// eight partial sums issued before the first is waited for.
+template <typename TD>
+__device__ __forceinline__ void delta4_at(const TD* dl, size_t i, int n_partials,
+                                          size_t partial_stride, float v[4]) {
+  load4<TD>(dl + i, v);
+  for (int p0 = 1; p0 < n_partials; p0 += 8) {
+    float t[8][4];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      if (p0 + q < n_partials) {
+        load4<TD>(dl + i + (size_t)(p0 + q) * partial_stride, t[q]);
+      } else {
+        t[q][0] = t[q][1] = t[q][2] = t[q][3] = 0.f;
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      if (p0 + q < n_partials) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] += t[q][e];
+      }
+    }
+  }
 }
 
 // General form: two passes over the row, any width.
@@ -83,8 +132,10 @@ add_rmsnorm_regs_kernel(float* __restrict__ residual, const TD* __restrict__ del
         h[v][0] = h[v][1] = h[v][2] = h[v][3] = 0.f;
       }
       if (dl) {
+        float d4[4];
+        delta4_at<TD>(dl, i, n_partials, partial_stride, d4);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) h[v][e] += delta_at<TD>(dl, i + e, n_partials, partial_stride);
+        for (int e = 0; e < 4; ++e) h[v][e] += d4[e];
       }
       if (write_residual)
         *reinterpret_cast<float4*>(x + i) = make_float4(h[v][0], h[v][1], h[v][2], h[v][3]);
@@ -99,10 +150,9 @@ add_rmsnorm_regs_kernel(float* __restrict__ residual, const TD* __restrict__ del
     const int i = (threadIdx.x + v * 256) * 4;
     if (i < width) {
       const float4 w = *reinterpret_cast<const float4*>(weight + i);
-      o[i] = from_f32<TO>(h[v][0] * scale * w.x);
-      o[i + 1] = from_f32<TO>(h[v][1] * scale * w.y);
-      o[i + 2] = from_f32<TO>(h[v][2] * scale * w.z);
-      o[i + 3] = from_f32<TO>(h[v][3] * scale * w.w);
+      const float y[4] = {h[v][0] * scale * w.x, h[v][1] * scale * w.y, h[v][2] * scale * w.z,
+                          h[v][3] * scale * w.w};
+      store4<TO>(o + i, y);
     }
   }
 }

@@ -177,6 +177,9 @@ def embed_gather(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
 # Above this many rows a bfloat16 projection without bias goes to the library
 # (measured: the decode kernel wins up to 16 rows, the library from there on).
 LIBRARY_GEMM_ROWS = 16
+# Up to this many rows the library is given K in ranges when the consumer takes
+# partial sums (a decode batch is too few rows to fill the chip with tiles of N alone).
+LIBRARY_SPLIT_ROWS = 512
 
 
 def check_projection_weight(weight: torch.Tensor, what: str) -> None:
@@ -189,14 +192,33 @@ def check_projection_weight(weight: torch.Tensor, what: str) -> None:
 
 
 def _k_splits(M: int, N: int, K: int) -> int:
-    """Into how many ranges the decode kernel cuts K when its consumer accepts
-    partial sums: enough to give every compute unit work when N alone is too
-    small, each range at least 512 long."""
-    if M > 16 or N > 4096 or K < 4096:
-        return 1       # measured: below this the consumer's extra reads cost more than is won
-    for split in (4, 2):
-        if K % (split * 32) == 0:
-            return split
+    """Into how many ranges K is cut when the consumer accepts partial sums:
+    enough to give every compute unit work when N alone is too small.  Measured
+    together with the norm that adds the stack up, N = 2048:
+
+    * up to 16 rows (the decode kernel): 4 ranges from K = 4096 on (8192: 15 us
+      instead of 19.5), 2 ranges from 2048 on (8.3 instead of 8.9);
+    * more rows (the library, as one batched product over the ranges): 8 ranges
+      from K = 4096 on up to ``LIBRARY_SPLIT_ROWS`` rows (64 rows: 18 us instead
+      of 26; 512 rows: 33 instead of 41), and from K = 2048 on up to 64 rows
+      (12 instead of 13; no gain with more rows)."""
+    if N > 4096:
+        return 1
+    if M <= 16:
+        if K >= 4096:
+            choices = (4, 2)
+        elif K >= 2048 and N <= 2048:
+            choices = (2,)
+        else:
+            return 1
+        for split in choices:
+            if K % (split * 32) == 0:
+                return split
+        return 1
+    if M <= LIBRARY_SPLIT_ROWS and (K >= 4096 or (K >= 2048 and M <= 64)):
+        for split in (8, 4, 2):
+            if K % (split * 128) == 0:
+                return split
     return 1
 
 
@@ -206,14 +228,15 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     """``x [M, K] @ weight[N, K]^T + bias`` with 32-bit accumulation.
 
     bfloat16 weights use the matrix-core kernels of csrc/gemm.hip up to
-    ``LIBRARY_GEMM_ROWS`` rows (a decode batch), and always when a bias or 32-bit
-    output is asked for; larger plain products go to the GEMM library.  32-bit weights use the
-    all-32-bit kernel (``x`` may be either type and is widened): no library, no
-    reduced-precision matrix mode.
+    ``LIBRARY_GEMM_ROWS`` rows (a decode batch), and always when a bias is asked
+    for; larger plain products go to the GEMM library, with bfloat16 or 32-bit
+    output.  32-bit weights use the all-32-bit kernel (``x`` may be either type and
+    is widened): no library, no reduced-precision matrix mode.
 
     With ``partial_ok`` the result may come back as a stack ``[P, M, N]`` of 32-bit
-    partial sums (K split over more workgroups when N is small and M is a decode
-    batch); ``add_rmsnorm`` adds such a stack up while it reads it."""
+    partial sums (K cut into ranges, for more workgroups, when N is small and M is
+    at most ``LIBRARY_SPLIT_ROWS``); ``add_rmsnorm`` adds such a stack up while it
+    reads it."""
     if x.dim() != 2 or weight.dim() != 2:
         raise KernelError(f"linear takes x [M, K] and weight [N, K], got {tuple(x.shape)} and "
                           f"{tuple(weight.shape)}")
@@ -224,33 +247,43 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     if bias is not None:
         _need(bias, "bias", torch.float32, (N,))
     out_dtype = out_dtype or x.dtype
-    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     if weight.dtype == torch.float32:
+        out = torch.empty((M, N), dtype=out_dtype, device=x.device)
         rc = _fn("gemm", "za_gemm_f32")(_ptr(x), _code(x.dtype), _ptr(weight), _ptr(bias), _ptr(out),
                                         _code(out_dtype), M, N, K, _stream())
         _check(rc, "gemm_f32", f"M={M} N={N} K={K}")
-    else:
-        if x.dtype != torch.bfloat16:
-            raise KernelError("a bfloat16 weight needs bfloat16 activations")
-        if K % 8:
-            raise KernelError(f"the bfloat16 GEMM needs K to be a multiple of 8, got K={K}")
-        splits = _k_splits(M, N, K) if (partial_ok and not force_tiled and K <= 8192 * 4) else 1
-        if splits > 1:
-            stack = torch.empty((splits, M, N), dtype=torch.float32, device=x.device)
-            rc = _fn("gemm", "za_gemm_bf16_rows16")(_ptr(x), _ptr(weight), _ptr(bias), _ptr(stack),
-                                                    0, M, N, K, splits, 0, _stream())
-            _check(rc, "gemm_bf16_rows16", f"M={M} N={N} K={K} splits={splits}")
-            return stack
-        if M > LIBRARY_GEMM_ROWS and bias is None and out_dtype == torch.bfloat16 \
-                and not force_tiled:
-            # Many rows: the vendor's GEMM library, as the reference does for every
-            # projection (/root/reference/src/matmul/root.zig:292-313 calls cuBLAS).
-            torch.mm(x, weight.t(), out=out)
-            return out
-        rc = _fn("gemm", "za_gemm_bf16")(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out),
-                                         _code(out_dtype), M, N, K, 1 if force_tiled else 0,
-                                         _stream())
-        _check(rc, "gemm_bf16", f"M={M} N={N} K={K}")
+        return out
+    if x.dtype != torch.bfloat16:
+        raise KernelError("a bfloat16 weight needs bfloat16 activations")
+    if K % 8:
+        raise KernelError(f"the bfloat16 GEMM needs K to be a multiple of 8, got K={K}")
+    # Many rows: the vendor's GEMM library, as the reference does for every
+    # projection (/root/reference/src/matmul/root.zig:292-313 calls cuBLAS).
+    library = M > LIBRARY_GEMM_ROWS and bias is None and not force_tiled \
+        and out_dtype in (torch.bfloat16, torch.float32)
+    splits = 1
+    if partial_ok and not force_tiled and K <= 8192 * 4 and (M <= 16 or library):
+        splits = _k_splits(M, N, K)
+    if splits > 1 and M <= 16:
+        stack = torch.empty((splits, M, N), dtype=torch.float32, device=x.device)
+        rc = _fn("gemm", "za_gemm_bf16_rows16")(_ptr(x), _ptr(weight), _ptr(bias), _ptr(stack),
+                                                0, M, N, K, splits, 0, _stream())
+        _check(rc, "gemm_bf16_rows16", f"M={M} N={N} K={K} splits={splits}")
+        return stack
+    if splits > 1:
+        # One batched product over the ranges of K: [P, M, K/P] x [P, K/P, N], both views.
+        xs = x.view(M, splits, K // splits).transpose(0, 1)
+        ws = weight.view(N, splits, K // splits).permute(1, 2, 0)
+        return torch.bmm(xs, ws, out_dtype=torch.float32)
+    if library:
+        if out_dtype == torch.float32:
+            return torch.mm(x, weight.t(), out_dtype=torch.float32)
+        return torch.mm(x, weight.t())
+    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    rc = _fn("gemm", "za_gemm_bf16")(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out),
+                                     _code(out_dtype), M, N, K, 1 if force_tiled else 0,
+                                     _stream())
+    _check(rc, "gemm_bf16", f"M={M} N={N} K={K}")
     return out
 
 
