@@ -661,12 +661,24 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
   const int ps_shift = page_shift_of(page_size);
   auto fetch = [&](int tile0, bf16x8_t (&kfr)[4][KSTEPS], bf16x4_t (&vfr)[DBLK][4]) {
     int kpage[4], vpage[4];
+    if (ps_shift >= 4) {
+      // Tiles start at multiples of 16 keys, so with pages of 16, 32, 64 ... keys a
+      // block of 16 keys lies in one page: one entry for the whole wave, which the
+      // scalar unit reads without waiting for the vector loads in flight.
+      const int t0 = __builtin_amdgcn_readfirstlane(tile0);
 #pragma unroll
-    for (int jb = 0; jb < 4; ++jb) {
-      const int e = page_entry(tile0 + jb * 16 + r16, page_size, ps_shift);
-      kpage[jb] = table[e < last_entry ? e : last_entry];
-      const int ev = page_entry(tile0 + jb * 16 + grp * 4, page_size, ps_shift);
-      vpage[jb] = table[ev < last_entry ? ev : last_entry];
+      for (int jb = 0; jb < 4; ++jb) {
+        const int e = (t0 + jb * 16) >> ps_shift;
+        kpage[jb] = vpage[jb] = table[e < last_entry ? e : last_entry];
+      }
+    } else {
+#pragma unroll
+      for (int jb = 0; jb < 4; ++jb) {
+        const int e = page_entry(tile0 + jb * 16 + r16, page_size, ps_shift);
+        kpage[jb] = table[e < last_entry ? e : last_entry];
+        const int ev = page_entry(tile0 + jb * 16 + grp * 4, page_size, ps_shift);
+        vpage[jb] = table[ev < last_entry ? ev : last_entry];
+      }
     }
 #pragma unroll
     for (int jb = 0; jb < 4; ++jb) {
