@@ -15,13 +15,14 @@ import torch
 
 import engine_util as eu
 import plain_lfm2 as plain
-from tiny_configs import REAL_2L, TINY_A, TINY_B, TINY_C, TINY_D, TINY_E
+from tiny_configs import REAL_2L, TINY_A, TINY_B, TINY_C, TINY_D, TINY_E, TINY_F
 
 pytestmark = pytest.mark.gpu
 
 TOL = {"float32": 1e-4, "bfloat16": 2.5e-2}
-CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3)}
-LENGTHS = {"A": [5, 17, 33, 70], "B": [1, 8, 31, 64, 100], "C": [40, 3, 77], "D": [150, 9, 66, 40]}
+CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3), "F": (TINY_F, 5)}
+LENGTHS = {"A": [5, 17, 33, 70], "B": [1, 8, 31, 64, 100], "C": [40, 3, 77], "D": [150, 9, 66, 40],
+           "F": [130, 20, 75]}
 
 _cache = {}
 
@@ -54,7 +55,7 @@ def check(got, expect, dtype, what):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "F"])
 def test_whole_requests(name, dtype):
     model, expect, prompts = setup(name, dtype)
     runner = runner_for(model, 16, 16)
@@ -65,7 +66,7 @@ def test_whole_requests(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "F"])
 def test_bulk_then_last_32_one_by_one(name, dtype):
     model, expect, prompts = setup(name, dtype)
     runner = runner_for(model, 4 if name == "A" else 8, 64)
@@ -74,7 +75,7 @@ def test_bulk_then_last_32_one_by_one(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "F"])
 def test_portions_of_changing_size(name, dtype):
     model, expect, prompts = setup(name, dtype)
     for seed in (0, 3):
@@ -84,7 +85,7 @@ def test_portions_of_changing_size(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "F"])
 def test_mixed_steps_with_page_reuse(name, dtype):
     model, expect, prompts = setup(name, dtype)
     # the same requests twice over, so that late ones land on pages early ones used

@@ -44,6 +44,18 @@ TINY_D = {
     "tie_embedding": True, "max_position_embeddings": 4096,
 }
 
+# head_dim 128 on the matrix-core attention kernels, three query heads per group, a
+# head width that is not the hidden size's share
+TINY_F = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 192, "num_hidden_layers": 2, "num_attention_heads": 3,
+    "num_key_value_heads": 1, "head_dim": 128, "vocab_size": 520,
+    "layer_types": ["conv", "full_attention"],
+    "intermediate_size": 264,
+    "rope_theta": 100000.0, "norm_eps": 2e-5, "conv_L_cache": 4, "conv_bias": True,
+    "tie_embedding": False, "max_position_embeddings": 2048,
+}
+
 # two layers at the sizes of the LFM2-1.2B shape: the kernels' large-size paths
 REAL_2L = {
     "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
