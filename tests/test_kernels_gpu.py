@@ -723,7 +723,7 @@ def test_argmax_long_rows(rows, vocab):
     assert out[0] == 7
 
 
-@pytest.mark.parametrize("vocab", [50, 1000, 65536])
+@pytest.mark.parametrize("vocab", [50, 1000, 1003, 65536])
 def test_sample_matches_plain(vocab):
     R = 12
     logits = rand((R, vocab), torch.float32, 101, 3.0)
@@ -746,6 +746,67 @@ def test_sample_matches_plain(vocab):
             cdf = torch.cumsum(e, 0) / e.sum()
             lo = float(cdf[out[r] - 1]) if out[r] > 0 else 0.0
             assert lo - 1e-5 <= float(u[r]) <= float(cdf[out[r]]) + 1e-5, (r, out[r], want)
+
+
+def sample_settings(R, vocab, seed):
+    g = torch.Generator().manual_seed(seed)
+    temps = torch.tensor([0.3, 0.7, 1.0, 1.7])[torch.randint(0, 4, (R,), generator=g)]
+    ks = torch.tensor([0, 1, 2, 7, 50, 1000, vocab - 1, vocab + 5])[torch.randint(0, 8, (R,), generator=g)]
+    ps = torch.tensor([1.0, 0.999, 0.95, 0.9, 0.5, 0.1, 1e-6, 0.0])[torch.randint(0, 8, (R,), generator=g)]
+    u = torch.rand(R, generator=g)
+    return temps, ks.clamp(max=2 ** 31 - 1).to(torch.int32), ps, u
+
+
+@pytest.mark.parametrize("vocab", [640, 4099, 65536, 200003])
+@pytest.mark.parametrize("ties", [False, True])
+def test_sample_thresholds_two_ways_agree(vocab, ties):
+    """The thresholds of top-k and top-p are searched in one bin's values or, for a
+    bin too full, over the whole row; probability mass is summed in integers, so
+    both find the same key: the same tokens, exactly.  With logits rounded to
+    halves, bins hold thousands of equal values and the first way gives up."""
+    R = 32
+    logits = rand((R, vocab), torch.float32, 110, 3.0)
+    if ties:
+        logits = torch.round(logits * 2) / 2
+    logits[3, ::2] = float("-inf")
+    temps, ks, ps, u = sample_settings(R, vocab, 111)
+    args = [t.to(dev()) for t in (logits, temps, ks, ps, u)]
+    fast = ops().sample(*args).cpu()
+    slow = ops().sample(*args, whole_row_only=True).cpu()
+    assert torch.equal(fast, slow)
+    for r in range(R):                                  # and the token is one the plain rule keeps
+        v = logits[r].double() / float(temps[r])
+        keep = plain.kept_after_top_k_top_p(v, int(ks[r]), float(ps[r]))
+        tok = int(fast[r])
+        if not bool(keep[tok]):
+            # only a value within rounding of the threshold may differ
+            edge = v[keep].min()
+            assert abs(float(v[tok] - edge)) <= 1e-5 * max(1.0, abs(float(edge))), (r, tok)
+
+
+def test_sample_flat_and_tied_rows():
+    """All values equal: top-k keeps them all (ties with the k-th are kept), and the
+    draw walks the row in index order.  Five values tied for third place: all five
+    stay candidates."""
+    vocab = 65536
+    logits = torch.zeros((4, vocab))
+    u = torch.tensor([0.0, 0.25, 0.5, 0.999])
+    out = ops().sample(logits.to(dev()), torch.ones(4, device=dev()),
+                       torch.full((4,), 10, dtype=torch.int32, device=dev()),
+                       torch.ones(4, device=dev()), u.to(dev())).cpu().tolist()
+    for r in range(4):
+        want = max(0, int(math.ceil(float(u[r]) * vocab)) - 1)
+        assert abs(out[r] - want) <= 1, (r, out[r], want)
+    n = 512
+    row = torch.full((vocab,), -5.0)
+    row[[11, 70000 % vocab]] = 4.0
+    tied = [5, 1000, 30000, 50000, 65535]
+    row[tied] = 3.0
+    us = (torch.arange(n, dtype=torch.float32) + 0.5) / n
+    out = ops().sample(row.repeat(n, 1).to(dev()), torch.ones(n, device=dev()),
+                       torch.full((n,), 3, dtype=torch.int32, device=dev()),
+                       torch.ones(n, device=dev()), us.to(dev())).cpu().tolist()
+    assert set(out) == set(tied) | {11, 70000 % vocab}
 
 
 def test_sample_distribution():

@@ -57,7 +57,7 @@ _SIGNATURES = {
     ("gemm", "za_gemm_bf16_rows16_swiglu"): [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                              c_void_p],
     ("sampling", "za_sample"): [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
-                                c_void_p, c_void_p],
+                                c_void_p, c_int, c_void_p],
     ("sampling", "za_repetition_penalty"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                                             c_void_p],
 }
@@ -598,8 +598,8 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
         raise KernelError("argmax takes [rows, vocab]")
     R, V = logits.shape
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
-    # few rows of a long vocabulary: cut each row so that the machine is busy
-    chunks = 1 if R >= 64 else max(1, min(64, V // 4096))
+    # few rows of a long vocabulary: cut each row so that some 512 workgroups run
+    chunks = max(1, min((512 + R - 1) // R, 64, V // 4096))
     part_v = part_i = None
     if chunks > 1:
         part_v = torch.empty((R, chunks), dtype=torch.float32, device=logits.device)
@@ -611,7 +611,10 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
-           top_p: torch.Tensor, uniform: torch.Tensor) -> torch.Tensor:
+           top_p: torch.Tensor, uniform: torch.Tensor, whole_row_only: bool = False) -> torch.Tensor:
+    """One token per row: greedy where temperature <= 0, else temperature, top-k, top-p
+    and a draw with the row's uniform number; see csrc/sampling.hip.  ``whole_row_only``
+    makes the kernel search its thresholds the slow way only (tests compare the two)."""
     _need(logits, "logits", torch.float32)
     if logits.dim() != 2:
         raise KernelError("sample takes [rows, vocab]")
@@ -622,8 +625,9 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     _need(uniform, "uniform", torch.float32, (R,))
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
     rc = _fn("sampling", "za_sample")(_ptr(logits), R, logits.shape[1], _ptr(temperature),
-                                      _ptr(top_k), _ptr(top_p), _ptr(uniform), _ptr(out), _stream())
-    _check(rc, "sample")
+                                      _ptr(top_k), _ptr(top_p), _ptr(uniform), _ptr(out),
+                                      1 if whole_row_only else 0, _stream())
+    _check(rc, "sample", f"rows={R} vocab={logits.shape[1]}")
     return out
 
 
