@@ -95,7 +95,16 @@ def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else c_void_p(t.data_ptr())
 
 
+# The current stream's handle, asked for before every launch: torch's binding that
+# returns the raw handle costs a fraction of a microsecond, building a Stream object
+# some eight; the latter is the fallback where the binding is missing.
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream():
+    if _raw_stream is not None and _raw_device is not None:
+        return c_void_p(_raw_stream(_raw_device()))
     return c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
