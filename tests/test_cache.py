@@ -172,3 +172,31 @@ def test_random_orders_keep_the_books(seed):
     assert all(g.pool.free_count == g.pool.size for g in m.groups)
     assert m.slots.free_count == 5
     assert m.pages_reused > 0
+
+
+def test_scattered_pools_hand_out_every_page_once():
+    """A cache made with scatter_pages hands its pages out in a fixed shuffled order:
+    every page exactly once, the same order in every cache of that size, and the
+    books stay right when pages come back."""
+    orders = []
+    for _ in range(2):
+        m = CacheManager({0: PagedNeed(1, 16)}, 4, 257, 2, allocate=False, scatter_pages=True)
+        m.admit("r")
+        m.reserve("r", 257 * 4)
+        order = m.table("r", 0)
+        assert sorted(order) == list(range(257))
+        m.admit("s")
+        with pytest.raises(OutOfPages):
+            m.reserve("s", 1)
+        m.release("r")
+        m.check()
+        assert m.groups[0].pool.free_count == 257
+        orders.append(order)
+    assert orders[0] == orders[1]
+    assert orders[0] != list(range(257))
+    runs = sum(1 for a, b in zip(orders[0], orders[0][1:]) if b == a + 1)
+    assert runs < 16                                   # no long stretches in address order
+    plain = CacheManager({0: PagedNeed(1, 16)}, 4, 257, 2, allocate=False)
+    plain.admit("r")
+    plain.reserve("r", 40)
+    assert plain.table("r", 0) == list(range(10))      # the default: 0, 1, 2 ...

@@ -73,10 +73,12 @@ class CacheManager:
 
     def __init__(self, needs: Mapping[int, object], page_size: int, num_pages, num_slots: int,
                  device: Optional[torch.device] = None, dtype: torch.dtype = torch.bfloat16,
-                 allocate: bool = True):
+                 allocate: bool = True, scatter_pages: bool = False):
         """``needs``: cache id -> PagedNeed | StateNeed | None.  ``num_pages``: an int
         (every group gets that many) or a mapping from group key
-        ``(kv_heads, head_dim, window)`` to a count."""
+        ``(kv_heads, head_dim, window)`` to a count.  ``scatter_pages``: fresh pools hand
+        their pages out in a fixed pseudo-random order rather than 0, 1, 2 ..., so that
+        requests filled one after the other do not lie a constant distance apart."""
         if page_size <= 0:
             raise ValueError("page_size must be positive")
         self.page_size = page_size
@@ -116,7 +118,8 @@ class CacheManager:
         G = len(group_needs)
         windows = (ctypes.c_int * max(G, 1))(*[n.window for n in group_needs])
         pages = (ctypes.c_int * max(G, 1))(*group_pages)
-        self._ptr = self._lib.za_cache_new(G, windows, pages, int(page_size), int(num_slots))
+        self._ptr = self._lib.za_cache_new(G, windows, pages, int(page_size), int(num_slots),
+                                           1 if scatter_pages else 0)
         if not self._ptr:
             raise ValueError("the host library refused the cache's sizes")
         self.groups: List[PagedGroup] = [

@@ -147,9 +147,11 @@ class DecoderModel:
         model.config = config
         return model
 
-    def make_cache(self, page_size: int, num_pages, num_slots: int) -> CacheManager:
+    def make_cache(self, page_size: int, num_pages, num_slots: int,
+                   scatter_pages: bool = True) -> CacheManager:
         return CacheManager(self.cache_needs, page_size, num_pages, num_slots,
-                            device=self.runtime.device, dtype=self.runtime.dtype)
+                            device=self.runtime.device, dtype=self.runtime.dtype,
+                            scatter_pages=scatter_pages)
 
     def cache_views(self, cache: CacheManager) -> List[CacheView]:
         """One view per run-order entry."""

@@ -28,7 +28,7 @@ _SIGNATURES = {
     "za_pool_check": (c_int, [c_void_p]),
     "za_pool_stats": (None, [c_void_p, _P(c_longlong)]),
     "za_pool_owner": (c_int, [c_void_p, c_int, _P(c_int64)]),
-    "za_cache_new": (c_void_p, [c_int, _P(c_int), _P(c_int), c_int, c_int]),
+    "za_cache_new": (c_void_p, [c_int, _P(c_int), _P(c_int), c_int, c_int, c_int]),
     "za_cache_free": (None, [c_void_p]),
     "za_cache_pool": (c_void_p, [c_void_p, c_int]),
     "za_cache_admit": (c_int, [c_void_p, c_int64, _P(c_int)]),
