@@ -256,6 +256,45 @@ def test_real_layer_sizes(dtype):
     check(got, expect, dtype, "portions beside single tokens")
 
 
+def test_graph_replays_with_library_products():
+    """Decode batches beyond 16 rows send their projections to the GEMM library (K in
+    ranges as a batched product where N is small, 32-bit logits): such steps are
+    recorded too.  Every replay, with eager work and synchronisations between the
+    replays, must give what the same step gives unrecorded."""
+    from zig_ai_amd.engine import DecoderModel, ModelRunner, StepEntry
+    folder = eu.model_folder(REAL_2L, 7, torch.bfloat16, std=0.02, norm_init="around_one",
+                             role_std={"norm": 0.2, "filter": 0.5, "q_proj.weight": 0.05,
+                                       "k_proj.weight": 0.05})
+    model = DecoderModel.from_folder(folder, "bfloat16")
+    B = 24
+    prompts = [eu.random_tokens(5 + r % 7, 65536, 700 + r) for r in range(B)]
+    tails = [eu.random_tokens(8, 65536, 800 + r) for r in range(B)]
+    runners = [ModelRunner(model, page_size=16, num_pages=3 * B, num_slots=B + 1, use_graphs=g)
+               for g in (True, False)]
+    for runner in runners:
+        for r in range(B):
+            runner.admit(r)
+        runner.step([StepEntry(r, prompts[r], []) for r in range(B)])
+    extra = eu.random_tokens(30, 65536, 999)
+    for step in range(8):
+        batch = [StepEntry(r, [tails[r][step]], [0]) for r in range(B)]
+        recorded, eager = (runner.step(batch).cpu() for runner in runners)
+        # the recorded step plans its attention for a rounded-up context length, so
+        # the two may differ as two cuts of the same work do: in rounding
+        assert eu.rel_err(recorded, eager.double()) < TOL["bfloat16"], f"step {step}"
+        if step % 2 == 1:                     # other work between the replays
+            for runner in runners:
+                runner.admit(("x", step))
+                runner.step([StepEntry(("x", step), extra, [29])])
+                runner.release(("x", step))
+        torch.cuda.synchronize()
+    assert runners[0].graphs.replays >= 6 and runners[1].graphs is None
+    oracle = plain.PlainLfm2(folder)                     # and the last replay is right
+    for r in (0, 12, 23):
+        want = oracle.logits(prompts[r] + tails[r])[-1:]
+        assert eu.rel_err(recorded[r:r + 1], want) < TOL["bfloat16"], f"request {r}"
+
+
 def test_widths_that_are_no_multiple_of_eight():
     """Any width runs in 32-bit; bfloat16 projections need rows that start on 16-byte
     boundaries and say so when the model is built, before anything runs."""
