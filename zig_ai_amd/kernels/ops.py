@@ -92,7 +92,7 @@ def _check(rc: int, name: str, detail: str = "") -> None:
 
 
 def _ptr(t: Optional[torch.Tensor]):
-    return None if t is None else c_void_p(t.data_ptr())
+    return None if t is None else t.data_ptr()      # an int converts to void*, None to NULL
 
 
 # The current stream's handle, asked for before every launch: torch's binding that
@@ -104,8 +104,8 @@ _raw_device = getattr(torch._C, "_cuda_getDevice", None)
 
 def _stream():
     if _raw_stream is not None and _raw_device is not None:
-        return c_void_p(_raw_stream(_raw_device()))
-    return c_void_p(torch.cuda.current_stream().cuda_stream)
+        return _raw_stream(_raw_device())
+    return torch.cuda.current_stream().cuda_stream
 
 
 def _code(dtype: torch.dtype) -> int:
