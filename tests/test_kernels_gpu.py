@@ -627,7 +627,7 @@ def test_short_conv_whole_and_in_portions(dtype, H, L, bias):
         n = [p.shape[0] for p in parts]
         token_seq = torch.cat([torch.full((m,), i, dtype=torch.int32) for i, m in enumerate(n)])
         seq_start = torch.tensor([0] + list(torch.tensor(n).cumsum(0)), dtype=torch.int32)
-        return ops().short_conv(z, w.to(dev()), b.to(dev()) if bias else None, state,
+        return ops().short_conv(z, w.t().contiguous().to(dev()), b.to(dev()) if bias else None, state,
                                 token_seq.to(dev()), seq_start.to(dev()),
                                 torch.tensor(slot_ids, dtype=torch.int32, device=dev()))
 
@@ -673,7 +673,7 @@ def test_short_conv_identity_filter():
     w = torch.zeros(H, L)
     w[:, L - 1] = 1.0
     state = torch.zeros((1, H, L), device=dev())
-    y = ops().short_conv(z.to(dev()), w.to(dev()), None, state,
+    y = ops().short_conv(z.to(dev()), w.t().contiguous().to(dev()), None, state,
                          torch.zeros(T, dtype=torch.int32, device=dev()),
                          torch.tensor([0, T], dtype=torch.int32, device=dev()),
                          torch.zeros(1, dtype=torch.int32, device=dev())).cpu()

@@ -4,9 +4,11 @@
 //
 //   z = in_proj(x) = [B | C | X] per token (three blocks of `width` channels)
 //   u[t]   = B[t] * X[t]
-//   c[t]   = bias + sum_{j<L} w[ch][j] * u[t - (L-1) + j]      (u before the portion comes
+//   c[t]   = bias + sum_{j<L} w[j][ch] * u[t - (L-1) + j]      (u before the portion comes
 //                                                               from the request's state)
 //   y[t]   = C[t] * c[t]
+//   (the filter is given tap by tap, w[j] holding tap j of every channel: a thread's
+//   channels, and neighbouring threads', then lie side by side)
 //   state <- the last L values of u, oldest first  (state[slot] starts slot_stride floats
 //            after state[slot - 1]; within a slot the layout is [channel][L])
 //
@@ -17,7 +19,7 @@
 //
 // Tokens are packed request after request; `token_seq` names each token's request, so
 // a thread never uses inputs from across a request's edge.  Two kinds of workgroups
-// share a launch (told apart by their place in the grid):
+// share a launch (told apart by their place in the grid, heads first):
 //   * body: one thread per (4 consecutive tokens, 8 channels) with 16-byte accesses
 //     (one channel for widths that are no multiple of 8), for the tokens whose L
 //     inputs all lie in the portion itself.  The inputs of the 4 + L - 1 rows are
@@ -67,30 +69,40 @@ short_conv_kernel(const T* __restrict__ z, const float* __restrict__ w,
   // state, and at least one, so that a step of single tokens needs no body
   const int reach = L > 1 ? L - 1 : 1;
 
-  if ((int)blockIdx.x < body_total) {
+  // The heads come first in the grid: their chain of dependent loads (request, slot,
+  // state, inputs) is long, and started last it would stand alone at the kernel's end.
+  const int head_total = (int)gridDim.x - body_total;
+  if ((int)blockIdx.x >= head_total) {
     // ---- body: tokens t0 .. t0 + SC_TOK - 1, those whose inputs all lie in their portion
-    const int t0 = ((int)blockIdx.x / body_blocks) * SC_TOK;
-    const int ch = (((int)blockIdx.x % body_blocks) * blockDim.x + threadIdx.x) * VEC;
+    const int bb_ = (int)blockIdx.x - head_total;
+    const int t0 = (bb_ / body_blocks) * SC_TOK;
+    const int ch = ((bb_ % body_blocks) * blockDim.x + threadIdx.x) * VEC;
     if (ch >= width) return;
-    bool mine[SC_TOK];
-    bool any = false;
+    // Every load below is issued before anything is waited for: which of the four
+    // tokens are this thread's to write is known only after two dependent lookups
+    // (the token's request, that request's first token), and the inputs' addresses do
+    // not depend on it.
+    int seq_of[SC_TOK];
 #pragma unroll
-    for (int i = 0; i < SC_TOK; ++i) {
-      const int t = t0 + i;
-      mine[i] = false;
-      if (t < n_tokens) mine[i] = t - seq_start[token_seq[t]] >= reach;
-      any = any || mine[i];
-    }
-    if (!any) return;
+    for (int i = 0; i < SC_TOK; ++i) seq_of[i] = t0 + i < n_tokens ? token_seq[t0 + i] : -1;
     float wt[SC_MAX_L][VEC], c[SC_TOK][VEC];
 #pragma unroll
     for (int j = 0; j < SC_MAX_L; ++j)
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) wt[j][v] = j < L ? w[(size_t)(ch + v) * L + j] : 0.f;
+      for (int v = 0; v < VEC; ++v) wt[j][v] = 0.f;
+#pragma unroll
+    for (int j = 0; j < SC_MAX_L; ++j)
+      if (j < L) load_vec<float, VEC>(w + (size_t)j * width + ch, wt[j]);
 #pragma unroll
     for (int i = 0; i < SC_TOK; ++i)
 #pragma unroll
       for (int v = 0; v < VEC; ++v) c[i][v] = bias ? bias[ch + v] : 0.f;
+    float cc[SC_TOK][VEC];
+#pragma unroll
+    for (int i = 0; i < SC_TOK; ++i) {
+      const int t = t0 + i < n_tokens ? t0 + i : n_tokens - 1;
+      load_vec<T, VEC>(z + (size_t)t * zs + width + ch, cc[i]);
+    }
     // row r of the window is token t0 - (L - 1) + r; output i uses rows i .. i + L - 1
 #pragma unroll
     for (int r = 0; r < SC_TOK + SC_MAX_L - 1; ++r)
@@ -111,20 +123,20 @@ short_conv_kernel(const T* __restrict__ z, const float* __restrict__ w,
         }
       }
 #pragma unroll
-    for (int i = 0; i < SC_TOK; ++i)
-      if (mine[i]) {
-        const int t = t0 + i;
-        float cc[VEC], o[VEC];
-        load_vec<T, VEC>(z + (size_t)t * zs + width + ch, cc);
+    for (int i = 0; i < SC_TOK; ++i) {
+      // mine: the token exists and all its L inputs lie in its own portion
+      if (seq_of[i] >= 0 && t0 + i - seq_start[seq_of[i]] >= reach) {
+        float o[VEC];
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) o[v] = cc[v] * c[i][v];
-        store_vec<T, VEC>(y + (size_t)t * width + ch, o);
+        for (int v = 0; v < VEC; ++v) o[v] = cc[i][v] * c[i][v];
+        store_vec<T, VEC>(y + (size_t)(t0 + i) * width + ch, o);
       }
+    }
     return;
   }
 
   // ---- head: the outputs that reach into the carried state, then the new state
-  const int hb = (int)blockIdx.x - body_total;
+  const int hb = (int)blockIdx.x;
   const int s = hb / head_blocks;
   const int ch = (hb % head_blocks) * blockDim.x + threadIdx.x;
   if (ch >= width) return;
@@ -134,7 +146,7 @@ short_conv_kernel(const T* __restrict__ z, const float* __restrict__ w,
   if (n <= 0) return;
   float wt[SC_MAX_L];
 #pragma unroll
-  for (int j = 0; j < SC_MAX_L; ++j) wt[j] = j < L ? w[(size_t)ch * L + j] : 0.f;
+  for (int j = 0; j < SC_MAX_L; ++j) wt[j] = j < L ? w[(size_t)j * width + ch] : 0.f;
   const float b = bias ? bias[ch] : 0.f;
   auto gate_in = [&](int row) -> float {
     const T* zr = z + (size_t)row * zs;

@@ -539,17 +539,20 @@ def paged_attention_decode_mfma(q: torch.Tensor, kv_cache: torch.Tensor,
 
 
 # ---------------------------------------------------------------- short conv
-def short_conv(z: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+def short_conv(z: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tensor],
                state: torch.Tensor, token_seq: torch.Tensor, seq_start: torch.Tensor,
                slot_id: torch.Tensor) -> torch.Tensor:
     """Gated causal depth-wise convolution with carried state; see
-    csrc/shortconv.hip.  ``z [T, 3*width]``, ``weight [width, L]``,
-    ``state [slots, width, L]`` (updated in place; slots may be spaced
+    csrc/shortconv.hip.  ``z [T, 3*width]``; ``taps [L, width]``, the filter tap by
+    tap (a checkpoint's ``[width, L]`` turned round, so that a thread's channels lie
+    side by side); ``state [slots, width, L]`` (updated in place; slots may be spaced
     further apart than ``width * L`` floats)."""
     T = z.shape[0]
-    width, L = weight.shape
+    if taps.dim() != 2:
+        raise KernelError(f"taps must be [L, width], got {tuple(taps.shape)}")
+    L, width = taps.shape
     _need(z, "z", (torch.float32, torch.bfloat16), (T, 3 * width))
-    _need(weight, "weight", torch.float32)
+    _need(taps, "taps", torch.float32)
     if L > 8:
         raise KernelError(f"convolution length {L} exceeds the kernel's limit of 8")
     if bias is not None:
@@ -565,7 +568,7 @@ def short_conv(z: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tenso
     _need(seq_start, "seq_start", torch.int32)
     _need(slot_id, "slot_id", torch.int32)
     y = torch.empty((T, width), dtype=z.dtype, device=z.device)
-    rc = _fn("shortconv", "za_short_conv")(_ptr(z), _ptr(weight), _ptr(bias), _ptr(state),
+    rc = _fn("shortconv", "za_short_conv")(_ptr(z), _ptr(taps), _ptr(bias), _ptr(state),
                                            _ptr(token_seq), _ptr(seq_start), _ptr(slot_id), _ptr(y),
                                            _code(z.dtype), T, slot_id.numel(), width, L,
                                            state.stride(0), _stream())

@@ -52,7 +52,8 @@ class ShortConv(Mixer):
             raise ValueError(f"conv kernel_size {self.kernel_size} exceeds the kernel's limit of 8")
         self.w_in = tensors["in_proj.weight"]
         self.w_out = tensors["out_proj.weight"]
-        self.w_conv = tensors["conv.weight"].reshape(self.hidden, self.kernel_size).contiguous()
+        # the kernel takes the filter tap by tap, [L, hidden]
+        self.w_conv = tensors["conv.weight"].reshape(self.hidden, self.kernel_size).t().contiguous()
         self.b_in = tensors.get("in_proj.bias")
         self.b_conv = tensors.get("conv.bias")
         self.b_out = tensors.get("out_proj.bias")
