@@ -256,6 +256,7 @@ attention_combine_kernel(const float* __restrict__ part_acc, const float* __rest
 // (l % 16) of the product.
 #define AM_KT 64
 #define AM_ROWS 128
+#define ZA_DECODE_WIDE_BELOW 384   // workgroups: up to here the decode kernel runs eight waves
 
 
 // A query row's scores for a tile are spread over the four lanes l, l ^ 16, l ^ 32,
@@ -583,7 +584,7 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
 
 // Decoding on the matrix cores: work items of at most 16 rows (one or a few
 // tokens times the query heads of the group), which become the 16 columns of the
-// second operand.  The four waves of a workgroup take the key tiles of the
+// second operand.  The waves of a workgroup (NWV: four or eight) take the key tiles of the
 // workgroup's key range in turn and never wait for each other inside the loop:
 // keys go from global memory straight into first-operand registers (a lane needs
 // 8 consecutive head-dim elements of one key), and so do the values (a lane needs,
@@ -591,8 +592,8 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
 // side by side).  At the end the four partial (m, l, O) are merged in LDS; with
 // `nsplit` > 1 the merged partial goes to `attention_combine_kernel` like those of
 // the plain kernel.
-template <int D>
-__global__ void __launch_bounds__(256)
+template <int D, int NWV>
+__global__ void __launch_bounds__(NWV * 64)
 paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                                    const bf16_t* __restrict__ kv,
                                    const int* __restrict__ block_table, int bt_stride,
@@ -603,8 +604,8 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
                                    float scale, int window, int keys_per_split, int nsplit) {
   constexpr int KSTEPS = D / 32;
   constexpr int DBLK = D / 16;
-  __shared__ float mg_m[4][16], mg_l[4][16];
-  __shared__ float mg_o[4][DBLK][64][4];
+  __shared__ float mg_m[NWV][16], mg_l[NWV][16];
+  __shared__ float mg_o[NWV][DBLK][64][4];
 
   const int item = blockIdx.x, gkv = blockIdx.y, z = blockIdx.z;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -713,10 +714,10 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
 
   int tile0 = tile_first + wave * AM_KT;
   if (tile0 <= range_hi) fetch(tile0, kf, vf);
-  for (; tile0 <= range_hi; tile0 += 4 * AM_KT) {
+  for (; tile0 <= range_hi; tile0 += NWV * AM_KT) {
     bf16x8_t kfn[4][KSTEPS];
     bf16x4_t vfn[DBLK][4];
-    const int next = tile0 + 4 * AM_KT;
+    const int next = tile0 + NWV * AM_KT;
     if (next <= range_hi) fetch(next, kfn, vfn);
 
     f32x4_t s[4];
@@ -786,7 +787,7 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
     }
   }
 
-  // merge the four waves' partial results
+  // merge the waves' partial results
   if (grp == 0) { mg_m[wave][r16] = m; mg_l[wave][r16] = l; }
 #pragma unroll
   for (int db = 0; db < DBLK; ++db)
@@ -796,11 +797,11 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
   if (wave == 0 && row_valid) {
     float mx = mg_m[0][r16];
 #pragma unroll
-    for (int w = 1; w < 4; ++w) mx = fmaxf(mx, mg_m[w][r16]);
+    for (int w = 1; w < NWV; ++w) mx = fmaxf(mx, mg_m[w][r16]);
     const float mu = mx > -INFINITY ? mx : 0.f;
-    float wgt[4], total = 0.f;
+    float wgt[NWV], total = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < NWV; ++w) {
       wgt[w] = expf(mg_m[w][r16] - mu);
       total += mg_l[w][r16] * wgt[w];
     }
@@ -811,7 +812,7 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
       for (int i = 0; i < 4; ++i) {
         float acc = 0.f;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) acc = fmaf(mg_o[w][db][lane][i], wgt[w], acc);
+        for (int w = 0; w < NWV; ++w) acc = fmaf(mg_o[w][db][lane][i], wgt[w], acc);
         const int dim = db * 16 + grp * 4 + i;
         if (nsplit == 1)
           out[orow * D + dim] = (bf16_t)(total > 0.f ? acc / total : 0.f);
@@ -977,13 +978,21 @@ extern "C" int za_paged_attention_decode_mfma(const void* q, void* out, const vo
   if (nsplit > 1 && (!part_acc || !part_ml || keys_per_split <= 0 || keys_per_split % 64 != 0))
     return ZA_ERR_ARG;
   dim3 grid(n_items, nkv, nsplit), block(256);
-  if (d == 64) {
-    hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<64>), grid, block, 0, stream,
+  // Few workgroups (a small batch): eight waves each, so that a compute unit that
+  // gets one workgroup still has eight waves' loads in flight.
+  const long long workgroups = (long long)n_items * nkv * nsplit;
+  if (d == 64 && workgroups <= ZA_DECODE_WIDE_BELOW) {
+    hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<64, 8>), grid, dim3(512), 0, stream,
+                       (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
+                       positions, wi_seq, wi_row0, wi_count, part_acc, part_ml, nh, nkv,
+                       page_size, scale, window, keys_per_split, nsplit);
+  } else if (d == 64) {
+    hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<64, 4>), grid, block, 0, stream,
                        (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
                        positions, wi_seq, wi_row0, wi_count, part_acc, part_ml, nh, nkv,
                        page_size, scale, window, keys_per_split, nsplit);
   } else {
-    hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<128>), grid, block, 0, stream,
+    hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<128, 4>), grid, block, 0, stream,
                        (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
                        positions, wi_seq, wi_row0, wi_count, part_acc, part_ml, nh, nkv,
                        page_size, scale, window, keys_per_split, nsplit);
