@@ -315,6 +315,66 @@ def test_qk_norm_rope_kv_write(dtype, nh, nkv, d, rot, pairing):
     assert (untouched_k == 0).all() and (untouched_v == 0).all()   # nothing else was touched
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,d,rot,pairing,page_size", [
+    (32, 8, 64, 64, "half", 16), (3, 1, 128, 128, "half", 8), (4, 2, 32, 16, "adjacent", 16),
+    (8, 2, 64, 64, "half", 4), (2, 2, 16, 16, "adjacent", 32)])
+def test_qk_norm_rope_kv_write_many_tokens(dtype, nh, nkv, d, rot, pairing, page_size):
+    """A step with prompt portions: blocks take eight tokens each and store the
+    values of eight neighbouring offsets side by side.  Stretches that start at a
+    multiple of eight, one that starts at offset 5, single decoded tokens between
+    them, a tail that is no multiple of eight: bit for bit what the same tokens give
+    in calls small enough to go one token per block, and right."""
+    theta, eps = 10000.0, 1e-5
+    stretches = [(0, 0, 64), (1, 5, 70), (2, 300, 1), (3, 17, 1), (4, 32, 40), (5, 999, 1),
+                 (6, 8, 27)]                          # (request, first position, tokens)
+    per_req = (1024 + page_size - 1) // page_size + 1
+    pages = per_req * len(stretches)
+    order = torch.randperm(pages, generator=torch.Generator().manual_seed(31)).tolist()
+    positions, slots = [], []
+    for r, first, n in stretches:
+        for p in range(first, first + n):
+            positions.append(p)
+            slots.append(order[r * per_req + p // page_size] * page_size + p % page_size)
+    T = len(positions)
+    assert T >= 128 and T % 8 != 0
+    positions = torch.tensor(positions, dtype=torch.int32)
+    slots = torch.tensor(slots, dtype=torch.int32)
+    qkv = rand((T, (nh + 2 * nkv) * d), dtype, 32)
+    qw, kw = rand((d,), torch.float32, 33) + 1.0, rand((d,), torch.float32, 34) + 1.0
+    inv = (1.0 / torch.pow(torch.tensor(theta, dtype=torch.float64),
+                           2.0 * torch.arange(0, rot // 2, dtype=torch.float64) / rot)).float()
+
+    def run(cuts):
+        cache = torch.zeros((pages, 2, nkv, page_size, d), dtype=dtype, device=dev())
+        qs = []
+        for a, b in zip(cuts[:-1], cuts[1:]):
+            qs.append(ops().qk_norm_rope_kv_write(
+                qkv[a:b].contiguous().to(dev()), positions[a:b].to(dev()), slots[a:b].to(dev()),
+                qw.to(dev()), kw.to(dev()), inv.to(dev()), cache, nh, nkv, d, rot,
+                pairing == "adjacent", eps))
+        return torch.cat(qs).cpu(), cache.cpu()
+
+    q_all, cache_all = run([0, T])
+    q_few, cache_few = run(list(range(0, T, 50)) + [T])
+    assert torch.equal(q_all, q_few) and torch.equal(cache_all, cache_few)
+    heads = qkv.double().view(T, nh + 2 * nkv, d)
+    qe = plain.apply_rope(plain.rms_norm(heads[:, :nh], qw.double(), eps), positions, theta, rot, pairing)
+    ke = plain.apply_rope(plain.rms_norm(heads[:, nh:nh + nkv], kw.double(), eps), positions, theta,
+                          rot, pairing)
+    tol = tol_of(dtype) + 1100 * 1.2e-7
+    assert rel_err(q_all, qe) < tol
+    got_k = torch.stack([cache_all[s // page_size, 0, :, s % page_size, :] for s in slots.tolist()])
+    cv = cache_all[:, 1].reshape(pages, nkv, d, page_size)
+    got_v = torch.stack([cv[s // page_size, :, :, s % page_size] for s in slots.tolist()])
+    assert rel_err(got_k, ke) < tol
+    assert torch.equal(got_v.double(), heads[:, nh + nkv:])
+    written = torch.zeros(pages * page_size, dtype=torch.bool)
+    written[slots.long()] = True
+    untouched_v = cv.permute(0, 3, 1, 2).reshape(pages * page_size, -1)[~written]
+    assert (untouched_v == 0).all()
+
+
 def test_rope_position_zero_is_identity_and_norm_is_kept():
     """rope.zig:226-253 holds the rotation to preserving the norm; position 0 rotates
     by nothing."""

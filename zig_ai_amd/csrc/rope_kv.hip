@@ -100,10 +100,59 @@ qk_norm_rope_kv_write_pow2_kernel(const T* __restrict__ qkv, const int* __restri
                                   const float* __restrict__ k_norm_w,
                                   const float* __restrict__ inv_freq, T* __restrict__ q_out,
                                   T* __restrict__ kv_cache, int nh, int nkv, int rot, int adjacent,
-                                  float eps, int page_size, int write_kv) {
+                                  float eps, int page_size, int write_kv, int n_tokens,
+                                  int value_blocks) {
   constexpr int LPH = D / 8;   // lanes per head
   __shared__ float cs_tab[D / 2], sn_tab[D / 2];
-  const int t = blockIdx.x;
+  if ((int)blockIdx.x < value_blocks) {
+    // ---- values only, for steps of many tokens: a wave takes eight consecutive tokens
+    // and stores, where these lie at eight neighbouring offsets of one page from a
+    // multiple of eight on (a stretch of a prompt), each head-dim element's eight
+    // values with one 16-byte access (32 bytes in 32-bit) instead of eight 2-byte
+    // ones a page row apart.  Other groups (a request's edge, single tokens between
+    // prompts) store element by element.
+    const int lane = threadIdx.x & 63;
+    const int t0 = ((int)blockIdx.x * 4 + ((int)threadIdx.x >> 6)) * 8;   // a wave's 8 tokens
+    if (t0 >= n_tokens) return;
+    const int total = nh + 2 * nkv;
+    int slot[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) slot[j] = t0 + j < n_tokens ? slots[t0 + j] : -1;
+    bool side_by_side = page_size % 8 == 0 && slot[0] >= 0 && slot[0] % 8 == 0;
+#pragma unroll
+    for (int j = 1; j < 8; ++j) side_by_side = side_by_side && slot[j] == slot[0] + j;
+    for (int pair = lane; pair < nkv * LPH; pair += 64) {
+      const int hv = pair / LPH, e0 = (pair % LPH) * 8;
+      float x[8][8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (t0 + j < n_tokens)
+          load8<T>(qkv + ((size_t)(t0 + j) * total + nh + nkv + hv) * D + e0, x[j]);
+      if (side_by_side) {
+        T* dst = kv_cache + (((size_t)(slot[0] / page_size) * 2 + 1) * nkv + hv) * page_size * D +
+                 (size_t)e0 * page_size + slot[0] % page_size;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          float run[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) run[j] = x[j][i];
+          store8<T>(dst + (size_t)i * page_size, run);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (slot[j] >= 0) {
+            T* dst = kv_cache +
+                     (((size_t)(slot[j] / page_size) * 2 + 1) * nkv + hv) * page_size * D +
+                     (size_t)e0 * page_size + slot[j] % page_size;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) dst[(size_t)i * page_size] = from_f32<T>(x[j][i]);
+          }
+      }
+    }
+    return;
+  }
+  const int t = (int)blockIdx.x - value_blocks;
   const int half = rot / 2;
   if ((int)threadIdx.x < half) {
     const float angle = (float)positions[t] * inv_freq[threadIdx.x];
@@ -114,9 +163,10 @@ qk_norm_rope_kv_write_pow2_kernel(const T* __restrict__ qkv, const int* __restri
   }
   __syncthreads();
   const int total = nh + 2 * nkv;
+  const int heads_here = value_blocks > 0 ? nh + nkv : total;   // values go their own way
   const int li = threadIdx.x % LPH;
   const int e0 = li * 8;        // this lane's first element of the head
-  for (int head = threadIdx.x / LPH; head < total; head += 256 / LPH) {
+  for (int head = threadIdx.x / LPH; head < heads_here; head += 256 / LPH) {
     const bool is_q = head < nh;
     const bool is_k = !is_q && head < nh + nkv;
     float x[8];
@@ -177,6 +227,8 @@ qk_norm_rope_kv_write_pow2_kernel(const T* __restrict__ qkv, const int* __restri
   }
 }
 
+#define RK_VALUE_BLOCKS_FROM 128   // tokens in a step from which values get blocks of their own
+
 template <typename T>
 static bool launch_pow2(const void* qkv, const int* positions, const int* slots,
                         const float* q_norm_w, const float* k_norm_w, const float* inv_freq,
@@ -184,10 +236,14 @@ static bool launch_pow2(const void* qkv, const int* positions, const int* slots,
                         int adjacent, float eps, int page_size, int write_kv,
                         hipStream_t stream) {
   if (!adjacent && (rot / 2) % 8 != 0) return false;
+  // many tokens (prompt portions): the values are written by blocks of their own, first
+  // in the grid, 32 tokens each
+  const int value_blocks = (write_kv && n_tokens >= RK_VALUE_BLOCKS_FROM) ? (n_tokens + 31) / 32 : 0;
 #define ZA_RK_LAUNCH(DD)                                                                        \
-  hipLaunchKernelGGL((qk_norm_rope_kv_write_pow2_kernel<T, DD>), dim3(n_tokens), dim3(256), 0,   \
-                     stream, (const T*)qkv, positions, slots, q_norm_w, k_norm_w, inv_freq,      \
-                     (T*)q_out, (T*)kv_cache, nh, nkv, rot, adjacent, eps, page_size, write_kv)
+  hipLaunchKernelGGL((qk_norm_rope_kv_write_pow2_kernel<T, DD>), dim3(n_tokens + value_blocks),  \
+                     dim3(256), 0, stream, (const T*)qkv, positions, slots, q_norm_w, k_norm_w,  \
+                     inv_freq, (T*)q_out, (T*)kv_cache, nh, nkv, rot, adjacent, eps, page_size,  \
+                     write_kv, n_tokens, value_blocks)
   switch (d) {
     case 16: ZA_RK_LAUNCH(16); return true;
     case 32: ZA_RK_LAUNCH(32); return true;
