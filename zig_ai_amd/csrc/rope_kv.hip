@@ -154,6 +154,15 @@ qk_norm_rope_kv_write_pow2_kernel(const T* __restrict__ qkv, const int* __restri
   }
   const int t = (int)blockIdx.x - value_blocks;
   const int half = rot / 2;
+  const int total = nh + 2 * nkv;
+  const int heads_here = value_blocks > 0 ? nh + nkv : total;   // values go their own way
+  const int li = threadIdx.x % LPH;
+  const int e0 = li * 8;        // this lane's first element of the head
+  // this thread's first head is requested before the angles are worked out, and each
+  // further head while the one before it is being processed
+  float xn[8];
+  if ((int)threadIdx.x / LPH < heads_here)
+    load8<T>(qkv + ((size_t)t * total + threadIdx.x / LPH) * D + e0, xn);
   if ((int)threadIdx.x < half) {
     const float angle = (float)positions[t] * inv_freq[threadIdx.x];
     float sn, cs;
@@ -162,15 +171,14 @@ qk_norm_rope_kv_write_pow2_kernel(const T* __restrict__ qkv, const int* __restri
     sn_tab[threadIdx.x] = sn;
   }
   __syncthreads();
-  const int total = nh + 2 * nkv;
-  const int heads_here = value_blocks > 0 ? nh + nkv : total;   // values go their own way
-  const int li = threadIdx.x % LPH;
-  const int e0 = li * 8;        // this lane's first element of the head
   for (int head = threadIdx.x / LPH; head < heads_here; head += 256 / LPH) {
     const bool is_q = head < nh;
     const bool is_k = !is_q && head < nh + nkv;
     float x[8];
-    load8<T>(qkv + ((size_t)t * total + head) * D + e0, x);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = xn[i];
+    if (head + 256 / LPH < heads_here)
+      load8<T>(qkv + ((size_t)t * total + head + 256 / LPH) * D + e0, xn);
     const float* nw = is_q ? q_norm_w : (is_k ? k_norm_w : nullptr);
     if (nw) {
       float ss = 0.f;
@@ -179,8 +187,10 @@ qk_norm_rope_kv_write_pow2_kernel(const T* __restrict__ qkv, const int* __restri
 #pragma unroll
       for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
       const float scale = 1.0f / sqrtf(ss / (float)D + eps);
+      float w8[8];
+      load8<float>(nw + e0, w8);     // two 16-byte loads, not eight of 4 bytes
 #pragma unroll
-      for (int i = 0; i < 8; ++i) x[i] = x[i] * scale * nw[e0 + i];
+      for (int i = 0; i < 8; ++i) x[i] = x[i] * scale * w8[i];
     }
     if ((is_q || is_k) && rot > 0) {
       if (adjacent) {
