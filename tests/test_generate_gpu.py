@@ -225,3 +225,36 @@ def test_trace_run(dtype, tmp_path):
                 err = eu.rel_err(data[r:r + len(places)], expect[i][places])
                 assert err < tol, f"step {step} request {i}: {err:.3e}"
             r += len(places)
+
+
+def test_an_engine_used_again_and_again_keeps_nothing():
+    """Forty calls of generate() on one engine, with other batch sizes, lengths and
+    sampling options each time and a pool that forces preemptions now and then:
+    afterwards no request, page, slot or name is held, and device memory has not
+    grown since the first calls."""
+    import random
+
+    from zig_ai_amd.engine import Engine
+    folder = folder_for(TINY_B, 1)
+    engine = Engine(folder, dtype="bfloat16", page_size=8, num_pages=48, max_num_seqs=5,
+                    chunk_size=32, max_num_batched_tokens=80)
+    rng = random.Random(3)
+    allocated = []
+    for call in range(40):
+        n = rng.randint(1, 7)
+        prompts = [eu.random_tokens(rng.randint(1, 90), 512, 1000 * call + i) for i in range(n)]
+        kw = rng.choice([dict(temperature=0.0), dict(temperature=0.8, seed=call),
+                         dict(temperature=1.1, top_k=20, top_p=0.9, seed=call),
+                         dict(temperature=0.0, repetition_penalty=1.2)])
+        new = rng.randint(1, 24)
+        out = engine.generate(prompts, max_new_tokens=new, eos_token_id=-1, **kw)
+        assert [len(o) for o in out] == [new] * n
+        stats = engine.stats()
+        assert stats["requests"] == 0
+        assert all(g["pages_free"] == g["pages"] for g in stats["groups"])
+        assert stats["slots_free"] == stats["slots"]
+        assert len(engine.runner.cache.handles) == 0
+        torch.cuda.synchronize()
+        allocated.append(torch.cuda.memory_allocated())
+    assert engine.stats()["preemptions"] > 0
+    assert max(allocated[20:]) <= max(allocated[:20])
