@@ -649,10 +649,18 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
   float m = -INFINITY, l = 0.f;
 
   // One tile's keys and values as first-operand fragments in registers; the next tile
-  // is fetched while this one is being computed.  vf[db][jb] holds, for head-dim
-  // element db * 16 + r16, keys jb * 16 + grp * 4 .. + 3 of the tile.
+  // is fetched while this one is being computed.
+  //
+  // Which key sits in which row of a 16-row block is free as long as scores, masks
+  // and values agree.  Rows are dealt so that a lane's scores of blocks 2kk and
+  // 2kk + 1 are those of EIGHT consecutive keys: row r of block jb is key
+  //   (jb / 2) * 32 + (r / 4) * 8 + (jb % 2) * 4 + r % 4          of the tile,
+  // so lane group grp ends up with keys kk * 32 + grp * 8 .. + 7, in that order, as
+  // the 8 k-slots of the second product.  The values of those eight keys for one
+  // head-dim element lie side by side in the page: vf[db][kk] is ONE 16-byte load
+  // (two of 8 bytes when the page size is no multiple of 8).
   bf16x8_t kf[4][KSTEPS];
-  bf16x4_t vf[DBLK][4];
+  bf16x8_t vf[DBLK][2];
   // The block-table entries are read whether or not the key turns out to be in
   // range (unused entries hold -1 and read page 0 instead), so that these loads do
   // not wait for the positions the range is computed from.  A key that must not
@@ -660,30 +668,40 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
   // since 0 * (not a number) would not be 0.
   const int last_entry = bt_stride - 1;
   const int ps_shift = page_shift_of(page_size);
-  auto fetch = [&](int tile0, bf16x8_t (&kfr)[4][KSTEPS], bf16x4_t (&vfr)[DBLK][4]) {
-    int kpage[4], vpage[4];
+  const bool wide = page_size % 8 == 0;
+  const int krow_in_pair = (r16 >> 2) * 8 + (r16 & 3);   // + (jb / 2) * 32 + (jb % 2) * 4
+  auto entry_of = [&](int key) {
+    const int e = page_entry(key, page_size, ps_shift);
+    return table[e < last_entry ? e : last_entry];
+  };
+  auto fetch = [&](int tile0, bf16x8_t (&kfr)[4][KSTEPS], bf16x8_t (&vfr)[DBLK][2]) {
+    int kpage[4], vpage[4];      // vpage: per run of 4 keys, kk * 2 + half
     if (ps_shift >= 4) {
       // Tiles start at multiples of 16 keys, so with pages of 16, 32, 64 ... keys a
       // block of 16 keys lies in one page: one entry for the whole wave, which the
       // scalar unit reads without waiting for the vector loads in flight.
       const int t0 = __builtin_amdgcn_readfirstlane(tile0);
+      int pg[4];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int e = (t0 + b * 16) >> ps_shift;
+        pg[b] = table[e < last_entry ? e : last_entry];
+      }
 #pragma unroll
       for (int jb = 0; jb < 4; ++jb) {
-        const int e = (t0 + jb * 16) >> ps_shift;
-        kpage[jb] = vpage[jb] = table[e < last_entry ? e : last_entry];
+        kpage[jb] = (r16 & 8) ? pg[(jb >> 1) * 2 + 1] : pg[(jb >> 1) * 2];
+        vpage[jb] = (grp & 2) ? pg[(jb >> 1) * 2 + 1] : pg[(jb >> 1) * 2];
       }
     } else {
 #pragma unroll
       for (int jb = 0; jb < 4; ++jb) {
-        const int e = page_entry(tile0 + jb * 16 + r16, page_size, ps_shift);
-        kpage[jb] = table[e < last_entry ? e : last_entry];
-        const int ev = page_entry(tile0 + jb * 16 + grp * 4, page_size, ps_shift);
-        vpage[jb] = table[ev < last_entry ? ev : last_entry];
+        kpage[jb] = entry_of(tile0 + (jb >> 1) * 32 + (jb & 1) * 4 + krow_in_pair);
+        vpage[jb] = entry_of(tile0 + (jb >> 1) * 32 + grp * 8 + (jb & 1) * 4);
       }
     }
 #pragma unroll
     for (int jb = 0; jb < 4; ++jb) {
-      const int kp = tile0 + jb * 16 + r16;
+      const int kp = tile0 + (jb >> 1) * 32 + (jb & 1) * 4 + krow_in_pair;
       const int page = kpage[jb] < 0 ? 0 : kpage[jb];
       const bf16_t* krow = kv + ((((size_t)page * 2) * nkv + gkv) * page_size +
                                  page_offset(kp, page_size, ps_shift)) * D;
@@ -693,21 +711,32 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
     }
     const bool inner = tile0 >= lo && tile0 + AM_KT - 1 <= range_hi;
 #pragma unroll
-    for (int jb = 0; jb < 4; ++jb) {
-      const int kp = tile0 + jb * 16 + grp * 4;
-      const int page = vpage[jb] < 0 ? 0 : vpage[jb];
-      const bf16_t* vbase = kv + (((size_t)page * 2 + 1) * nkv + gkv) * page_size * D +
-                            page_offset(kp, page_size, ps_shift);
+    for (int kk = 0; kk < 2; ++kk) {
+      const int kp = tile0 + kk * 32 + grp * 8;          // this lane's eight keys
+      const int page_a = vpage[2 * kk] < 0 ? 0 : vpage[2 * kk];
+      const int page_b = vpage[2 * kk + 1] < 0 ? 0 : vpage[2 * kk + 1];
+      const bf16_t* va = kv + (((size_t)page_a * 2 + 1) * nkv + gkv) * page_size * D +
+                         page_offset(kp, page_size, ps_shift);
+      const bf16_t* vb = kv + (((size_t)page_b * 2 + 1) * nkv + gkv) * page_size * D +
+                         page_offset(kp + 4, page_size, ps_shift);
 #pragma unroll
       for (int db = 0; db < DBLK; ++db) {
-        bf16x4_t x =
-            *reinterpret_cast<const bf16x4_t*>(vbase + (size_t)(db * 16 + r16) * page_size);
+        const size_t row = (size_t)(db * 16 + r16) * page_size;
+        bf16x8_t x;
+        if (wide) {
+          x = *reinterpret_cast<const bf16x8_t*>(va + row);
+        } else {
+          const bf16x4_t xa = *reinterpret_cast<const bf16x4_t*>(va + row);
+          const bf16x4_t xb = *reinterpret_cast<const bf16x4_t*>(vb + row);
+          x = __builtin_shufflevector(xa, xb, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
         if (!inner) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (vpage[jb] < 0 || kp + e < lo || kp + e > range_hi) x[e] = (bf16_t)0.f;
+          for (int e = 0; e < 8; ++e)
+            if (vpage[2 * kk + (e >> 2)] < 0 || kp + e < lo || kp + e > range_hi)
+              x[e] = (bf16_t)0.f;
         }
-        vfr[db][jb] = x;
+        vfr[db][kk] = x;
       }
     }
   };
@@ -716,7 +745,7 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
   if (tile0 <= range_hi) fetch(tile0, kf, vf);
   for (; tile0 <= range_hi; tile0 += NWV * AM_KT) {
     bf16x8_t kfn[4][KSTEPS];
-    bf16x4_t vfn[DBLK][4];
+    bf16x8_t vfn[DBLK][2];
     const int next = tile0 + NWV * AM_KT;
     if (next <= range_hi) fetch(next, kfn, vfn);
 
@@ -733,7 +762,7 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
     for (int jb = 0; jb < 4; ++jb)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int kp = tile0 + jb * 16 + grp * 4 + i;
+        const int kp = tile0 + (jb >> 1) * 32 + grp * 8 + (jb & 1) * 4 + i;
         bool valid = kp <= pos_row && kp >= lo && kp <= range_hi;
         if (window > 0 && kp <= pos_row - window) valid = false;
         const float v = valid ? s[jb][i] * scale : -INFINITY;
@@ -771,18 +800,18 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
 #pragma unroll
     for (int db = 0; db < DBLK; ++db)
 #pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
-        const bf16x8_t vv = __builtin_shufflevector(vf[db][2 * kk], vf[db][2 * kk + 1], 0, 1, 2,
-                                                    3, 4, 5, 6, 7);
-        o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, pf[kk], o[db], 0, 0, 0);
-      }
+      for (int kk = 0; kk < 2; ++kk)
+        o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[db][kk], pf[kk], o[db], 0, 0, 0);
     if (next <= range_hi) {
 #pragma unroll
       for (int jb = 0; jb < 4; ++jb) {
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) kf[jb][ks] = kfn[jb][ks];
+      }
 #pragma unroll
-        for (int db = 0; db < DBLK; ++db) vf[db][jb] = vfn[db][jb];
+      for (int db = 0; db < DBLK; ++db) {
+        vf[db][0] = vfn[db][0];
+        vf[db][1] = vfn[db][1];
       }
     }
   }
