@@ -588,8 +588,8 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
 // workgroup's key range in turn and never wait for each other inside the loop:
 // keys go from global memory straight into first-operand registers (a lane needs
 // 8 consecutive head-dim elements of one key), and so do the values (a lane needs,
-// for one head-dim element, two runs of 4 consecutive keys, which the cache holds
-// side by side).  At the end the waves' partial (m, l, O) are merged in LDS; with
+// for one head-dim element, 8 consecutive keys, which the cache holds side by
+// side).  At the end the waves' partial (m, l, O) are merged in LDS; with
 // `nsplit` > 1 the merged partial goes to `attention_combine_kernel` like those of
 // the plain kernel.
 template <int D, int NWV>
