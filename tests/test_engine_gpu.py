@@ -361,3 +361,60 @@ def test_decode_steps_hand_tokens_over_on_the_device(dtype):
     assert [tight.cache.num_tokens(r) for r in ids] == [n + drawn.shape[0] for n in lens]
     if dtype == "float32":
         assert drawn.tolist() == want[:drawn.shape[0]]
+
+
+def random_case(seed: int):
+    """A random small LFM2 configuration, requests, page size and way of cutting."""
+    import random
+    rng = random.Random(seed)
+    d = rng.choice([16, 32, 48, 64, 64, 128])
+    nkv = rng.choice([1, 2, 3])
+    nh = nkv * rng.choice([1, 2, 4, 5] if d <= 64 else [1, 2])
+    layers = rng.randint(2, 5)
+    types = [rng.choice(["conv", "full_attention"]) for _ in range(layers)]
+    if "full_attention" not in types:
+        types[rng.randrange(layers)] = "full_attention"
+    if "conv" not in types:
+        types[rng.randrange(layers)] = "conv"
+    cfg = {"architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+           "hidden_size": rng.choice([64, 96, 128, 160, 200]), "num_hidden_layers": layers,
+           "num_attention_heads": nh, "num_key_value_heads": nkv, "head_dim": d,
+           "vocab_size": rng.randint(40, 700), "layer_types": types,
+           "intermediate_size": 8 * rng.randint(5, 40), "rope_theta": rng.choice([1e4, 1e6]),
+           "norm_eps": rng.choice([1e-5, 1e-6]), "conv_L_cache": rng.randint(1, 6),
+           "conv_bias": rng.random() < 0.5, "tie_embedding": rng.random() < 0.5,
+           "max_position_embeddings": 4096}
+    lengths = [rng.choice([1, 2, 3, 9, 17, 40, 77, 130, 200]) for _ in range(rng.randint(2, 5))]
+    page = rng.choice([4, 8, 16, 32])
+    kind = rng.choice(["whole", "bulk", "portions", "mixed"])
+    if kind == "whole":
+        schedule = eu.whole(lengths)
+    elif kind == "bulk":
+        schedule = eu.bulk_then_single(lengths, rng.choice([5, 32]))
+    elif kind == "portions":
+        schedule = eu.changing_portions(lengths, rng.randrange(9))
+    else:
+        schedule = eu.mixed(lengths, seed=rng.randrange(100), max_live=rng.choice([2, 3, 4]))
+    pages = eu.peak_tokens(lengths, schedule, round_to=page) // page
+    return cfg, lengths, page, pages, schedule
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_configurations_and_cuts(seed):
+    """Sixteen configurations drawn at random (head sizes 16 to 128, one to fifteen
+    query heads in groups of one to five, convolution lengths 1 to 6, with and without
+    biases and tied heads, vocabularies and widths that are no powers of two), each with
+    its own requests, page size and way of cutting the work: in 32-bit the engine is the
+    plain implementation to 1e-4, whatever the draw; bfloat16 stays within its tolerance."""
+    from zig_ai_amd.engine import DecoderModel, ModelRunner
+    cfg, lengths, page, pages, schedule = random_case(seed)
+    for dtype in ("float32", "bfloat16"):
+        store = torch.float32 if dtype == "float32" else torch.bfloat16
+        folder = eu.model_folder(cfg, seed, store, **eu.sharp_kwargs())
+        model = DecoderModel.from_folder(folder, dtype)
+        oracle = plain.PlainLfm2(folder)
+        prompts = [eu.random_tokens(n, cfg["vocab_size"], 31 * seed + i) for i, n in enumerate(lengths)]
+        expect = [oracle.logits(p) for p in prompts]
+        runner = ModelRunner(model, page_size=page, num_pages=pages, num_slots=4)
+        check(eu.run_schedule(runner, prompts, schedule), expect, dtype, f"seed {seed}")
+        assert runner.cache.stats()["requests"] == 0
