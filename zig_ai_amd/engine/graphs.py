@@ -31,6 +31,7 @@ from .batch import PreparedEntries, StepEntry, StepError, build_step
 
 PAGE_BUCKET = 64        # block-table width is rounded up to a multiple of this
 KEYS_BUCKET = 1024      # and the longest context to a multiple of this
+MAX_GRAPHS = 96         # recorded shapes kept; the one replayed longest ago goes first
 
 
 def _round_up(n: int, m: int) -> int:
@@ -47,7 +48,7 @@ class DecodeGraphs:
         self._vocab = vocab_size
         self._granularities = tuple(item_granularities)
         self._max_position = max_position
-        self.entries: Dict[Tuple[int, int, int], dict] = {}
+        self.entries: Dict[Tuple[int, int, int], dict] = {}   # in order of last use
         self._arrays: Dict[int, dict] = {}       # per number of entries: arrays for the library
         self._lib = hostlib.lib()
         self.captures = 0
@@ -115,6 +116,8 @@ class DecodeGraphs:
         widest, longest = int(sc["extent"][0]), int(sc["extent"][1])
         key = (S, _round_up(widest, PAGE_BUCKET), _round_up(longest, KEYS_BUCKET))
         slot = self.entries.get(key)
+        if slot is not None:
+            self.entries[key] = self.entries.pop(key)     # now the most recently used
         if slot is not None and slot["graph"] is not None:
             # Bring the persistent integer buffer up to date: the host library lays the
             # step out in the pinned staging buffer, and one copy that does not block
@@ -165,6 +168,12 @@ class DecodeGraphs:
             slot["grans_ptr"] = grans.ctypes.data
             slot["sections_ptr"] = slot["sections"].ctypes.data
             slot["pinned_ptr"] = slot["pinned"].data_ptr()
+            # a graph holds its intermediate tensors for good: a process that sees many
+            # batch sizes and context lengths keeps the shapes it used last
+            if len(self.entries) >= MAX_GRAPHS:
+                torch.cuda.current_stream().synchronize()    # its last replay may still run
+                while len(self.entries) >= MAX_GRAPHS:
+                    self.entries.pop(next(iter(self.entries)))
             self.entries[key] = slot
         ctx = build_step(asked, cache, runner.device, self._vocab, self._granularities,
                          self._max_position, min_pages=key[1], max_keys=key[2],
