@@ -258,3 +258,28 @@ def test_an_engine_used_again_and_again_keeps_nothing():
         allocated.append(torch.cuda.memory_allocated())
     assert engine.stats()["preemptions"] > 0
     assert max(allocated[20:]) <= max(allocated[:20])
+
+
+def test_a_failed_generate_leaves_nothing_behind():
+    """One request of the call can never fit the pool: generate() raises, and what the
+    other requests of that call held is given back; the engine then serves the next call
+    as if nothing had happened."""
+    from zig_ai_amd.cache import OutOfPages
+    from zig_ai_amd.engine import Engine
+    folder = folder_for(TINY_B, 1)
+    oracle = plain.PlainLfm2(folder)
+    engine = Engine(folder, dtype="float32", page_size=8, num_pages=6, max_num_seqs=4,
+                    max_model_len=400)
+    small = [eu.random_tokens(n, 512, 70 + n) for n in (5, 9)]
+    too_long = eu.random_tokens(60, 512, 99)             # 60 tokens need 8 pages; there are 6
+    with pytest.raises(OutOfPages):
+        engine.generate(small + [too_long], max_new_tokens=4, temperature=0.0, eos_token_id=-1)
+    stats = engine.stats()
+    assert stats["requests"] == 0 and stats["slots_free"] == stats["slots"]
+    assert all(g["pages_free"] == g["pages"] for g in stats["groups"])
+    assert len(engine.runner.cache.handles) == 0
+    got = engine.generate(small, max_new_tokens=5, temperature=0.0, eos_token_id=-1)
+    assert got == [oracle.greedy(p, 5) for p in small]
+    with pytest.raises(ValueError):                      # refused on entry: also nothing left
+        engine.generate(small + [[1] * 500], max_new_tokens=4, temperature=0.0)
+    assert engine.stats()["requests"] == 0 and len(engine.runner.cache.handles) == 0

@@ -257,3 +257,30 @@ def test_the_random_workloads_reach_the_hard_cases():
             total[k] = total.get(k, 0) + v
     assert total["preemptions"] >= 10 and total["refused"] >= 1
     assert total["freed"] >= 10 and total["eos"] >= 3 and total["steps"] >= 300
+
+
+def test_abort_gives_everything_back():
+    """A request taken out while it waits, while it runs, and after it has finished:
+    pages, slot and name go back, the others carry on."""
+    cache, sched = make(num_pages=8, page_size=4, num_slots=2, max_num_seqs=2)
+    a, b, c = (Request(n, list(range(6)), 3) for n in "abc")
+    for r in (a, b, c):
+        sched.add(r)
+    plan = sched.schedule()                          # a and b run, c waits (two slots)
+    assert [e.request.id for e in plan] == ["a", "b"]
+    for e in plan:
+        cache.reserve(e.request.id, e.count)
+        cache.commit(e.request.id, e.count)
+    sched.update(plan, {"a": 7, "b": 8})
+    sched.abort(a)                                   # running
+    sched.abort(c)                                   # waiting
+    assert a.phase == FINISHED and a.finish_reason == "aborted" and c.finish_reason == "aborted"
+    assert "a" not in cache.requests and len(cache.handles) == 1
+    cache.check()
+    drive(cache, sched)
+    assert b.phase == FINISHED and b.finish_reason == "length" and len(b.output) == 3
+    sched.abort(b)                                   # finished already: nothing happens
+    assert b.finish_reason == "length"
+    assert not sched.has_work() and len(cache.handles) == 0
+    assert all(g.pool.free_count == g.pool.size for g in cache.groups)
+    assert cache.slots.free_count == 2

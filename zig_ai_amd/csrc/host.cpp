@@ -796,6 +796,17 @@ ZA_EXPORT int za_sched_forget(void* sp, int64_t id) {
   s->reqs.erase(it);
   return ZA_HOST_OK;
 }
+// take a request out, whatever it is doing: what it holds is given back
+ZA_EXPORT int za_sched_abort(void* sp, int64_t id) {
+  Scheduler* s = static_cast<Scheduler*>(sp);
+  auto it = s->reqs.find(id);
+  if (it == s->reqs.end()) return fail(ZA_HOST_ARG, "not a request of this scheduler");
+  if (s->cache->find(id)) s->cache->release(id);
+  s->waiting.erase(std::remove(s->waiting.begin(), s->waiting.end(), id), s->waiting.end());
+  s->running.erase(std::remove(s->running.begin(), s->running.end(), id), s->running.end());
+  s->reqs.erase(it);
+  return ZA_HOST_OK;
+}
 ZA_EXPORT int za_sched_has_work(void* sp) {
   Scheduler* s = static_cast<Scheduler*>(sp);
   return !s->waiting.empty() || !s->running.empty();

@@ -188,10 +188,20 @@ class Engine:
         params = SamplingParams(temperature, top_k, top_p, repetition_penalty, seed)
         if eos_token_id is None:
             eos_token_id = getattr(getattr(self.model, "config", None), "eos_token_id", None)
-        reqs = [self.add_request(p, max_new_tokens, params, eos_token_id)
-                for p in prompt_token_ids]
-        self.run()
+        reqs: List[Request] = []
+        try:
+            for p in prompt_token_ids:
+                reqs.append(self.add_request(p, max_new_tokens, params, eos_token_id))
+            self.run()
+        except BaseException:
+            for r in reqs:                   # leave nothing of this call behind
+                self.abort(r)
+            raise
         return [list(r.output) for r in reqs]
+
+    def abort(self, request: Request) -> None:
+        """Take a request out of the engine; what it holds is given back."""
+        self.scheduler.abort(request)
 
     def stats(self) -> dict:
         out = self.runner.cache.stats()

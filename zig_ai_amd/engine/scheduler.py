@@ -225,6 +225,17 @@ class Scheduler:
             done.append(req)
         return done
 
+    def abort(self, req: Request) -> None:
+        """Take a request out, waiting or running: its pages and slot are given back."""
+        handle = self.cache.handles.known(req.id)
+        if handle is None or handle not in self._requests:
+            return                                   # finished already, or never added
+        raise_for(self._lib.za_sched_abort(self._ptr, handle))
+        req.phase = FINISHED
+        req.finish_reason = "aborted"
+        self._requests.pop(handle, None)
+        self.cache.unpin(req.id)
+
     def _finished(self, req: Request, reason: str) -> None:
         handle = self.cache.handles.of(req.id)
         req.phase = FINISHED

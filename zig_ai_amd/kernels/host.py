@@ -53,6 +53,7 @@ _SIGNATURES = {
     "za_sched_free": (None, [c_void_p]),
     "za_sched_add": (c_int, [c_void_p, c_int64, c_int, c_int, c_int, c_int, _P(c_longlong)]),
     "za_sched_forget": (c_int, [c_void_p, c_int64]),
+    "za_sched_abort": (c_int, [c_void_p, c_int64]),
     "za_sched_has_work": (c_int, [c_void_p]),
     "za_sched_schedule": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                   _P(c_int), c_void_p, _P(c_int)]),
