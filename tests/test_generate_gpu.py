@@ -283,3 +283,21 @@ def test_a_failed_generate_leaves_nothing_behind():
     with pytest.raises(ValueError):                      # refused on entry: also nothing left
         engine.generate(small + [[1] * 500], max_new_tokens=4, temperature=0.0)
     assert engine.stats()["requests"] == 0 and len(engine.runner.cache.handles) == 0
+
+
+def test_command_line_says_what_is_wrong(tmp_path):
+    """No such folder, a folder without weights, a token outside the vocabulary: one
+    line on standard error and exit status 1, no traceback."""
+    folder = folder_for(TINY_A, 0)
+    empty = tmp_path / "empty"
+    empty.mkdir()
+    (empty / "config.json").write_text(open(os.path.join(folder, "config.json")).read())
+    cases = [(["-m", str(tmp_path / "nowhere"), "--prompt-ids", "1 2"], "nowhere"),
+             (["-m", str(empty), "--prompt-ids", "1 2"], "safetensors"),
+             (["-m", folder, "--prompt-ids", "1 999999", "--dtype", "float32"], "999999")]
+    for args, word in cases:
+        out = subprocess.run([sys.executable, "-m", "zig_ai_amd"] + args + ["-n", "2"], cwd=ROOT,
+                             capture_output=True, text=True, timeout=600)
+        assert out.returncode == 1, (args, out.stderr[-500:])
+        assert "Traceback" not in out.stderr and word in out.stderr, (args, out.stderr[-500:])
+        assert out.stderr.strip().splitlines()[-1].startswith("zig-ai: ")

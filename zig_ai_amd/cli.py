@@ -89,7 +89,20 @@ def load_tokenizer(model_dir: str):
 
 
 def main(argv: Optional[List[str]] = None) -> int:
+    """Run the command line; failures the user can act on (no GPU, no such model, a
+    bad configuration or checkpoint, a prompt beyond the limits) are one line on
+    standard error and exit status 1, with the traceback under --verbose."""
     args = build_parser().parse_args(argv)
+    try:
+        return run(args)
+    except (OSError, ValueError, RuntimeError, MemoryError) as err:
+        if args.verbose:
+            raise
+        print(f"zig-ai: {type(err).__name__}: {err}", file=sys.stderr)
+        return 1
+
+
+def run(args) -> int:
     if args.backend == "cpu":
         print("this engine has no CPU path; use --backend gpu", file=sys.stderr)
         return 2
