@@ -48,6 +48,10 @@ int fail(int code, const char* fmt, A... args) {
   g_error = buf;
   return code;
 }
+inline int fail(int code, const char* message) {   // no arguments: not a format string
+  g_error = message;
+  return code;
+}
 
 // ------------------------------------------------------------------ pools
 // `size` numbered items; take() pops the most recently returned one.  A LIFO free
@@ -167,7 +171,7 @@ struct Cache {
   }
   int admit(int64_t req, int* slot_out) {
     if (requests.count(req)) return fail(ZA_HOST_POOL, "the request is already admitted");
-    int slot;
+    int slot = 0;
     if (int rc = slots.take(req, &slot)) return rc;
     RequestCache r;
     r.slot = slot;
@@ -191,7 +195,7 @@ struct Cache {
     for (size_t g = 0; g < groups.size(); ++g) {
       const int n = pages_wanted(*rc, (int)g, n_new);
       for (int i = 0; i < n; ++i) {
-        int page;
+        int page = 0;
         if (int e = groups[g].pool.take(req, &page)) return e;
         if (groups[g].ever_used[page]) ++pages_reused;
         groups[g].ever_used[page] = 1;
