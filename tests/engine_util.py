@@ -1,7 +1,6 @@
 """Helpers shared by the engine tests: model folders in a temporary place, and
 ways of cutting the same requests into steps."""
 
-import os
 import random
 import tempfile
 

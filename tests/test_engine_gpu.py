@@ -8,7 +8,6 @@ request): 32-bit 1e-4 (accumulation order over a few layers); bfloat16 2.5e-2
 (about 40 roundings of 2^-9 along the path, worst entry of thousands).
 """
 
-import math
 
 import pytest
 import torch

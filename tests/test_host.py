@@ -2,13 +2,12 @@
 layout computed here independently, the preparation of decode steps, the uniform
 streams."""
 
-import ctypes
 
 import numpy as np
 import pytest
 import torch
 
-from zig_ai_amd.cache import FREED, CacheManager, OutOfPages
+from zig_ai_amd.cache import FREED, CacheManager
 from zig_ai_amd.engine import StepEntry, StepError, build_step
 from zig_ai_amd.kernels import host as hostlib
 from zig_ai_amd.parts import PagedNeed, StateNeed

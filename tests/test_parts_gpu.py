@@ -2,7 +2,6 @@
 the plain formulas: norm, embedding and head, SwiGLU, the ShortConv mixer with its
 state slot, the attention mixer with its pages, and the block arrangement."""
 
-import math
 
 import pytest
 import torch

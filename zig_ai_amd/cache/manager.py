@@ -35,7 +35,7 @@ import torch
 
 from ..kernels import host
 from ..parts.base import PagedNeed, StateNeed
-from .pages import OutOfPages, OutOfSlots, Pool, PoolError, raise_for
+from .pages import Pool, raise_for
 
 FREED = -1   # block-table entry of a page that was given back (behind the window)
 

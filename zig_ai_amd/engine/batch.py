@@ -17,7 +17,7 @@ from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 import numpy as np
 import torch
 
-from ..cache.manager import FREED, CacheManager
+from ..cache.manager import CacheManager
 from ..cache.pages import raise_for
 from ..kernels import host as hostlib
 

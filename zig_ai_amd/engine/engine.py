@@ -9,7 +9,7 @@ requests at once.
 from __future__ import annotations
 
 import time
-from typing import Dict, Hashable, List, Optional, Sequence
+from typing import Hashable, List, Optional, Sequence
 
 import torch
 

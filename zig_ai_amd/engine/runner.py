@@ -14,11 +14,10 @@ written for several sequences (``num_seqs``, ``block_tables[seq]``:
 
 from __future__ import annotations
 
-from typing import Callable, Hashable, List, Optional, Sequence
+from typing import Callable, Hashable, List, Sequence
 
 import torch
 
-from ..cache.manager import CacheManager
 from ..cache.pages import OutOfPages
 from .batch import StepContext, StepEntry, StepError, build_step
 from .graphs import DecodeGraphs

@@ -10,7 +10,7 @@ handles; ``Handles`` is that table.
 from __future__ import annotations
 
 import ctypes
-from ctypes import POINTER, c_char_p, c_float, c_int, c_int64, c_longlong, c_uint64, c_void_p
+from ctypes import POINTER, c_char_p, c_int, c_int64, c_longlong, c_void_p
 from typing import Dict, Hashable, Optional
 
 from . import build

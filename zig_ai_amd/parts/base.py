@@ -20,7 +20,7 @@ the other; ``step`` says where each request's rows begin and what it has cached.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Callable, Dict, Mapping, Optional, Tuple
+from typing import Any, Dict, Mapping, Optional, Tuple
 
 import torch
 

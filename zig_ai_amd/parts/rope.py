@@ -11,11 +11,9 @@ fused query/key kernel; this part only owns the constants.
 
 from __future__ import annotations
 
-from typing import Any, Dict, Mapping
-
 import torch
 
-from .base import PositionEncoding, Runtime, TensorRule, register_position
+from .base import PositionEncoding, Runtime, register_position
 
 
 class RotaryEmbedding(PositionEncoding):

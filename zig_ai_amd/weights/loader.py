@@ -19,7 +19,7 @@ Precision kept on the device:
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Dict, Iterator, List, Mapping, Tuple
+from typing import Any, Dict, Iterator, List, Tuple
 
 import torch
 
