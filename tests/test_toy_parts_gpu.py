@@ -2,7 +2,9 @@
 toy architecture around it, both defined here, are registered, built from a
 model folder, and stepped through the engine's step function, cache manager and
 run order without a change to the framework's files.  Also: a run order that
-names a layer twice, and a layer that reads another layer's cache.
+names a layer twice, and a layer that reads another layer's cache; and a second
+toy architecture with a feed-forward that routes tokens to experts and a position
+encoding of another kind, beside the framework's own ShortConv mixer.
 """
 
 import pytest
@@ -174,3 +176,197 @@ def test_toy_architecture_steps_through_the_engine(dtype):
         # the window of 9 lets pages behind it go back while the request still runs
         assert runner.cache.stats()["groups"][0]["pages_high_water"] < sum(
             (n + 3) // 4 for n in lengths)
+
+
+# ------------------------------ a feed-forward with routing, another position encoding
+def routed_classes():
+    from zig_ai_amd.kernels import ops
+    from zig_ai_amd.parts import (FeedForward, PositionEncoding, TensorRule, register_feed_forward,
+                                  register_position)
+
+    class TopOneExperts(FeedForward):
+        """Every token goes to the expert whose router logit is largest (the first of
+        equals) and takes that expert's SwiGLU, weighted by the softmax probability
+        of the choice.  Router logits and softmax in 32-bit.  The part looks at the
+        choices on the host, so it is not safe to record into a graph."""
+        kind = "toy_top_one_experts"
+        kernel_sources = ("gemm", "activation")
+
+        @classmethod
+        def tensor_rules(cls, params):
+            H, I, E = int(params["hidden_size"]), int(params["intermediate_size"]), int(params["experts"])
+            rules = {"router.weight": TensorRule(((E, H),))}
+            for e in range(E):
+                rules[f"experts.{e}.gate_up.weight"] = TensorRule(((2 * I, H),))
+                rules[f"experts.{e}.down.weight"] = TensorRule(((H, I),))
+            return rules
+
+        def __init__(self, params, tensors, runtime):
+            super().__init__(params, tensors, runtime)
+            self.experts = int(params["experts"])
+            self.router = tensors["router.weight"].float()
+            self.gate_up = [tensors[f"experts.{e}.gate_up.weight"] for e in range(self.experts)]
+            self.down = [tensors[f"experts.{e}.down.weight"] for e in range(self.experts)]
+
+        def forward(self, x, step=None):
+            logits = ops.linear(x, self.router, out_dtype=torch.float32)
+            prob = torch.softmax(logits, dim=-1)
+            weight, choice = prob.max(dim=-1)
+            out = torch.zeros((x.shape[0], x.shape[1]), dtype=torch.float32, device=x.device)
+            for e in range(self.experts):
+                rows = (choice == e).nonzero().view(-1)
+                if rows.numel() == 0:
+                    continue
+                a = ops.swiglu(ops.linear(x.index_select(0, rows).contiguous(), self.gate_up[e]))
+                y = ops.linear(a, self.down[e], out_dtype=torch.float32)
+                out.index_copy_(0, rows, y * weight.index_select(0, rows)[:, None])
+            return out.to(x.dtype)
+
+    class AddedWaves(PositionEncoding):
+        """Absolute positions: element i of every query and key head takes
+        ``amplitude * sin(position * rate^i + i)``."""
+        kind = "toy_added_waves"
+
+        def __init__(self, params, tensors, runtime):
+            super().__init__(params, tensors, runtime)
+            d = int(params["head_dim"])
+            i = torch.arange(d, dtype=torch.float32, device=runtime.device)
+            self.rates = float(params["rate"]) ** i
+            self.phase = i
+            self.amplitude = float(params["amplitude"])
+
+        def apply(self, q, k, positions):
+            wave = self.amplitude * torch.sin(positions.float()[:, None] * self.rates + self.phase)
+            return (q.float() + wave[:, None, :]).to(q.dtype), (k.float() + wave[:, None, :]).to(k.dtype)
+
+    register_feed_forward(TopOneExperts.kind, TopOneExperts)
+    register_position(AddedWaves.kind, AddedWaves)
+
+
+class RoutedConfig:
+    """Attention with the toy position encoding, and the framework's own ShortConv
+    mixer, each followed by the routed feed-forward."""
+
+    def __init__(self, data):
+        self.data = dict(data)
+
+    @classmethod
+    def from_dict(cls, data):
+        return cls(data)
+
+    def to_dict(self):
+        return dict(self.data)
+
+    def to_spec(self):
+        from zig_ai_amd.config.spec import LayerCall, LayerSpec, ModelSpec, PartSpec
+        d = self.data
+        H, V, E, I = d["width"], d["vocab_size"], d["experts"], d["ffn"]
+        layers = []
+        for i, kind in enumerate(d["kinds"]):
+            p = f"layers.{i}."
+            if kind == "conv":
+                mixer = PartSpec("short_conv", {"hidden_size": H, "kernel_size": d["taps"], "bias": False},
+                                 {k + ".weight": (p + k + ".weight",) for k in ("in_proj", "conv", "out_proj")})
+            else:
+                waves = PartSpec("toy_added_waves", {"head_dim": d["head_dim"], "rate": 0.7, "amplitude": 0.5})
+                mixer = PartSpec("gqa_attention",
+                                 {"hidden_size": H, "num_heads": d["heads"], "num_kv_heads": d["kv_heads"],
+                                  "head_dim": d["head_dim"], "qk_norm": True, "norm_eps": 1e-5,
+                                  "bias": False, "position": waves},
+                                 {k + ".weight": (p + k + ".weight",)
+                                  for k in ("q_proj", "k_proj", "v_proj", "out_proj", "q_norm", "k_norm")})
+            names = {"router.weight": (p + "router.weight",)}
+            for e in range(E):
+                names[f"experts.{e}.gate_up.weight"] = (p + f"experts.{e}.gate_up.weight",)
+                names[f"experts.{e}.down.weight"] = (p + f"experts.{e}.down.weight",)
+            ffn = PartSpec("toy_top_one_experts", {"hidden_size": H, "intermediate_size": I, "experts": E}, names)
+            n1 = PartSpec("rms_norm", {"width": H, "eps": 1e-5}, {"weight": (p + "norm1.weight",)})
+            n2 = PartSpec("rms_norm", {"width": H, "eps": 1e-5}, {"weight": (p + "norm2.weight",)})
+            layers.append(LayerSpec(mixer, ffn, n1, n2))
+        schedule = tuple(LayerCall(i, i) for i in range(len(layers)))
+        return ModelSpec("ToyRoutedForCausalLM", H, V,
+                         PartSpec("token_embedding", {"vocab_size": V, "hidden_size": H},
+                                  {"weight": ("embed.weight",)}),
+                         tuple(layers), schedule,
+                         PartSpec("rms_norm", {"width": H, "eps": 1e-5}, {"weight": ("norm.weight",)}),
+                         PartSpec("linear_head", {"vocab_size": V, "hidden_size": H, "tied": True}, {}))
+
+
+ROUTED = {"architectures": ["ToyRoutedForCausalLM"], "width": 40, "vocab_size": 83, "ffn": 56,
+          "experts": 3, "heads": 5, "kv_heads": 1, "head_dim": 16, "taps": 2,
+          "kinds": ["attn", "conv", "attn"]}
+
+
+def routed_oracle(folder, tokens):
+    """The routed toy model, whole sequence, float64, written out directly; also
+    returns the smallest gap between the two largest router logits of any token
+    (a choice within rounding of a tie is no fault of the engine's)."""
+    from safetensors.torch import load_file
+    w = {k: v.double() for k, v in load_file(folder + "/model.safetensors").items()}
+    d = ROUTED
+    H, nh, nkv, hd, L = d["width"], d["heads"], d["kv_heads"], d["head_dim"], d["taps"]
+    T = len(tokens)
+    x = w["embed.weight"][torch.tensor(tokens)]
+    pos = torch.arange(T, dtype=torch.float64)
+    i = torch.arange(hd, dtype=torch.float64)
+    wave = 0.5 * torch.sin(pos[:, None] * (0.7 ** i) + i)
+    gap = float("inf")
+    for layer, kind in enumerate(d["kinds"]):
+        p = f"layers.{layer}."
+        n1 = plain.rms_norm(x, w[p + "norm1.weight"], 1e-5)
+        if kind == "conv":
+            z = n1 @ w[p + "in_proj.weight"].T
+            u = z[:, :H] * z[:, 2 * H:]
+            m = (z[:, H:2 * H] * plain.causal_depthwise_conv(u, w[p + "conv.weight"].view(H, L), None)) \
+                @ w[p + "out_proj.weight"].T
+        else:
+            q = plain.rms_norm((n1 @ w[p + "q_proj.weight"].T).view(T, nh, hd), w[p + "q_norm.weight"], 1e-5)
+            k = plain.rms_norm((n1 @ w[p + "k_proj.weight"].T).view(T, nkv, hd), w[p + "k_norm.weight"], 1e-5)
+            v = (n1 @ w[p + "v_proj.weight"].T).view(T, nkv, hd)
+            o = plain.causal_attention(q + wave[:, None, :], k + wave[:, None, :], v)
+            m = o.reshape(T, nh * hd) @ w[p + "out_proj.weight"].T
+        h = x + m
+        n2 = plain.rms_norm(h, w[p + "norm2.weight"], 1e-5)
+        logits = n2 @ w[p + "router.weight"].T
+        top = torch.sort(logits, dim=-1, descending=True).values
+        gap = min(gap, float((top[:, 0] - top[:, 1]).min()))
+        prob = torch.softmax(logits, dim=-1)
+        f = torch.zeros_like(h)
+        for t in range(T):
+            e = int(torch.argmax(logits[t]))
+            gu = n2[t] @ w[p + f"experts.{e}.gate_up.weight"].T
+            a = torch.nn.functional.silu(gu[: d["ffn"]]) * gu[d["ffn"]:]
+            f[t] = prob[t, e] * (a @ w[p + f"experts.{e}.down.weight"].T)
+        x = h + f
+    return plain.rms_norm(x, w["norm.weight"], 1e-5) @ w["embed.weight"].T, gap
+
+
+def test_toy_routing_and_position_parts_step_through_the_engine():
+    """A feed-forward that routes and a position encoding of another kind, both
+    defined here, beside the framework's own mixers: registered, built and stepped
+    in 32-bit under three ways of cutting the work.  (In bfloat16 a token whose two
+    best router logits lie within rounding of each other may go to the other expert,
+    which no tolerance of the logits covers; the 32-bit path decides the same as the
+    plain formulas as long as no gap is within 1e-4, which is asserted.)"""
+    from zig_ai_amd.config import register_architecture
+    from zig_ai_amd.engine import DecoderModel, ModelRunner
+    routed_classes()
+    register_architecture("ToyRoutedForCausalLM", RoutedConfig)
+    folder = eu.model_folder(ROUTED, 13, torch.float32, std=0.2, norm_init="around_one",
+                             role_std={"norm": 0.2, "filter": 0.5})
+    model = DecoderModel.from_folder(folder, "float32")
+    assert not model.graph_safe          # the routed feed-forward looks at its choices on the host
+    lengths = [31, 6, 18]
+    prompts = [eu.random_tokens(n, 83, 700 + n) for n in lengths]
+    expect = []
+    for p in prompts:
+        logits, gap = routed_oracle(folder, p)
+        assert gap > 1e-4
+        expect.append(logits)
+    for schedule in (eu.whole(lengths), eu.changing_portions(lengths, 2),
+                     eu.mixed(lengths, seed=5, max_live=3, decode_tail=4)):
+        runner = ModelRunner(model, page_size=4, num_pages=20, num_slots=3)
+        assert runner.graphs is None
+        got = eu.run_schedule(runner, prompts, schedule)
+        for g, e in zip(got, expect):
+            assert eu.rel_err(g, e) < 1e-4
