@@ -1,0 +1,152 @@
+// Plain bfloat16 matrix products with many rows through the GEMM library (hipBLASLt),
+// called directly: the reference sends every projection to its vendor's library too
+// (/root/reference/src/matmul/root.zig:292-313 calls cuBLAS).
+//
+//   y [M, N] = x [M, K] . w [N, K]^T          bfloat16 in, 32-bit sums, bfloat16 or
+//                                              32-bit out
+//   y [P, M, N] (32-bit) with K cut into P ranges, as one batched product: partial
+//                                              sums that the consumer adds up
+//
+// No device code here.  What a call costs on the host matters for steps of a few
+// hundred tokens, which issue some sixty of these products: the descriptors and the
+// algorithm the library's heuristic names for a shape are made once per (device,
+// M, N, K, output type, P) and kept, so a later call is one hipblasLtMatmul.
+// The same shape therefore always runs the same kernel, recorded in a graph or not.
+#include <hip/hip_runtime.h>
+#include <hipblaslt/hipblaslt.h>
+
+#include <map>
+#include <mutex>
+#include <string>
+#include <tuple>
+
+#include "common.h"
+
+#define ZA_API extern "C" __attribute__((visibility("default")))
+
+namespace {
+
+struct Plan {
+  hipblasLtMatmulDesc_t op = nullptr;
+  hipblasLtMatrixLayout_t a = nullptr, b = nullptr, c = nullptr;
+  hipblasLtMatmulAlgo_t algo;
+  size_t workspace = 0;
+  bool usable = false;
+};
+
+using Key = std::tuple<int, int, int, int, int, int>;   // device, M, N, K, output type, P
+
+std::mutex g_lock;
+std::map<int, hipblasLtHandle_t> g_handles;
+std::map<Key, Plan> g_plans;
+thread_local std::string g_error;
+
+int fail(int code, const std::string& what) {
+  g_error = what;
+  return code;
+}
+
+bool ok(hipblasStatus_t s, const char* what, std::string* why) {
+  if (s == HIPBLAS_STATUS_SUCCESS) return true;
+  *why = std::string(what) + " failed with hipBLAS status " + std::to_string((int)s);
+  return false;
+}
+
+// Column-major terms: y^T (N x M, leading dimension N) = w (stored K x N, transposed)
+// times x^T (stored K x M).  A range p of K starts p * K/P elements into a row of
+// either operand; its result is the p-th [M, N] block of y.
+bool make_plan(hipblasLtHandle_t handle, int M, int N, int K, int out_f32, int P,
+               size_t workspace_bytes, Plan* plan, std::string* why) {
+  const int kp = K / P;
+  const hipDataType out_type = out_f32 ? HIP_R_32F : HIP_R_16BF;
+  if (!ok(hipblasLtMatmulDescCreate(&plan->op, HIPBLAS_COMPUTE_32F, HIP_R_32F), "MatmulDescCreate", why))
+    return false;
+  const int32_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
+  if (!ok(hipblasLtMatmulDescSetAttribute(plan->op, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta)),
+          "set TRANSA", why) ||
+      !ok(hipblasLtMatmulDescSetAttribute(plan->op, HIPBLASLT_MATMUL_DESC_TRANSB, &tb, sizeof(tb)),
+          "set TRANSB", why))
+    return false;
+  if (!ok(hipblasLtMatrixLayoutCreate(&plan->a, HIP_R_16BF, kp, N, K), "layout of w", why) ||
+      !ok(hipblasLtMatrixLayoutCreate(&plan->b, HIP_R_16BF, kp, M, K), "layout of x", why) ||
+      !ok(hipblasLtMatrixLayoutCreate(&plan->c, out_type, N, M, N), "layout of y", why))
+    return false;
+  if (P > 1) {
+    const int32_t count = P;
+    const int64_t in_stride = kp, out_stride = (int64_t)M * N;
+    hipblasLtMatrixLayout_t layouts[3] = {plan->a, plan->b, plan->c};
+    for (int i = 0; i < 3; ++i) {
+      const int64_t stride = i < 2 ? in_stride : out_stride;
+      if (!ok(hipblasLtMatrixLayoutSetAttribute(layouts[i], HIPBLASLT_MATRIX_LAYOUT_BATCH_COUNT, &count,
+                                                sizeof(count)), "set batch count", why) ||
+          !ok(hipblasLtMatrixLayoutSetAttribute(layouts[i], HIPBLASLT_MATRIX_LAYOUT_STRIDED_BATCH_OFFSET,
+                                                &stride, sizeof(stride)), "set batch stride", why))
+        return false;
+    }
+  }
+  hipblasLtMatmulPreference_t pref = nullptr;
+  if (!ok(hipblasLtMatmulPreferenceCreate(&pref), "PreferenceCreate", why)) return false;
+  const uint64_t limit = workspace_bytes;
+  hipblasLtMatmulHeuristicResult_t found[1];
+  int n_found = 0;
+  bool good = ok(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES,
+                                                       &limit, sizeof(limit)), "set workspace limit", why) &&
+              ok(hipblasLtMatmulAlgoGetHeuristic(handle, plan->op, plan->a, plan->b, plan->c, plan->c, pref,
+                                                 1, found, &n_found), "AlgoGetHeuristic", why);
+  hipblasLtMatmulPreferenceDestroy(pref);
+  if (!good) return false;
+  if (n_found < 1 || found[0].state != HIPBLAS_STATUS_SUCCESS || found[0].workspaceSize > workspace_bytes) {
+    *why = "the library names no algorithm for this shape";
+    return true;   // a plan that is not usable: the caller takes another kernel
+  }
+  plan->algo = found[0].algo;
+  plan->workspace = found[0].workspaceSize;
+  plan->usable = true;
+  return true;
+}
+
+}  // namespace
+
+ZA_API const char* za_lt_last_error() { return g_error.c_str(); }
+
+// Returns 0, ZA_ERR_ARG, ZA_ERR_UNSUPPORTED (the library has no algorithm for the
+// shape: nothing was launched) or a positive hipBLAS status.
+ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int K, int out_f32,
+                        int P, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  if (!x || !w || !y || M < 1 || N < 1 || K < 1 || P < 1 || K % P || (P > 1 && !out_f32))
+    return fail(ZA_ERR_ARG, "za_lt_matmul: bad argument");
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return fail(ZA_ERR_ARG, "za_lt_matmul: no current device");
+  Plan plan;
+  hipblasLtHandle_t handle = nullptr;
+  {
+    std::lock_guard<std::mutex> guard(g_lock);
+    auto h = g_handles.find(device);
+    if (h == g_handles.end()) {
+      hipblasLtHandle_t made = nullptr;
+      const hipblasStatus_t s = hipblasLtCreate(&made);
+      if (s != HIPBLAS_STATUS_SUCCESS) return fail((int)s, "hipblasLtCreate failed");
+      h = g_handles.emplace(device, made).first;
+    }
+    handle = h->second;
+    const Key key(device, M, N, K, out_f32, P);
+    auto it = g_plans.find(key);
+    if (it == g_plans.end()) {
+      Plan made;
+      std::string why;
+      if (!make_plan(handle, M, N, K, out_f32, P, workspace_bytes, &made, &why))
+        return fail(ZA_ERR_ARG, "za_lt_matmul: " + why);
+      it = g_plans.emplace(key, made).first;
+    }
+    plan = it->second;
+  }
+  if (!plan.usable || plan.workspace > workspace_bytes)
+    return fail(ZA_ERR_UNSUPPORTED, "za_lt_matmul: the library names no algorithm for this shape");
+  const float one = 1.0f, zero = 0.0f;
+  const hipblasStatus_t s = hipblasLtMatmul(handle, plan.op, &one, w, plan.a, x, plan.b, &zero, y, plan.c,
+                                            y, plan.c, &plan.algo, workspace, workspace_bytes, stream);
+  if (s != HIPBLAS_STATUS_SUCCESS)
+    return fail((int)s > 0 ? (int)s : ZA_ERR_ARG,
+                "hipblasLtMatmul failed with hipBLAS status " + std::to_string((int)s));
+  return 0;
+}

@@ -100,7 +100,9 @@ class DecoderModel:
         # Compile what this model's parts use (and the host library), together, before
         # the first step.
         if self.kernel_sources:
-            wanted = list(self.kernel_sources) + list(kernel_build.HOST_SOURCES)
+            wanted = list(self.kernel_sources) + ["host"]
+            if "gemm" in self.kernel_sources and runtime.dtype == torch.bfloat16:
+                wanted.append("blaslt")     # products of many rows go to the GEMM library
             kernel_build.build_all(wanted, jobs=len(wanted))
 
     # ------------------------------------------------------------- construction

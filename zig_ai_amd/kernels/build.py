@@ -27,7 +27,7 @@ from typing import Dict, Iterable, List, Optional
 PACKAGE_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC_DIR = os.path.join(PACKAGE_DIR, "csrc")
 ARCH = "gfx950"
-SOURCES = ("norm", "gemm", "rope_kv", "attention", "shortconv", "activation", "sampling")
+SOURCES = ("norm", "gemm", "rope_kv", "attention", "shortconv", "activation", "sampling", "blaslt")
 HOST_SOURCES = ("host", "plain")    # plain C++, no device code: usable without a GPU or ROCm
 ALL_SOURCES = SOURCES + HOST_SOURCES
 CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden"]
@@ -36,6 +36,8 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
+
+EXTRA_FLAGS = {"blaslt": ["-lhipblaslt"]}   # host code around the GEMM library, no kernels
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
@@ -96,7 +98,7 @@ def source_digest(name: str) -> str:
     for path in ([] if host else [os.path.join(CSRC_DIR, "common.h")]) + [_source_of(name)]:
         with open(path, "rb") as f:
             h.update(f.read())
-    h.update(" ".join(CXX_FLAGS if host else HIPCC_FLAGS).encode())
+    h.update(" ".join((CXX_FLAGS if host else HIPCC_FLAGS) + EXTRA_FLAGS.get(name, [])).encode())
     return h.hexdigest()
 
 
@@ -146,7 +148,7 @@ def compile_one(name: str) -> str:
     out_dir = _writable_lib_dir()
     so = os.path.join(out_dir, f"lib{name}.so")
     tmp = os.path.join(out_dir, f".lib{name}.{os.getpid()}.{threading.get_ident()}.so")
-    cmd = [cxx] + flags + ["-I", CSRC_DIR, "-o", tmp, src]
+    cmd = [cxx] + flags + ["-I", CSRC_DIR, "-o", tmp, src] + EXTRA_FLAGS.get(name, [])
     what = os.path.basename(src)
     env = dict(os.environ)
     home = env.get("HOME", "")

@@ -17,6 +17,7 @@ import torch
 from . import build
 
 c_int, c_float, c_void_p, c_longlong = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_longlong
+c_size_t = ctypes.c_size_t
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 
@@ -60,6 +61,8 @@ _SIGNATURES = {
                                 c_void_p, c_int, c_void_p],
     ("sampling", "za_repetition_penalty"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                                             c_void_p],
+    ("blaslt", "za_lt_matmul"): [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                 c_void_p, c_size_t, c_void_p],
 }
 _functions = {}
 
@@ -231,6 +234,37 @@ def _k_splits(M: int, N: int, K: int) -> int:
     return 1
 
 
+LIBRARY_WORKSPACE_BYTES = 64 << 20
+_library_workspace = {}
+
+
+def _library_matmul(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype,
+                    splits: int) -> Optional[torch.Tensor]:
+    """``x @ weight^T`` through the GEMM library (csrc/blaslt.hip): ``[M, N]``, or the
+    stack ``[splits, M, N]`` of 32-bit partial sums over ranges of K.  ``None`` when
+    the library names no algorithm for the shape (nothing was launched)."""
+    M, K = x.shape
+    N = weight.shape[0]
+    device = x.device.index or 0
+    work = _library_workspace.get(device)
+    if work is None:
+        work = torch.empty((LIBRARY_WORKSPACE_BYTES,), dtype=torch.uint8, device=x.device)
+        _library_workspace[device] = work
+    f32 = splits > 1 or out_dtype == torch.float32
+    shape = (splits, M, N) if splits > 1 else (M, N)
+    out = torch.empty(shape, dtype=torch.float32 if f32 else torch.bfloat16, device=x.device)
+    rc = _fn("blaslt", "za_lt_matmul")(_ptr(x), _ptr(weight), _ptr(out), M, N, K, 1 if f32 else 0,
+                                       splits, _ptr(work), LIBRARY_WORKSPACE_BYTES, _stream())
+    if rc == -2:
+        return None
+    if rc != 0:
+        why = build.load("blaslt").za_lt_last_error
+        why.restype = ctypes.c_char_p
+        raise KernelError(f"library matmul M={M} N={N} K={K} splits={splits}: "
+                          f"{why().decode('utf-8', 'replace')}")
+    return out
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
            out_dtype: Optional[torch.dtype] = None, force_tiled: bool = False,
            partial_ok: bool = False) -> torch.Tensor:
@@ -279,15 +313,11 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
                                                 0, M, N, K, splits, 0, _stream())
         _check(rc, "gemm_bf16_rows16", f"M={M} N={N} K={K} splits={splits}")
         return stack
-    if splits > 1:
-        # One batched product over the ranges of K: [P, M, K/P] x [P, K/P, N], both views.
-        xs = x.view(M, splits, K // splits).transpose(0, 1)
-        ws = weight.view(N, splits, K // splits).permute(1, 2, 0)
-        return torch.bmm(xs, ws, out_dtype=torch.float32)
     if library:
-        if out_dtype == torch.float32:
-            return torch.mm(x, weight.t(), out_dtype=torch.float32)
-        return torch.mm(x, weight.t())
+        # (with ranges of K: one batched product, [P, M, K/P] x [P, K/P, N])
+        out = _library_matmul(x, weight, out_dtype, splits)
+        if out is not None:
+            return out
     out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     rc = _fn("gemm", "za_gemm_bf16")(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out),
                                      _code(out_dtype), M, N, K, 1 if force_tiled else 0,
