@@ -77,7 +77,10 @@ def serve(cfg, name, n_requests, new_tokens) -> int:
         write_random_model(config_from_dict(cfg), folder, seed=0, dtype=torch.bfloat16)
         engine = Engine(folder, dtype="bfloat16", page_size=16, max_num_seqs=64,
                         max_num_batched_tokens=4096, chunk_size=2048, max_model_len=4096)
-        engine.generate(prompts[:2], max_new_tokens=4, temperature=0.0, eos_token_id=-1)   # warm-up
+        # warm-up: every kind of step once (more than 16 rows of logits among them),
+        # so that no library loads its kernels inside the timed run
+        engine.generate([p[:64] for p in prompts[:20]], max_new_tokens=4, temperature=0.7, seed=3,
+                        eos_token_id=-1)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         out = engine.generate(prompts, max_new_tokens=new_tokens, temperature=0.7, seed=3,

@@ -364,13 +364,13 @@ def test_decode_steps_hand_tokens_over_on_the_device(dtype):
 
 def test_recorded_shapes_are_dropped_when_there_are_too_many(monkeypatch):
     """Only so many recorded steps are kept; the one used longest ago goes, and comes
-    back (recorded anew) when its shape does.  Three batch sizes in turn with room for
-    two: every step still gives the plain implementation's logits."""
+    back (recorded anew) when its shape does.  Three batch sizes in turn, three steps
+    each, with room for two: every step still gives the plain implementation's logits."""
     from zig_ai_amd.engine import StepEntry, graphs
     monkeypatch.setattr(graphs, "MAX_GRAPHS", 2)
     model, expect, prompts = setup("B", "float32")
     runner = runner_for(model, 8, 64, num_slots=4)
-    live = [2, 3, 4]                                   # 31, 64 and 100 tokens
+    live = [4, 3, 2]                                   # 100, 64 and 31 tokens
     got = {i: [] for i in live}
     cursor = {}
     for i in live:
@@ -378,7 +378,9 @@ def test_recorded_shapes_are_dropped_when_there_are_too_many(monkeypatch):
         got[i].append(runner.step([StepEntry(i, prompts[i][:20], list(range(20)))]).cpu())
         cursor[i] = 20
     for step in range(33):
-        members = live[:1 + step % 3]                  # batch sizes 1, 2, 3, 1, 2, 3 ...
+        # batch sizes 1, 1, 1, 2, 2, 2, 3, 3, 3, 1 ...: a shape's first step runs
+        # unrecorded, its second is recorded and replayed, its third replayed
+        members = live[:1 + (step // 3) % 3]
         members = [i for i in members if cursor[i] < len(prompts[i])]
         if not members:
             break
@@ -388,6 +390,7 @@ def test_recorded_shapes_are_dropped_when_there_are_too_many(monkeypatch):
             cursor[i] += 1
         assert len(runner.graphs.entries) <= 2
     assert runner.graphs.captures > 3                  # shapes were recorded again
+    assert runner.graphs.replays >= 2 * runner.graphs.captures - 1
     for i in live:
         have = torch.cat(got[i])
         assert eu.rel_err(have, expect[i][:have.shape[0]]) < TOL["float32"]

@@ -5,9 +5,9 @@ hundred small kernels; recorded once into a HIP graph and replayed, the step
 costs one launch.  The reference does the same for its single sequence
 (/root/reference/src/cuda/decode_graph.zig:44-143) and has to save and restore
 the recurrent state around its capture (85-112) because its capture run also
-executes; here the first step of a shape runs eagerly (its results are the
-step's results) and is then recorded without being executed, so no state is
-touched twice.
+executes; here the first step of a shape runs eagerly (so every kernel the shape
+needs is loaded before anything is recorded) and recording executes nothing, so
+no state is touched twice.
 
 A graph is recorded per shape: number of requests, width of the block tables
 (rounded up, so the table may grow inside the same graph) and the bucket of the
@@ -76,10 +76,17 @@ class DecodeGraphs:
         raise_for(rc)
 
     def run(self, runner, entries: Sequence[StepEntry],
-            device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
+            device_tokens: Optional[torch.Tensor] = None, more_to_come: bool = False) -> torch.Tensor:
         """Logits ``[len(entries), vocab]`` of a step of single tokens (one row per
         entry, whatever the entries want).  Takes the pages the new tokens need (all
         or none: ``OutOfPages`` leaves everything as it was).
+
+        A shape's first step runs eagerly.  Recording costs about as much again and
+        pays from the third step of the shape on, so the shape is recorded at once
+        only when the caller says that ``more_to_come`` (it is about to issue further
+        steps of the same requests); otherwise at its second step, which is then the
+        graph's first replay.  While requests finish one after the other, every step
+        has a batch size of its own that may never come back.
 
         With ``device_tokens`` (int32 ``[len(entries)]`` on the device, for instance
         what the sampler drew from the last step's logits) the entries' own tokens are
@@ -161,7 +168,7 @@ class DecodeGraphs:
             grans = np.asarray(sorted(set(int(g) for g in self._granularities)), dtype=np.int32)
             slot = {"buffer": torch.full((words,), -1, dtype=torch.int32, device=runner.device),
                     "pinned": torch.empty((words,), dtype=torch.int32, pin_memory=True),
-                    "graph": None, "logits": None, "copied": None, "words": words,
+                    "graph": None, "logits": None, "copied": None, "words": words, "seen": 0,
                     "grans": grans,
                     "sections": np.zeros((2 * (7 + 2 * len(cache.groups) + 3 * len(grans)),),
                                          dtype=np.int64)}
@@ -178,7 +185,12 @@ class DecodeGraphs:
         ctx = build_step(asked, cache, runner.device, self._vocab, self._granularities,
                          self._max_position, min_pages=key[1], max_keys=key[2],
                          into=slot["buffer"], prepared=prepared)
-        logits = model.forward(ctx, runner.views)          # this step, eagerly
+        first = slot["seen"] == 0
+        slot["seen"] += 1
+        if first:
+            logits = model.forward(ctx, runner.views)      # this step, eagerly
+            if not more_to_come:
+                return logits
         graph = torch.cuda.CUDAGraph()
         # No collection while the capture is open: a collector run could free
         # device memory or destroy an older graph, which a capture does not allow.
@@ -192,4 +204,8 @@ class DecodeGraphs:
                 gc.enable()
         slot["graph"] = graph
         self.captures += 1
-        return logits
+        if first:
+            return logits
+        graph.replay()                                     # the shape's second step
+        self.replays += 1
+        return slot["logits"]

@@ -91,7 +91,8 @@ class ModelRunner:
         for i in range(n_steps):
             try:
                 if self.graphs is not None:
-                    logits = self.graphs.run(self, entries, device_tokens=current)
+                    logits = self.graphs.run(self, entries, device_tokens=current,
+                                             more_to_come=n_steps > 2)
                 else:
                     if current is not None:
                         entries = [StepEntry(r, [t], [0])
