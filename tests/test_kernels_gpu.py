@@ -155,6 +155,24 @@ def test_gemm_bf16_skinny_and_tiled_agree(M):
     assert rel_err(a, c.double()) < F32_TOL
 
 
+@pytest.mark.parametrize("partial_ok", [False, True])
+def test_gemm_bf16_without_an_algorithm_of_the_library(monkeypatch, partial_ok):
+    """Where the library names no algorithm for a shape (made so here), the product
+    runs on this package's kernels, and the library's own answer agrees with theirs."""
+    x, w = rand((40, 4096), torch.bfloat16, 42), rand((200, 4096), torch.bfloat16, 43)
+    want = x.double() @ w.double().T
+
+    def total(out):
+        return out.sum(0) if out.dim() == 3 else out
+
+    with_library = ops().linear(x.to(dev()), w.to(dev()), out_dtype=torch.float32, partial_ok=partial_ok)
+    assert with_library.dim() == (3 if partial_ok else 2)
+    monkeypatch.setattr(ops(), "_library_matmul", lambda *a: None)
+    without = ops().linear(x.to(dev()), w.to(dev()), out_dtype=torch.float32, partial_ok=partial_ok)
+    assert without.shape == (40, 200)
+    assert rel_err(total(with_library), want) < F32_TOL and rel_err(without, want) < F32_TOL
+
+
 @pytest.mark.parametrize("M", [17, 40, 64, 65, 300])
 @pytest.mark.parametrize("N,K", [(50, 96), (257, 1024), (2048, 2048), (1000, 4096)])
 def test_gemm_bf16_library_keeps_32_bits(M, N, K):
