@@ -237,6 +237,105 @@ def test_gemm_bf16_partial_sums(M, N, K):
     assert many.dim() == 2                                  # only small batches are split
 
 
+def _normed_operands(x: torch.Tensor, weight: torch.Tensor, eps: float):
+    """What the decode kernels make of a norm handed to them: the operands
+    bf16(x * weight) and the row's scale, which multiplies the 32-bit sums."""
+    xd = x.double()
+    scale = 1.0 / torch.sqrt((xd * xd).mean(-1, keepdim=True) + eps)
+    return (x * weight).to(torch.bfloat16).double(), scale
+
+
+@pytest.mark.parametrize("K", [8, 512, 520, 1024, 1536, 2048, 2560, 3584, 4096, 4608])
+@pytest.mark.parametrize("M,N", [(1, 48), (8, 50), (16, 33), (16, 16400), (11, 16385)])
+def test_gemm_bf16_decode_rows_normalised_by_the_kernel(M, N, K):
+    """A norm that has not run yet as the product's input: every K the fused form takes
+    (multiples of 512 up to 4096, also those that leave waves idle; up to 8 rows, or up
+    to 16 with many outputs) and some it does not, with a bias, and rows picked out of a
+    longer stream.  The
+    row's scale is applied to the 32-bit sums, so against the same operands the error
+    is that of 32-bit summation; against the norm as a kernel of its own (which rounds
+    after scaling) it is one bfloat16 rounding."""
+    eps = 1e-5
+    stream = rand((M + 3, K), torch.float32, 50) * 3.0
+    nw = 1.0 + rand((K,), torch.float32, 51)
+    w, b = rand((N, K), torch.bfloat16, 52), rand((N,), torch.float32, 53)
+    rows = torch.tensor([(5 * i + 2) % (M + 3) for i in range(M)], dtype=torch.int32)
+    o = ops()
+    for pick in (None, rows):
+        x = stream[:M] if pick is None else stream[pick.long()]
+        src = stream[:M].contiguous() if pick is None else stream
+        normed = o.NormedRows(src.to(dev()), nw.to(dev()), eps, torch.bfloat16,
+                              None if pick is None else pick.to(dev()))
+        assert normed.shape == (M, K)
+        out = o.linear(normed, w.to(dev()), b.to(dev()), out_dtype=torch.float32)
+        if o.normed_rows_pay(M, N, K):
+            a, scale = _normed_operands(x, nw, eps)
+            assert rel_err(out, scale * (a @ w.double().T) + b.double()) < F32_TOL
+        separate = o.linear(normed.materialise(), w.to(dev()), b.to(dev()), out_dtype=torch.float32)
+        assert rel_err(out, separate.double()) < BF16_TOL
+        exact = plain.rms_norm(x.double(), nw.double(), eps) @ w.double().T + b.double()
+        assert rel_err(out, exact) < BF16_TOL
+
+
+def test_normed_rows_beyond_the_fused_kernel_run_the_norm_kernel():
+    """More than 16 rows, a K no workgroup covers, 32-bit weights: the norm runs as a
+    kernel of its own and the product is the usual one."""
+    o = ops()
+    eps = 1e-6
+    for M, K, wdtype in ((17, 512, torch.bfloat16), (4, 4608, torch.bfloat16), (4, 520, torch.bfloat16),
+                         (4, 512, torch.float32)):
+        x = rand((M, K), torch.float32, 54)
+        nw = 1.0 + rand((K,), torch.float32, 55)
+        w = rand((24, K), wdtype, 56)
+        dtype = torch.bfloat16 if wdtype == torch.bfloat16 else torch.float32
+        normed = o.NormedRows(x.to(dev()), nw.to(dev()), eps, dtype)
+        out = o.linear(normed, w.to(dev()), out_dtype=torch.float32)
+        same = o.linear(normed.materialise(), w.to(dev()), out_dtype=torch.float32)
+        assert torch.equal(out, same)
+        exact = plain.rms_norm(x.double(), nw.double(), eps) @ w.double().T
+        assert rel_err(out, exact) < (BF16_TOL if dtype == torch.bfloat16 else F32_TOL)
+
+
+@pytest.mark.parametrize("M,I,K", [(1, 40, 512), (8, 100, 1536), (16, 256, 2048), (5, 72, 4096)])
+def test_linear_swiglu_normalised_by_the_kernel(M, I, K):
+    eps = 1e-5
+    x = rand((M, K), torch.float32, 57) * 2.0
+    nw = 1.0 + rand((K,), torch.float32, 58)
+    w = rand((2 * I, K), torch.bfloat16, 59)
+    o = ops()
+    normed = o.NormedRows(x.to(dev()), nw.to(dev()), eps, torch.bfloat16)
+    out = o.linear_swiglu(normed, w.to(dev()))
+    a, scale = _normed_operands(x, nw, eps)
+    gu = scale * (a @ w.double().T)
+    g, u = gu[:, :I], gu[:, I:]
+    assert out.dtype == torch.bfloat16
+    assert rel_err(out, g / (1 + torch.exp(-g)) * u) < BF16_TOL
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 64, 4096), (8, 2048, 8192), (16, 2048, 2048), (8, 100, 4160),
+                                   (3, 4096, 512), (8, 2048, 16384), (2, 40, 72)])
+def test_gemm_bf16_decode_rows_added_to_the_stream(M, N, K):
+    """A decode batch's product added to the 32-bit stream by the kernel itself, K in
+    as many ranges as fill the chip; twice, since the stream keeps what it holds."""
+    x, w, b = rand((M, K), torch.bfloat16, 60), rand((N, K), torch.bfloat16, 61), rand((N,), torch.float32, 62)
+    stream0 = rand((M, N), torch.float32, 63)
+    stream = stream0.to(dev())
+    o = ops()
+    assert o.linear(x.to(dev()), w.to(dev()), b.to(dev()), partial_ok=True, accumulate=stream) is None
+    product = x.double() @ w.double().T + b.double()
+    assert rel_err(stream, stream0.double() + product) < F32_TOL
+    assert o.linear(x.to(dev()), w.to(dev()), b.to(dev()), accumulate=stream) is None
+    assert rel_err(stream, stream0.double() + 2 * product) < F32_TOL
+    # more than a decode batch, or 32-bit weights: the product comes back instead
+    many = rand((20, K), torch.bfloat16, 64).to(dev())
+    kept = torch.zeros((20, N), dtype=torch.float32, device=dev())
+    back = o.linear(many, w.to(dev()), accumulate=kept)
+    assert back is not None and not kept.any()
+    kept = torch.zeros((M, N), dtype=torch.float32, device=dev())
+    back = o.linear(x.float().to(dev()), w.float().to(dev()), accumulate=kept)
+    assert back is not None and not kept.any()
+
+
 @pytest.mark.parametrize("M", [17, 40, 64, 200])
 @pytest.mark.parametrize("N,K,few_rows,more_rows", [
     (2048, 8192, 8, 8), (2048, 2048, 8, 1), (300, 4096, 8, 8), (1024, 4608, 4, 4),

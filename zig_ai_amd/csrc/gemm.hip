@@ -16,6 +16,8 @@
 // differ from each other in rounding only).
 #include "common.h"
 
+#include <type_traits>
+
 // ---------------------------------------------------------------- 32-bit FMA
 #define F32_BM 64
 #define F32_BN 64
@@ -267,12 +269,119 @@ gemm_bf16_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__
 // K may also be split over workgroups (gridDim.y ranges of NW * KSTEPS * 32): each
 // range then writes a 32-bit partial result [range][M][N] that the consumer adds up
 // (the bias goes into range 0).
-template <int NW, int KSTEPS, typename TC>
-__global__ void __launch_bounds__(NW * 64)
-gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
-                        const float* __restrict__ bias, TC* __restrict__ C, int M, int N, int K,
-                        int groups_per_block) {
+//
+// With `accumulate` the result is not stored but added to the 32-bit tensor C with
+// floating-point atomics (C is then the residual stream, and the ranges of K meet
+// there instead of in a stack): the order of these additions is the hardware's, so
+// the sum is reproducible to rounding only.
+// The activations of the decode kernels may also be a norm that has not run yet:
+// rows of the 32-bit residual stream `x` (row m of the product is row rows[m] of
+// the stream when `rows` is given) and an RMSNorm's weight and eps
+// (/root/reference/src/transformer/norm.zig:6-33).  Every workgroup then reads the
+// rows itself (they are few and come from L2) and a kernel between the producer of
+// the stream and this product is saved.  The row's scale is a factor common to all of
+// its elements, so it is applied to the 32-bit sums instead of to the operands:
+//   y[m, n] = (1 / sqrt(mean_k(x[m, k]^2) + eps)) * sum_k W[n, k] * bf16(x[m, k] * weight[k])
+// with the sum of squares in 32-bit from the unrounded x; the operands are rounded to
+// bfloat16 once, as they are when the norm runs as a kernel of its own.  The
+// workgroup's waves must cover all of K, and K must be a multiple of a wave's 512.
+struct NormedRowsArg {
+  const float* x;
+  const int* rows;
+  const float* weight;
+  float eps;
+};
+
+// Fills xa with the wave's slice of bf16(x * weight) and leaves the sum of squares of
+// the slice of row r in ssw[wave][r]; `nws` is room for the norm weight of the
+// workgroup's K range.  Ends with a barrier.  K is a multiple of a wave's slice
+// (KSTEPS * 32 elements), so a wave is either all inside K or has nothing to do.  A lane
+// without a row reads row 0 with its neighbours and turns what it read into zeros:
+// straight-line loads from one address with the steps as constant offsets, all in
+// flight together.  `prefetch` is called once the rows are requested, by the waves
+// inside K only.
+template <int NW, int KSTEPS, typename Prefetch>
+__device__ __forceinline__ void load_normed_rows(bf16x8_t (&xa)[KSTEPS],
+                                                 const float* __restrict__ x,
+                                                 const int* __restrict__ rows,
+                                                 const float* __restrict__ weight, int M, int K,
+                                                 int tid, int kbase, float (&ssw)[NW][16],
+                                                 float* nws, Prefetch&& prefetch) {
+  static_assert(KSTEPS == 16, "a thread brings eight elements of the norm weight");
+  const int lane = tid & 63, wave = tid >> 6;
+  const int frag_row = lane & 15;
+  const bool rvalid = frag_row < M;
+  const bool inside = (wave + 1) * (KSTEPS * 32) <= K;      // the same for a whole wave
+  float ss = 0.f;
+  if (inside) {
+    const int row = rvalid ? frag_row : 0;
+    const size_t src = rows ? (size_t)rows[row] : (size_t)row;
+    const float* xk = x + src * K + kbase;
+    const f32x4_t n0 = *reinterpret_cast<const f32x4_t*>(weight + tid * 8);
+    const f32x4_t n1 = *reinterpret_cast<const f32x4_t*>(weight + tid * 8 + 4);
+    f32x4_t xf[KSTEPS][2];
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+      xf[s][0] = *reinterpret_cast<const f32x4_t*>(xk + s * 32);
+      xf[s][1] = *reinterpret_cast<const f32x4_t*>(xk + s * 32 + 4);
+    }
+    // the first weights are requested behind the rows and arrive while the rows are
+    // worked on (loads return in the order in which they were issued)
+    __builtin_amdgcn_sched_barrier(0);
+    prefetch();
+    __builtin_amdgcn_sched_barrier(0);
+    // a wave reads only the norm weights that its own lanes brought: no barrier yet
+    *reinterpret_cast<f32x4_t*>(nws + tid * 8) = n0;
+    *reinterpret_cast<f32x4_t*>(nws + tid * 8 + 4) = n1;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+      // four steps' norm weights at a time: all 32 reads hoisted to the front would
+      // take as many registers again as the rows
+      if (s % 4 == 0) __builtin_amdgcn_sched_barrier(0);
+      const f32x4_t w0 = *reinterpret_cast<const f32x4_t*>(nws + kbase + s * 32);
+      const f32x4_t w1 = *reinterpret_cast<const f32x4_t*>(nws + kbase + s * 32 + 4);
+      bf16x8_t r;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float a = rvalid ? xf[s][0][e] : 0.f;
+        const float b = rvalid ? xf[s][1][e] : 0.f;
+        ss += a * a;
+        ss += b * b;
+        r[e] = (bf16_t)(a * w0[e]);
+        r[4 + e] = (bf16_t)(b * w1[e]);
+      }
+      xa[s] = r;
+    }
+    // the four lanes that hold elements of a row; the waves are added up by the reader
+    ss += __shfl_xor(ss, 16, ZA_WAVE);
+    ss += __shfl_xor(ss, 32, ZA_WAVE);
+  } else {
+    const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) xa[s] = zero8;
+  }
+  if (lane < 16) ssw[wave][lane] = ss;
+  __syncthreads();
+}
+
+// The scale of row m from the waves' sums of squares, added in a fixed order.
+template <int NW>
+__device__ __forceinline__ float normed_row_scale(const float (&ssw)[NW][16], int m, int K, float eps) {
+  float total = ssw[0][m];
+#pragma unroll
+  for (int w = 1; w < NW; ++w) total += ssw[w][m];
+  return 1.0f / sqrtf(total / (float)K + eps);
+}
+
+template <int NW, int KSTEPS, typename TC, bool NORM>
+__global__ void __launch_bounds__(NW * 64, 2)
+gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
+                        const bf16_t* __restrict__ W, const float* __restrict__ bias,
+                        TC* __restrict__ C, int M, int N, int K, int groups_per_block,
+                        int accumulate) {
   __shared__ float red[2][NW][64][4];
+  __shared__ float ssw[NW][16];
+  __shared__ float nws[NORM ? NW * KSTEPS * 32 : 1];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int frag_row = lane & 15, frag_k = (lane >> 4) * 8;
@@ -281,34 +390,62 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__
   constexpr int HALF = KSTEPS > 16 ? 16 : KSTEPS;   // weight fragments in flight at once
 
   bf16x8_t xa[KSTEPS];
+  // NORM: a wave is all inside K or idle, and a row group's weights are loaded without
+  // conditions (a lane beyond N reads row N - 1; its sums are never stored), the first
+  // group's while the rows are on their way
+  [[maybe_unused]] bf16x8_t fn[NORM ? KSTEPS : 1];
+  [[maybe_unused]] const bool inside = (wave + 1) * (KSTEPS * 32) <= K;
+  [[maybe_unused]] auto load_group = [&](int g) {
+    const int wrow = min((int)(blockIdx.x * groups_per_block + g) * 16 + frag_row, N - 1);
+    const bf16_t* wp = W + (size_t)wrow * K + kbase;
 #pragma unroll
-  for (int s = 0; s < KSTEPS; ++s) {
-    const int k = kbase + s * 32;
-    xa[s] = (frag_row < M && k < K) ? *reinterpret_cast<const bf16x8_t*>(A + (size_t)frag_row * K + k)
-                                    : zero8;
+    for (int s = 0; s < KSTEPS; ++s) fn[s] = *reinterpret_cast<const bf16x8_t*>(wp + s * 32);
+  };
+  if constexpr (NORM) {
+    load_normed_rows<NW, KSTEPS>(xa, normed.x, normed.rows, normed.weight, M, K, tid, kbase,
+                                 ssw, nws, [&]() { load_group(0); });
+  } else {
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+      const int k = kbase + s * 32;
+      xa[s] = (frag_row < M && k < K)
+                  ? *reinterpret_cast<const bf16x8_t*>(A + (size_t)frag_row * K + k) : zero8;
+    }
   }
 
-  const bool partial = gridDim.y > 1;
+  const bool partial = gridDim.y > 1 && !accumulate;
   for (int g = 0; g < groups_per_block; ++g) {
     const int n0 = (blockIdx.x * groups_per_block + g) * 16;
     if (n0 >= N) break;
-    const int wrow = n0 + frag_row;
-    const bool wvalid = wrow < N;
-    const bf16_t* wp = W + (size_t)(wvalid ? wrow : 0) * K + kbase;
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-    // all of a row group's weight fragments (HALF of them when a wave's K slice is
-    // long) are requested before the first is used
+    if constexpr (NORM) {
+      if (inside) {
+        if (g > 0) {
+          load_group(g);
+          __builtin_amdgcn_sched_barrier(0);   // every load is requested before the first product
+        }
 #pragma unroll
-    for (int h = 0; h < KSTEPS; h += HALF) {
-      bf16x8_t fw[HALF];
-#pragma unroll
-      for (int s = 0; s < HALF; ++s) {
-        const int k = kbase + (h + s) * 32;
-        fw[s] = (wvalid && k < K) ? *reinterpret_cast<const bf16x8_t*>(wp + (h + s) * 32) : zero8;
+        for (int s = 0; s < KSTEPS; ++s)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fn[s], xa[s], acc, 0, 0, 0);
       }
+    } else {
+      const int wrow = n0 + frag_row;
+      const bool wvalid = wrow < N;
+      const bf16_t* wp = W + (size_t)(wvalid ? wrow : 0) * K + kbase;
+      // all of a row group's weight fragments (HALF of them when a wave's K slice is
+      // long) are requested before the first is used
 #pragma unroll
-      for (int s = 0; s < HALF; ++s)
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[s], xa[h + s], acc, 0, 0, 0);
+      for (int h = 0; h < KSTEPS; h += HALF) {
+        bf16x8_t fw[HALF];
+#pragma unroll
+        for (int s = 0; s < HALF; ++s) {
+          const int k = kbase + (h + s) * 32;
+          fw[s] = (wvalid && k < K) ? *reinterpret_cast<const bf16x8_t*>(wp + (h + s) * 32) : zero8;
+        }
+#pragma unroll
+        for (int s = 0; s < HALF; ++s)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[s], xa[h + s], acc, 0, 0, 0);
+      }
     }
     if (NW > 1) {
       float* mine = red[g & 1][wave][lane];
@@ -319,6 +456,8 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__
     if (wave == 0) {
       const int m = lane & 15, nn = n0 + (lane >> 4) * 4;
       if (m < M) {
+        float scale = 1.f;
+        if constexpr (NORM) scale = normed_row_scale<NW>(ssw, m, K, normed.eps);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int n = nn + r;
@@ -329,8 +468,11 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__
 #pragma unroll
             for (int w = 1; w < NW; ++w) v += red[g & 1][w][lane][r];
           }
+          if constexpr (NORM) v *= scale;
           if (bias && blockIdx.y == 0) v += bias[n];
-          if (partial)
+          if (accumulate)
+            unsafeAtomicAdd(reinterpret_cast<float*>(C) + (size_t)m * N + n, v);
+          else if (partial)
             reinterpret_cast<float*>(C)[((size_t)blockIdx.y * M + m) * N + n] = v;
           else
             C[(size_t)m * N + n] = from_f32<TC>(v);
@@ -346,12 +488,14 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__
 //   C[m, n] = silu(gate[m, n]) * up[m, n],   silu(g) = g / (1 + exp(-g)),
 // from the 32-bit accumulators (/root/reference/src/transformer/ffn.zig:24-30), so
 // the [M, 2I] intermediate never goes to memory.  K is not split over workgroups.
-template <int NW, int KSTEPS>
-__global__ void __launch_bounds__(NW * 64)
-gemm_bf16_rows16_swiglu_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
-                               bf16_t* __restrict__ C, int M, int I, int K,
-                               int groups_per_block) {
+template <int NW, int KSTEPS, bool NORM>
+__global__ void __launch_bounds__(NW * 64, 2)
+gemm_bf16_rows16_swiglu_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
+                               const bf16_t* __restrict__ W, bf16_t* __restrict__ C, int M, int I,
+                               int K, int groups_per_block) {
   __shared__ float red[2][2][NW][64][4];
+  __shared__ float ssw[NW][16];
+  __shared__ float nws[NORM ? NW * KSTEPS * 32 : 1];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int frag_row = lane & 15, frag_k = (lane >> 4) * 8;
@@ -360,34 +504,70 @@ gemm_bf16_rows16_swiglu_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
   constexpr int CHUNK = KSTEPS > 8 ? 8 : KSTEPS;   // fragments of each operand in flight
 
   bf16x8_t xa[KSTEPS];
+  // NORM: as in gemm_bf16_rows16_kernel, with all of a row group's gate and up rows in
+  // registers; the first group's first half is requested with the rows, its second half
+  // once the rows' registers are free
+  [[maybe_unused]] bf16x8_t ng[NORM ? KSTEPS : 1], nu[NORM ? KSTEPS : 1];
+  [[maybe_unused]] const bool inside = (wave + 1) * (KSTEPS * 32) <= K;
+  [[maybe_unused]] auto load_steps = [&](int g, auto first, auto last) {
+    const int wrow = min((int)(blockIdx.x * groups_per_block + g) * 16 + frag_row, I - 1);
+    const bf16_t* gp = W + (size_t)wrow * K + kbase;
+    const bf16_t* up = gp + (size_t)I * K;
 #pragma unroll
-  for (int s = 0; s < KSTEPS; ++s) {
-    const int k = kbase + s * 32;
-    xa[s] = (frag_row < M && k < K) ? *reinterpret_cast<const bf16x8_t*>(A + (size_t)frag_row * K + k)
-                                    : zero8;
+    for (int s = first; s < last; ++s) {
+      ng[s] = *reinterpret_cast<const bf16x8_t*>(gp + s * 32);
+      nu[s] = *reinterpret_cast<const bf16x8_t*>(up + s * 32);
+    }
+  };
+  constexpr std::integral_constant<int, 0> S0{};
+  constexpr std::integral_constant<int, KSTEPS / 2> S1{};
+  constexpr std::integral_constant<int, KSTEPS> S2{};
+  if constexpr (NORM) {
+    load_normed_rows<NW, KSTEPS>(xa, normed.x, normed.rows, normed.weight, M, K, tid, kbase,
+                                 ssw, nws, [&]() { load_steps(0, S0, S1); });
+  } else {
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+      const int k = kbase + s * 32;
+      xa[s] = (frag_row < M && k < K)
+                  ? *reinterpret_cast<const bf16x8_t*>(A + (size_t)frag_row * K + k) : zero8;
+    }
   }
 
   for (int g = 0; g < groups_per_block; ++g) {
     const int n0 = (blockIdx.x * groups_per_block + g) * 16;
     if (n0 >= I) break;
-    const int wrow = n0 + frag_row;
-    const bool wvalid = wrow < I;
-    const bf16_t* gp = W + (size_t)(wvalid ? wrow : 0) * K + kbase;
-    const bf16_t* up = gp + (size_t)I * K;
     f32x4_t ag = {0.f, 0.f, 0.f, 0.f}, au = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (NORM) {
+      if (inside) {
+        if (g > 0) load_steps(g, S0, S1);
+        load_steps(g, S1, S2);
+        __builtin_amdgcn_sched_barrier(0);   // every load is requested before the first product
 #pragma unroll
-    for (int h = 0; h < KSTEPS; h += CHUNK) {
-      bf16x8_t fg[CHUNK], fu[CHUNK];
-#pragma unroll
-      for (int s = 0; s < CHUNK; ++s) {
-        const bool ok = wvalid && kbase + (h + s) * 32 < K;
-        fg[s] = ok ? *reinterpret_cast<const bf16x8_t*>(gp + (h + s) * 32) : zero8;
-        fu[s] = ok ? *reinterpret_cast<const bf16x8_t*>(up + (h + s) * 32) : zero8;
+        for (int s = 0; s < KSTEPS; ++s) {
+          ag = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ng[s], xa[s], ag, 0, 0, 0);
+          au = __builtin_amdgcn_mfma_f32_16x16x32_bf16(nu[s], xa[s], au, 0, 0, 0);
+        }
       }
+    } else {
+      const int wrow = n0 + frag_row;
+      const bool wvalid = wrow < I;
+      const bf16_t* gp = W + (size_t)(wvalid ? wrow : 0) * K + kbase;
+      const bf16_t* up = gp + (size_t)I * K;
 #pragma unroll
-      for (int s = 0; s < CHUNK; ++s) {
-        ag = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fg[s], xa[h + s], ag, 0, 0, 0);
-        au = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fu[s], xa[h + s], au, 0, 0, 0);
+      for (int h = 0; h < KSTEPS; h += CHUNK) {
+        bf16x8_t fg[CHUNK], fu[CHUNK];
+#pragma unroll
+        for (int s = 0; s < CHUNK; ++s) {
+          const bool ok = wvalid && kbase + (h + s) * 32 < K;
+          fg[s] = ok ? *reinterpret_cast<const bf16x8_t*>(gp + (h + s) * 32) : zero8;
+          fu[s] = ok ? *reinterpret_cast<const bf16x8_t*>(up + (h + s) * 32) : zero8;
+        }
+#pragma unroll
+        for (int s = 0; s < CHUNK; ++s) {
+          ag = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fg[s], xa[h + s], ag, 0, 0, 0);
+          au = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fu[s], xa[h + s], au, 0, 0, 0);
+        }
       }
     }
     if (NW > 1) {
@@ -401,6 +581,8 @@ gemm_bf16_rows16_swiglu_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
     if (wave == 0) {
       const int m = lane & 15, nn = n0 + (lane >> 4) * 4;
       if (m < M) {
+        float scale = 1.f;
+        if constexpr (NORM) scale = normed_row_scale<NW>(ssw, m, K, normed.eps);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int n = nn + r;
@@ -415,6 +597,10 @@ gemm_bf16_rows16_swiglu_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
               uv += red[g & 1][1][w][lane][r];
             }
           }
+          if constexpr (NORM) {
+            gv *= scale;
+            uv *= scale;
+          }
           C[(size_t)m * I + n] = (bf16_t)(gv * (1.0f / (1.0f + expf(-gv))) * uv);
         }
       }
@@ -422,10 +608,21 @@ gemm_bf16_rows16_swiglu_kernel(const bf16_t* __restrict__ A, const bf16_t* __res
   }
 }
 
-static int launch_rows16(const bf16_t* a, const bf16_t* w, const float* bias, void* C, int c_dtype,
-                         int M, int N, int K, int ksplit, hipStream_t stream,
-                         int groups_per_block = 0) {
+// `normed` (with normed->x set) replaces the bfloat16 activations `a` by rows of the
+// 32-bit stream that the kernel normalises itself; it needs one workgroup to cover K
+// with 16 steps a wave (K <= 4096, a multiple of 512) and K not split over workgroups.
+static bool rows16_takes_norm(int K, int ksplit) {
+  return ksplit == 1 && K <= 4096 && K % 512 == 0;
+}
+
+static int launch_rows16(const bf16_t* a, const NormedRowsArg* normed, const bf16_t* w,
+                         const float* bias, void* C, int c_dtype, int M, int N, int K, int ksplit,
+                         int accumulate, hipStream_t stream, int groups_per_block = 0) {
   if (ksplit < 1 || (ksplit > 1 && (c_dtype != 0 || K % (ksplit * 32) != 0))) return ZA_ERR_ARG;
+  if (accumulate && c_dtype != 0) return ZA_ERR_ARG;
+  const bool norm = normed && normed->x;
+  if (norm && (!normed->weight || !rows16_takes_norm(K, ksplit))) return ZA_ERR_UNSUPPORTED;
+  if (!norm && !a) return ZA_ERR_ARG;
   const int kper = (K + ksplit - 1) / ksplit;   // K range of one workgroup
   if (kper > 8192) return ZA_ERR_UNSUPPORTED;
   const int groups = (N + 15) / 16;
@@ -437,15 +634,24 @@ static int launch_rows16(const bf16_t* a, const bf16_t* w, const float* bias, vo
   else if (groups >= 768) per_block = 2;
   if (groups_per_block > 0) per_block = groups_per_block;
   dim3 grid((groups + per_block - 1) / per_block, ksplit);
+  const NormedRowsArg none = {nullptr, nullptr, nullptr, 0.f};
+#define ZA_R16_LAUNCH(NW, KS, TC, NORM)                                                       \
+  hipLaunchKernelGGL((gemm_bf16_rows16_kernel<NW, KS, TC, NORM>), grid, dim3(NW * 64), 0,     \
+                     stream, a, NORM ? *normed : none, w, bias, (TC*)C, M, N, K, per_block,   \
+                     accumulate)
 #define ZA_R16_CASE(NW, KS)                                                                   \
   {                                                                                           \
-    dim3 block(NW * 64);                                                                      \
-    if (c_dtype == 0)                                                                         \
-      hipLaunchKernelGGL((gemm_bf16_rows16_kernel<NW, KS, float>), grid, block, 0,            \
-                         stream, a, w, bias, (float*)C, M, N, K, per_block);                  \
-    else                                                                                      \
-      hipLaunchKernelGGL((gemm_bf16_rows16_kernel<NW, KS, bf16_t>), grid, block, 0,           \
-                         stream, a, w, bias, (bf16_t*)C, M, N, K, per_block);                 \
+    if (norm) {                                                                               \
+      if constexpr (KS == 16) {                                                               \
+        if (c_dtype == 0) ZA_R16_LAUNCH(NW, KS, float, true);                                 \
+        else ZA_R16_LAUNCH(NW, KS, bf16_t, true);                                             \
+      } else {                                                                                \
+        return ZA_ERR_UNSUPPORTED;                                                            \
+      }                                                                                       \
+    } else {                                                                                  \
+      if (c_dtype == 0) ZA_R16_LAUNCH(NW, KS, float, false);                                  \
+      else ZA_R16_LAUNCH(NW, KS, bf16_t, false);                                              \
+    }                                                                                         \
     return za_launch_status();                                                                \
   }
   if (kper <= 512) ZA_R16_CASE(1, 16)
@@ -454,6 +660,7 @@ static int launch_rows16(const bf16_t* a, const bf16_t* w, const float* bias, vo
   if (kper <= 4096) ZA_R16_CASE(8, 16)
   ZA_R16_CASE(8, 32)
 #undef ZA_R16_CASE
+#undef ZA_R16_LAUNCH
 }
 
 // ------------------------------------------------------------------ launchers
@@ -486,7 +693,7 @@ extern "C" int za_gemm_bf16(const void* A, const void* W, const float* bias, voi
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
   if (M <= 16 && K <= 8192 && !force_tiled)
-    return launch_rows16(a, w, bias, C, c_dtype, M, N, K, 1, stream);
+    return launch_rows16(a, nullptr, w, bias, C, c_dtype, M, N, K, 1, 0, stream);
   if (M <= 64 && !force_tiled) {
     dim3 grid((N + 15) / 16), block(256);
     const int mt = (M + 15) / 16;
@@ -526,25 +733,60 @@ extern "C" int za_gemm_bf16_rows16(const void* A, const void* W, const float* bi
   if (M == 0 || N == 0) return 0;
   if (M < 0 || N < 0 || K <= 0 || !A || !W || !C) return ZA_ERR_ARG;
   if (M > 16 || K % 8 != 0 || (c_dtype != 0 && c_dtype != 1)) return ZA_ERR_UNSUPPORTED;
-  return launch_rows16((const bf16_t*)A, (const bf16_t*)W, bias, C, c_dtype, M, N, K, ksplit,
-                       stream, groups_per_block);
+  return launch_rows16((const bf16_t*)A, nullptr, (const bf16_t*)W, bias, C, c_dtype, M, N, K,
+                       ksplit, 0, stream, groups_per_block);
+}
+
+// The decode kernel between two states of the 32-bit residual stream.
+//   input:  bfloat16 activations A [M, K], or (A null) rows of the stream `x`
+//           ([*, K] 32-bit; row m of the product is row rows[m], or m without `rows`)
+//           that the kernel passes through an RMSNorm (norm_weight [K], eps) itself;
+//           that needs K <= 4096, K % 512 == 0 and ksplit == 1;
+//   output: stored to C [M, N] (c_dtype), or with `accumulate` added to the 32-bit
+//           C [M, N] with atomics, K cut into `ksplit` ranges that all add there.
+// Without `accumulate`, ksplit must be 1.
+extern "C" int za_gemm_bf16_rows16_stream(const void* A, const float* x, const int* rows,
+                                          const float* norm_weight, float eps, const void* W,
+                                          const float* bias, void* C, int c_dtype, int M, int N,
+                                          int K, int ksplit, int accumulate, hipStream_t stream) {
+  if (M == 0 || N == 0) return 0;
+  if (M < 0 || N < 0 || K <= 0 || !W || !C || (!A && !x)) return ZA_ERR_ARG;
+  if (M > 16 || K % 8 != 0 || (c_dtype != 0 && c_dtype != 1)) return ZA_ERR_UNSUPPORTED;
+  if (!accumulate && ksplit != 1) return ZA_ERR_ARG;
+  const NormedRowsArg normed = {A ? nullptr : x, rows, norm_weight, eps};
+  return launch_rows16((const bf16_t*)A, &normed, (const bf16_t*)W, bias, C, c_dtype, M, N, K,
+                       ksplit, accumulate ? 1 : 0, stream);
 }
 
 // Fused gate|up projection with the SwiGLU gate applied to the accumulators:
 // W is [2 * I, K] (gate rows, then up rows), C is bfloat16 [M, I], M <= 16, K <= 8192.
-extern "C" int za_gemm_bf16_rows16_swiglu(const void* A, const void* W, void* C, int M, int I,
-                                          int K, hipStream_t stream) {
+// The input is bfloat16 A [M, K], or (A null) rows of the 32-bit stream `x` that the
+// kernel passes through an RMSNorm itself (K <= 4096, K % 512 == 0), as
+// za_gemm_bf16_rows16_stream.
+extern "C" int za_gemm_bf16_rows16_swiglu(const void* A, const float* x, const int* rows,
+                                          const float* norm_weight, float eps, const void* W,
+                                          void* C, int M, int I, int K, hipStream_t stream) {
   if (M == 0 || I == 0) return 0;
-  if (M < 0 || I < 0 || K <= 0 || !A || !W || !C) return ZA_ERR_ARG;
+  if (M < 0 || I < 0 || K <= 0 || !W || !C || (!A && !x)) return ZA_ERR_ARG;
   if (M > 16 || K % 8 != 0 || K > 8192) return ZA_ERR_UNSUPPORTED;
+  const bool norm = !A;
+  if (norm && (!norm_weight || !rows16_takes_norm(K, 1))) return ZA_ERR_UNSUPPORTED;
+  const NormedRowsArg normed = {norm ? x : nullptr, rows, norm_weight, eps};
   const int groups = (I + 15) / 16;
   const int per_block = groups >= 2048 ? 4 : 1;
   dim3 grid((groups + per_block - 1) / per_block);
+#define ZA_SG_LAUNCH(NW, KS, NORM)                                                            \
+  hipLaunchKernelGGL((gemm_bf16_rows16_swiglu_kernel<NW, KS, NORM>), grid, dim3(NW * 64), 0,  \
+                     stream, (const bf16_t*)A, normed, (const bf16_t*)W, (bf16_t*)C, M, I, K, \
+                     per_block)
 #define ZA_SG_CASE(NW, KS)                                                                    \
   {                                                                                           \
-    hipLaunchKernelGGL((gemm_bf16_rows16_swiglu_kernel<NW, KS>), grid, dim3(NW * 64), 0,      \
-                       stream, (const bf16_t*)A, (const bf16_t*)W, (bf16_t*)C, M, I, K,       \
-                       per_block);                                                            \
+    if (norm) {                                                                               \
+      if constexpr (KS == 16) ZA_SG_LAUNCH(NW, KS, true);                                     \
+      else return ZA_ERR_UNSUPPORTED;                                                         \
+    } else {                                                                                  \
+      ZA_SG_LAUNCH(NW, KS, false);                                                            \
+    }                                                                                         \
     return za_launch_status();                                                                \
   }
   if (K <= 512) ZA_SG_CASE(1, 16)
@@ -553,4 +795,5 @@ extern "C" int za_gemm_bf16_rows16_swiglu(const void* A, const void* W, void* C,
   if (K <= 4096) ZA_SG_CASE(8, 16)
   ZA_SG_CASE(8, 32)
 #undef ZA_SG_CASE
+#undef ZA_SG_LAUNCH
 }

@@ -170,5 +170,9 @@ class DecoderModel:
         if step.n_logit_rows == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32,
                                device=self.runtime.device)
-        normed = self.final_norm.add_forward(residual, pending, rows=step.logit_rows)
+        normed = None
+        if pending is None and getattr(self.head, "takes_stream", False):
+            normed = self.final_norm.deferred(residual, rows=step.logit_rows)
+        if normed is None:
+            normed = self.final_norm.add_forward(residual, pending, rows=step.logit_rows)
         return self.head.forward(normed)

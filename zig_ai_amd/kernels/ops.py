@@ -55,8 +55,11 @@ _SIGNATURES = {
                                 c_void_p],
     ("gemm", "za_gemm_bf16_rows16"): [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                       c_int, c_int, c_int, c_void_p],
-    ("gemm", "za_gemm_bf16_rows16_swiglu"): [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                                             c_void_p],
+    ("gemm", "za_gemm_bf16_rows16_stream"): [c_void_p, c_void_p, c_void_p, c_void_p, c_float,
+                                             c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                             c_int, c_int, c_int, c_void_p],
+    ("gemm", "za_gemm_bf16_rows16_swiglu"): [c_void_p, c_void_p, c_void_p, c_void_p, c_float,
+                                             c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     ("sampling", "za_sample"): [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                 c_void_p, c_int, c_void_p],
     ("sampling", "za_repetition_penalty"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
@@ -185,6 +188,66 @@ def embed_gather(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
     return out
 
 
+class NormedRows:
+    """An RMSNorm that has not run yet: rows of the 32-bit residual stream (``rows``
+    selects and orders them; all of them without it) with the norm's weight and eps.
+    ``linear`` and ``linear_swiglu`` take it in place of activations and, for a decode
+    batch, let the projection's kernel normalise the rows on its way; everywhere else
+    ``materialise`` runs the norm kernel."""
+
+    __slots__ = ("residual", "weight", "eps", "dtype", "rows")
+
+    def __init__(self, residual: torch.Tensor, weight: torch.Tensor, eps: float,
+                 dtype: torch.dtype, rows: Optional[torch.Tensor] = None):
+        _need(residual, "residual", torch.float32)
+        if residual.dim() != 2:
+            raise KernelError(f"NormedRows takes [rows, width], got {tuple(residual.shape)}")
+        _need(weight, "weight", torch.float32, (residual.shape[1],))
+        if rows is not None:
+            _need(rows, "rows", torch.int32)
+        self.residual, self.weight, self.eps, self.dtype, self.rows = \
+            residual, weight, float(eps), dtype, rows
+
+    @property
+    def shape(self) -> Tuple[int, int]:
+        n = self.residual.shape[0] if self.rows is None else self.rows.numel()
+        return (n, self.residual.shape[1])
+
+    @property
+    def device(self) -> torch.device:
+        return self.residual.device
+
+    def materialise(self) -> torch.Tensor:
+        return add_rmsnorm(self.residual, None, self.weight, self.eps, self.dtype, rows=self.rows,
+                           write_residual=False)
+
+
+# The fused forms exist for a decode batch of bfloat16 products whose K one workgroup
+# covers in slices of 512, a wave's share.
+NORMED_ROWS_MAX_K = 4096
+NORMED_ROWS_K_MULTIPLE = 512
+NORMED_ROWS_MAX_ROWS = 16
+
+
+def normed_rows_fusable(rows: int, width: int) -> bool:
+    return rows <= NORMED_ROWS_MAX_ROWS and width <= NORMED_ROWS_MAX_K \
+        and width % NORMED_ROWS_K_MULTIPLE == 0
+
+
+def _takes_normed_rows(x, weight: torch.Tensor, M: int, K: int) -> bool:
+    """Whether the product's kernel runs the norm itself.  Every workgroup reads the rows
+    in 32-bit, which costs more the more rows there are (measured at K = 2048 against the
+    norm kernel followed by the product: 1 to 2 us saved per product up to 8 rows, about
+    even at 16), unless a workgroup walks many row groups with them (the output head:
+    5 to 7 us saved up to 16 rows)."""
+    return (isinstance(x, NormedRows) and x.dtype == torch.bfloat16
+            and weight.dtype == torch.bfloat16 and normed_rows_pay(M, weight.shape[0], K))
+
+
+def normed_rows_pay(M: int, N: int, K: int) -> bool:
+    return normed_rows_fusable(M, K) and (M <= 8 or N >= 16384)
+
+
 # --------------------------------------------------------------------- gemm
 # Above this many rows a bfloat16 projection without bias goes to the library
 # (measured: the decode kernel wins up to 16 rows, the library from there on).
@@ -265,9 +328,20 @@ def _library_matmul(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtyp
     return out
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+def _accumulate_splits(N: int, K: int) -> int:
+    """Into how many ranges K is cut when a decode batch's product is added to the
+    stream with atomics: until some 512 workgroups stream the weight."""
+    groups = (N + 15) // 16
+    for split in (8, 4, 2):
+        if groups * split <= 640 and K % (split * 32) == 0 and K // split >= 512:
+            return split
+    return 1
+
+
+def linear(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
            out_dtype: Optional[torch.dtype] = None, force_tiled: bool = False,
-           partial_ok: bool = False) -> torch.Tensor:
+           partial_ok: bool = False,
+           accumulate: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """``x [M, K] @ weight[N, K]^T + bias`` with 32-bit accumulation.
 
     bfloat16 weights use the matrix-core kernels of csrc/gemm.hip up to
@@ -279,12 +353,54 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     With ``partial_ok`` the result may come back as a stack ``[P, M, N]`` of 32-bit
     partial sums (K cut into ranges, for more workgroups, when N is small and M is
     at most ``LIBRARY_SPLIT_ROWS``); ``add_rmsnorm`` adds such a stack up while it
-    reads it."""
-    if x.dim() != 2 or weight.dim() != 2:
+    reads it.
+
+    ``x`` may be a ``NormedRows``: a decode batch is then normalised by the product's
+    own kernel.  With ``accumulate`` (the 32-bit ``[M, N]`` residual stream) a decode
+    batch's product is added to that tensor with atomics and ``None`` comes back (the
+    additions of the ranges of K arrive in the hardware's order: reproducible to
+    rounding only); otherwise the product comes back as usual and the caller adds it."""
+    if len(x.shape) != 2 or weight.dim() != 2:
         raise KernelError(f"linear takes x [M, K] and weight [N, K], got {tuple(x.shape)} and "
                           f"{tuple(weight.shape)}")
     M, K = x.shape
     N = weight.shape[0]
+    normed = None
+    if isinstance(x, NormedRows):
+        if _takes_normed_rows(x, weight, M, K) and not force_tiled:
+            normed = x
+        else:
+            x = x.materialise()
+    if accumulate is not None and not (
+            M <= 16 and weight.dtype == torch.bfloat16 and K % 8 == 0 and not force_tiled
+            and (normed is not None or x.dtype == torch.bfloat16)):
+        accumulate = None
+    if normed is not None or accumulate is not None:
+        _need(weight, "weight", torch.bfloat16, (N, K))
+        if bias is not None:
+            _need(bias, "bias", torch.float32, (N,))
+        if normed is None:
+            _need(x, "x", torch.bfloat16)
+        splits = 1
+        if accumulate is not None:
+            _need(accumulate, "accumulate", torch.float32, (M, N))
+            out, out_code = accumulate, 0
+            if normed is None:
+                splits = _accumulate_splits(N, K)
+        else:
+            out_dtype = out_dtype or normed.dtype
+            out = torch.empty((M, N), dtype=out_dtype, device=weight.device)
+            out_code = _code(out_dtype)
+        rc = _fn("gemm", "za_gemm_bf16_rows16_stream")(
+            None if normed is not None else _ptr(x),
+            _ptr(normed.residual) if normed is not None else None,
+            _ptr(normed.rows) if normed is not None else None,
+            _ptr(normed.weight) if normed is not None else None,
+            normed.eps if normed is not None else 0.0,
+            _ptr(weight), _ptr(bias), _ptr(out), out_code, M, N, K, splits,
+            1 if accumulate is not None else 0, _stream())
+        _check(rc, "gemm_bf16_rows16_stream", f"M={M} N={N} K={K} splits={splits}")
+        return None if accumulate is not None else out
     _need(x, "x", (torch.float32, torch.bfloat16))
     _need(weight, "weight", (torch.float32, torch.bfloat16), (N, K))
     if bias is not None:
@@ -326,24 +442,36 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     return out
 
 
-def linear_swiglu(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor:
+def linear_swiglu(x, gate_up_weight: torch.Tensor) -> torch.Tensor:
     """``silu(x Wg^T) * (x Wu^T)`` for ``gate_up_weight = [Wg; Wu]`` of shape ``[2I, K]``
-    and at most 16 rows of bfloat16 ``x``: the gate is applied to the 32-bit
-    accumulators, the ``[M, 2I]`` intermediate is never stored."""
-    if x.dim() != 2 or gate_up_weight.dim() != 2 or gate_up_weight.shape[0] % 2 \
+    and at most 16 rows of bfloat16 ``x`` (or a ``NormedRows``): the gate is applied to
+    the 32-bit accumulators, the ``[M, 2I]`` intermediate is never stored."""
+    if len(x.shape) != 2 or gate_up_weight.dim() != 2 or gate_up_weight.shape[0] % 2 \
             or gate_up_weight.shape[1] != x.shape[1]:
         raise KernelError(f"linear_swiglu takes x [M, K] and a weight [2I, K], got "
                           f"{tuple(x.shape)} and {tuple(gate_up_weight.shape)}")
     M, K = x.shape
     I = gate_up_weight.shape[0] // 2
-    _need(x, "x", torch.bfloat16)
     _need(gate_up_weight, "gate_up_weight", torch.bfloat16)
+    normed = None
+    if isinstance(x, NormedRows):
+        if _takes_normed_rows(x, gate_up_weight, M, K):
+            normed = x
+        else:
+            x = x.materialise()
+    if normed is None:
+        _need(x, "x", torch.bfloat16)
     if M > 16 or K % 8 or K > 8192:
         raise KernelError(f"linear_swiglu takes at most 16 rows and K <= 8192 in multiples of "
                           f"8, got M={M} K={K}")
-    out = torch.empty((M, I), dtype=torch.bfloat16, device=x.device)
-    rc = _fn("gemm", "za_gemm_bf16_rows16_swiglu")(_ptr(x), _ptr(gate_up_weight), _ptr(out), M, I,
-                                                   K, _stream())
+    out = torch.empty((M, I), dtype=torch.bfloat16, device=gate_up_weight.device)
+    rc = _fn("gemm", "za_gemm_bf16_rows16_swiglu")(
+        None if normed is not None else _ptr(x),
+        _ptr(normed.residual) if normed is not None else None,
+        _ptr(normed.rows) if normed is not None else None,
+        _ptr(normed.weight) if normed is not None else None,
+        normed.eps if normed is not None else 0.0,
+        _ptr(gate_up_weight), _ptr(out), M, I, K, _stream())
     _check(rc, "linear_swiglu", f"M={M} I={I} K={K}")
     return out
 

@@ -17,7 +17,7 @@ None).
 from __future__ import annotations
 
 import math
-from typing import Any, Dict, Mapping
+from typing import Any, Dict, Mapping, Optional
 
 import torch
 
@@ -56,6 +56,7 @@ def plan_split(n_items: int, num_kv_heads: int, max_keys: int, target: int = SPL
 class GroupedQueryAttention(Mixer):
     kind = "gqa_attention"
     graph_safe = True
+    takes_stream = True
     kernel_sources = ("gemm", "rope_kv", "attention", "norm")
 
     @classmethod
@@ -126,7 +127,7 @@ class GroupedQueryAttention(Mixer):
         ops.check_projection_weight(self.w_qkv, "attention w_qkv")
         ops.check_projection_weight(self.w_out, "attention w_out")
 
-    def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
+    def forward(self, x, step, cache, stream: Optional[torch.Tensor] = None):
         nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
         T = x.shape[0]
         qkv = ops.linear(x, self.w_qkv, self.b_qkv)
@@ -177,7 +178,8 @@ class GroupedQueryAttention(Mixer):
             o = ops.paged_attention(q, cache.kv, step.block_tables[cache.group], step.positions,
                                     item_seq, item_row0, item_count, n_items, self.scale,
                                     self.window, keys, nsplit)
-        return ops.linear(o.view(T, nh * d), self.w_out, self.b_out, partial_ok=True)
+        return ops.linear(o.view(T, nh * d), self.w_out, self.b_out, partial_ok=True,
+                          accumulate=stream)
 
 
 register_mixer(GroupedQueryAttention.kind, GroupedQueryAttention)

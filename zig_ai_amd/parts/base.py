@@ -92,6 +92,13 @@ class Part:
 
 
 class Mixer(Part):
+    # A part that sets ``takes_stream`` accepts, in place of the activations ``x``, what
+    # ``Norm.deferred`` returned (a norm that has not run yet, which the kernels of
+    # ``ops.linear`` / ``ops.linear_swiglu`` can run themselves), and a keyword
+    # ``stream``: the 32-bit residual stream, to which it may add its result itself;
+    # it then returns ``None``.
+    takes_stream = False
+
     @classmethod
     def cache_need(cls, params: Mapping[str, Any]):
         """``PagedNeed``, ``StateNeed`` or ``None``."""
@@ -102,6 +109,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    takes_stream = False      # as for Mixer
+
     def forward(self, x: torch.Tensor, step) -> torch.Tensor:
         raise NotImplementedError
 
@@ -127,6 +136,13 @@ class Norm(Part):
         if delta is not None:
             residual.add_(delta.float())
         return self.forward(residual)
+
+
+    def deferred(self, residual: torch.Tensor, rows: Optional[torch.Tensor] = None):
+        """The norm of ``residual`` (of its ``rows``) as something a part with
+        ``takes_stream`` accepts in place of activations, without running it now; or
+        ``None`` when this norm, or this step, has no such form."""
+        return None
 
 
 class PositionEncoding(Part):

@@ -8,7 +8,9 @@
 The residual stream is kept in 32-bit.  A block receives the stream and a
 ``pending`` tensor that has not been added to it yet, and returns the same
 pair: every add is then fused with the norm that follows it, including across
-the boundary between two blocks.
+the boundary between two blocks.  Where a part says so (``takes_stream``) the norm
+before it is handed over without having run (``Norm.deferred``) and the part may add
+its result to the stream itself; nothing is pending after it then.
 """
 
 from __future__ import annotations
@@ -30,12 +32,21 @@ class PreNormResidualBlock:
         self.feed_forward = feed_forward
 
     def forward(self, residual: torch.Tensor, pending: Optional[torch.Tensor], step,
-                cache) -> Tuple[torch.Tensor, torch.Tensor]:
-        n1 = self.mixer_norm.add_forward(residual, pending)
-        m = self.mixer.forward(n1, step, cache)
-        n2 = self.feed_forward_norm.add_forward(residual, m)
-        f = self.feed_forward.forward(n2, step)
+                cache) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+        m = apply_normed(self.mixer_norm, self.mixer, residual, pending, step, cache)
+        f = apply_normed(self.feed_forward_norm, self.feed_forward, residual, m, step)
         return residual, f
+
+
+def apply_normed(norm, part, residual: torch.Tensor, pending: Optional[torch.Tensor], *args):
+    """``part(norm(residual + pending))``: what is still to be added to the stream
+    afterwards, or ``None`` when the part has added it already."""
+    if not getattr(part, "takes_stream", False):
+        return part.forward(norm.add_forward(residual, pending), *args)
+    x = norm.deferred(residual) if pending is None else None
+    if x is None:
+        x = norm.add_forward(residual, pending)
+    return part.forward(x, *args, stream=residual)
 
 
 register_arrangement(PreNormResidualBlock.kind, PreNormResidualBlock)

@@ -36,6 +36,7 @@ class TokenEmbedding(Part):
 class LinearHead(Part):
     kind = "linear_head"
     graph_safe = True
+    takes_stream = True       # ``forward`` accepts a norm that has not run yet
     kernel_sources = ("gemm",)
 
     @classmethod
@@ -50,7 +51,7 @@ class LinearHead(Part):
         self.tied = bool(params.get("tied"))
         self.weight = tensors.get("weight")   # the model hands a tied head the embedding table
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    def forward(self, x) -> torch.Tensor:
         ops.check_projection_weight(self.weight, "output head")
         return ops.linear(x, self.weight, out_dtype=torch.float32)
 

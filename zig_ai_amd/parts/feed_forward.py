@@ -5,7 +5,7 @@ a stack of partial sums (see ``Norm.add_forward``)."""
 
 from __future__ import annotations
 
-from typing import Any, Dict, Mapping
+from typing import Any, Dict, Mapping, Optional
 
 import torch
 
@@ -24,6 +24,7 @@ def fuse_rows(*mats: torch.Tensor) -> torch.Tensor:
 class SwiGLU(FeedForward):
     kind = "swiglu"
     graph_safe = True
+    takes_stream = True
     kernel_sources = ("gemm", "activation")
 
     @classmethod
@@ -39,14 +40,16 @@ class SwiGLU(FeedForward):
         ops.check_projection_weight(self.gate_up, "feed_forward gate_up")
         ops.check_projection_weight(self.down, "feed_forward down")
 
-    def forward(self, x: torch.Tensor, step=None) -> torch.Tensor:
+    def forward(self, x, step=None, stream: Optional[torch.Tensor] = None):
         if x.shape[0] <= 16 and x.dtype == torch.bfloat16 and self.gate_up.dtype == torch.bfloat16 \
                 and x.shape[1] <= 8192:
             # a decode batch: the gate is applied to the projection's accumulators
             a = ops.linear_swiglu(x, self.gate_up)
         else:
+            if isinstance(x, ops.NormedRows):
+                x = x.materialise()
             a = ops.swiglu(ops.linear(x, self.gate_up))
-        return ops.linear(a, self.down, partial_ok=True)
+        return ops.linear(a, self.down, partial_ok=True, accumulate=stream)
 
 
 register_feed_forward(SwiGLU.kind, SwiGLU)

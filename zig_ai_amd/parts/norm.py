@@ -41,5 +41,12 @@ class RMSNorm(Norm):
                     rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         return ops.add_rmsnorm(residual, delta, self.weight, self.eps, self.runtime.dtype, rows=rows)
 
+    def deferred(self, residual: torch.Tensor, rows: Optional[torch.Tensor] = None):
+        # a decode batch in bfloat16: the projection that follows normalises the rows
+        n = residual.shape[0] if rows is None else rows.numel()
+        if self.runtime.dtype != torch.bfloat16 or not ops.normed_rows_fusable(n, self.width):
+            return None
+        return ops.NormedRows(residual, self.weight, self.eps, self.runtime.dtype, rows)
+
 
 register_norm(RMSNorm.kind, RMSNorm)

@@ -13,7 +13,7 @@ the model's definition, which the reference's layer does not follow
 
 from __future__ import annotations
 
-from typing import Any, Dict, Mapping
+from typing import Any, Dict, Mapping, Optional
 
 import torch
 
@@ -24,6 +24,7 @@ from .base import Mixer, Runtime, StateNeed, TensorRule, register_mixer
 class ShortConv(Mixer):
     kind = "short_conv"
     graph_safe = True
+    takes_stream = True
     kernel_sources = ("gemm", "shortconv")
 
     @classmethod
@@ -60,11 +61,11 @@ class ShortConv(Mixer):
         ops.check_projection_weight(self.w_in, "short_conv w_in")
         ops.check_projection_weight(self.w_out, "short_conv w_out")
 
-    def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
+    def forward(self, x, step, cache, stream: Optional[torch.Tensor] = None):
         z = ops.linear(x, self.w_in, self.b_in)
         y = ops.short_conv(z, self.w_conv, self.b_conv, cache.state, step.token_seq,
                            step.seq_start, step.slot_id)
-        return ops.linear(y, self.w_out, self.b_out, partial_ok=True)
+        return ops.linear(y, self.w_out, self.b_out, partial_ok=True, accumulate=stream)
 
 
 register_mixer(ShortConv.kind, ShortConv)
