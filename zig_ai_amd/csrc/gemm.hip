@@ -296,9 +296,10 @@ struct NormedRowsArg {
 // the slice of row r in ssw[wave][r]; `nws` is room for the norm weight of the
 // workgroup's K range.  Ends with a barrier.  K is a multiple of a wave's slice
 // (KSTEPS * 32 elements), so a wave is either all inside K or has nothing to do.  A lane
-// without a row reads row 0 with its neighbours and turns what it read into zeros:
-// straight-line loads from one address with the steps as constant offsets, all in
-// flight together.  `prefetch` is called once the rows are requested, by the waves
+// without a row reads row 0 with its neighbours (row m of the product depends on row m
+// of the operand alone, and rows from M on are never stored): straight-line loads from
+// one address with the steps as constant offsets, all in flight together, and no
+// arithmetic beyond what a row needs (every workgroup repeats it).  `prefetch` is called once the rows are requested, by the waves
 // inside K only.
 template <int NW, int KSTEPS, typename Prefetch>
 __device__ __forceinline__ void load_normed_rows(bf16x8_t (&xa)[KSTEPS],
@@ -343,8 +344,7 @@ __device__ __forceinline__ void load_normed_rows(bf16x8_t (&xa)[KSTEPS],
       bf16x8_t r;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const float a = rvalid ? xf[s][0][e] : 0.f;
-        const float b = rvalid ? xf[s][1][e] : 0.f;
+        const float a = xf[s][0][e], b = xf[s][1][e];
         ss += a * a;
         ss += b * b;
         r[e] = (bf16_t)(a * w0[e]);
