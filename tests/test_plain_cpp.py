@@ -217,6 +217,33 @@ def test_kernel_linear_against_twin(dtype, M, N, K, bias):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K,bias", [(1, 50, 512, False), (8, 130, 1536, True), (5, 70, 2048, False),
+                                        (16, 16400, 1024, False)])
+def test_kernel_decode_forms_against_twins(M, N, K, bias):
+    """A decode batch in bfloat16: the projection that runs the norm before it against
+    the norm's twin followed by the product's twin (the twin rounds nothing, the kernel
+    rounds the operands once), also into the SwiGLU gate; and the projection that adds
+    to the stream against the product's twin plus the stream."""
+    o = ops()
+    res, nw = rand((M, K), 70, 2.0), 1.0 + rand((K,), 71, 0.3)
+    w = rand((N, K), 72, 0.05).to(torch.bfloat16)
+    b = rand((N,), 73) if bias else None
+    _, normed = twin.add_rmsnorm(res, None, nw, 1e-5)
+    want = twin.linear(normed, w.float(), b)
+    x = o.NormedRows(res.to(dev()), nw.to(dev()), 1e-5, torch.bfloat16)
+    assert o.normed_rows_pay(M, N, K)
+    got = o.linear(x, w.to(dev()), b.to(dev()) if bias else None, out_dtype=torch.float32)
+    assert rel_err(got, want) < BF16_TOL
+    if N % 2 == 0 and not bias:
+        assert rel_err(o.linear_swiglu(x, w.to(dev())), twin.swiglu(want)) < BF16_TOL
+    a = rand((M, K), 74).to(torch.bfloat16)
+    stream = rand((M, N), 75)
+    on_device = stream.clone().to(dev())
+    assert o.linear(a.to(dev()), w.to(dev()), b.to(dev()) if bias else None, accumulate=on_device) is None
+    assert rel_err(on_device, stream + twin.linear(a.float(), w.float(), b)) < F32_TOL
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_kernel_embed_against_twin(dtype):
     table = rand((300, 72), 57).to(dtype)

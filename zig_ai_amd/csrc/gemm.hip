@@ -299,8 +299,8 @@ struct NormedRowsArg {
 // without a row reads row 0 with its neighbours (row m of the product depends on row m
 // of the operand alone, and rows from M on are never stored): straight-line loads from
 // one address with the steps as constant offsets, all in flight together, and no
-// arithmetic beyond what a row needs (every workgroup repeats it).  `prefetch` is called once the rows are requested, by the waves
-// inside K only.
+// arithmetic beyond what a row needs (every workgroup repeats it).  `prefetch` is
+// called once the rows are requested, by the waves inside K only.
 template <int NW, int KSTEPS, typename Prefetch>
 __device__ __forceinline__ void load_normed_rows(bf16x8_t (&xa)[KSTEPS],
                                                  const float* __restrict__ x,
