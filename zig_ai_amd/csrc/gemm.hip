@@ -632,6 +632,9 @@ static int launch_rows16(const bf16_t* a, const NormedRowsArg* normed, const bf1
   int per_block = 1;
   if (groups >= 2048) per_block = 8;
   else if (groups >= 768) per_block = 2;
+  // with the norm in the kernel every workgroup prepares the step's rows first: two row
+  // groups share that from 384 groups on (8 rows: in_proj 10.7 -> 9.1 us)
+  if (norm && per_block == 1 && groups >= 384) per_block = 2;
   if (groups_per_block > 0) per_block = groups_per_block;
   dim3 grid((groups + per_block - 1) / per_block, ksplit);
   const NormedRowsArg none = {nullptr, nullptr, nullptr, 0.f};
@@ -773,7 +776,9 @@ extern "C" int za_gemm_bf16_rows16_swiglu(const void* A, const float* x, const i
   if (norm && (!norm_weight || !rows16_takes_norm(K, 1))) return ZA_ERR_UNSUPPORTED;
   const NormedRowsArg normed = {norm ? x : nullptr, rows, norm_weight, eps};
   const int groups = (I + 15) / 16;
-  const int per_block = groups >= 2048 ? 4 : 1;
+  // (with the norm in the kernel two row groups share the preparation of the step's rows:
+  // 8 rows, I = 8192: 18.1 -> 16.9 us)
+  const int per_block = groups >= 2048 ? 4 : (norm && groups >= 384 ? 2 : 1);
   dim3 grid((groups + per_block - 1) / per_block);
 #define ZA_SG_LAUNCH(NW, KS, NORM)                                                            \
   hipLaunchKernelGGL((gemm_bf16_rows16_swiglu_kernel<NW, KS, NORM>), grid, dim3(NW * 64), 0,  \
