@@ -89,3 +89,20 @@ def test_block_with_parts_that_add_to_the_stream_leaves_nothing_pending():
         total = out if pending is None else out + pending
         assert (pending is None) == adds
         assert torch.equal(total, torch.full((2, 3), 13.0))
+
+
+def test_a_runtime_that_forbids_additions_to_the_stream_hands_no_stream_over():
+    from zig_ai_amd.parts import Runtime
+
+    class Recording(StreamPart):
+        def forward(self, x, *args, stream=None):
+            self.stream = stream
+            return super().forward(x, *args, stream=torch.zeros(2, 3) if stream is None else stream)
+
+    for allowed in (True, False):
+        part = Recording(adds=False)
+        part.runtime = Runtime(device=torch.device("cpu"), dtype=torch.float32,
+                               stream_additions=allowed)
+        residual = torch.ones(2, 3)
+        apply_normed(Norm(True), part, residual, None, "step")
+        assert (part.stream is residual) == allowed

@@ -255,6 +255,37 @@ def test_real_layer_sizes(dtype):
     check(got, expect, dtype, "portions beside single tokens")
 
 
+def test_reproducible_decoding_at_real_layer_sizes():
+    """With ``reproducible`` two runs of the same steps give the same bits in bfloat16
+    (no atomic additions to the stream: the norms add the stacks of partial sums up in
+    their order); without it they agree within the tolerance, and both agree with the
+    plain implementation."""
+    from zig_ai_amd.engine import DecoderModel, ModelRunner, StepEntry
+    folder = eu.model_folder(REAL_2L, 7, torch.bfloat16, std=0.02, norm_init="around_one",
+                             role_std={"norm": 0.2, "filter": 0.5, "q_proj.weight": 0.05,
+                                       "k_proj.weight": 0.05})
+    prompts = [eu.random_tokens(n, 65536, 950 + n) for n in (24, 9, 17)]
+    oracle = plain.PlainLfm2(folder)
+    expect = [oracle.logits(p) for p in prompts]
+
+    def run(reproducible):
+        model = DecoderModel.from_folder(folder, "bfloat16", reproducible=reproducible)
+        assert model.runtime.stream_additions == (not reproducible)
+        runner = ModelRunner(model, page_size=16, num_pages=12, num_slots=3)
+        # the first tokens as one portion each, the rest as decode steps of three requests
+        schedule = [([(0, 0, 5), (1, 0, 5), (2, 0, 5)], [])]
+        for t in range(5, 24):
+            live = [(r, t, t + 1) for r, n in enumerate((24, 9, 17)) if t < n]
+            schedule.append((live, [r for r, n in enumerate((24, 9, 17)) if t == n - 1]))
+        return eu.run_schedule(runner, prompts, schedule)
+
+    first, second = run(True), run(True)
+    for a, b in zip(first, second):
+        assert torch.equal(a, b)
+    check(first, expect, "bfloat16", "reproducible")
+    check(run(False), expect, "bfloat16", "with additions to the stream")
+
+
 def test_graph_replays_with_library_products():
     """Decode batches beyond 16 rows send their projections to the GEMM library (K in
     ranges as a batched product where N is small, 32-bit logits): such steps are

@@ -55,6 +55,10 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--max-model-len", type=int, default=None,
                     help="longest prompt + generation (default: the model's, at most 8192)")
     ap.add_argument("--eos", type=int, default=None, help="stop token id (default: the config's)")
+    ap.add_argument("--reproducible", action="store_true",
+                    help="every sum in a fixed order: bitwise the same logits run after run "
+                         "(bfloat16 decoding otherwise adds to the residual stream with atomics, "
+                         "which is faster and reproducible to rounding only)")
     ap.add_argument("--no-graph", action="store_true",
                     help="launch decode steps kernel by kernel instead of replaying HIP graphs "
                          "(the reference's NOGRAPH)")
@@ -163,7 +167,7 @@ def run(args) -> int:
     engine = Engine(args.model, dtype=args.dtype, page_size=args.page_size,
                     num_pages=args.num_pages, max_num_seqs=args.max_num_seqs,
                     max_num_batched_tokens=args.batch_size, chunk_size=args.ubatch_size,
-                    max_model_len=args.max_model_len, use_graphs=not args.no_graph,
+                    max_model_len=args.max_model_len, use_graphs=not args.no_graph, reproducible=args.reproducible,
                     on_step=on_step if (args.dump_logits or args.verbose or args.profile) else None)
     load_s = time.perf_counter() - load_start
     start = time.perf_counter()

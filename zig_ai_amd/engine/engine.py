@@ -27,7 +27,8 @@ class Engine:
                  num_pages: Optional[int] = None, max_num_seqs: int = 64,
                  max_num_batched_tokens: int = 2048, chunk_size: int = 512,
                  max_model_len: Optional[int] = None, use_graphs: bool = True,
-                 on_step=None, memory_fraction: float = 0.85, multi_step: int = 8):
+                 on_step=None, memory_fraction: float = 0.85, multi_step: int = 8,
+                 reproducible: bool = False):
         """``num_pages``: pages per cache group; by default enough for
         ``max_num_seqs`` requests of ``max_model_len`` tokens (the model's
         ``max_position_embeddings`` if not given, capped at 8192), but no more than
@@ -42,8 +43,13 @@ class Engine:
         ``on_step(info)``, if given, is called after every step with a dict:
         ``step``, ``plan`` (the scheduled entries), ``logits`` (32-bit, one row per
         entry that samples, on the device), ``tokens`` (what was drawn from them),
-        ``seconds``."""
-        self.model = DecoderModel.from_folder(model_dir, dtype)
+        ``seconds``.
+        ``reproducible``: in bfloat16 the projections of a decode batch add to the residual
+        stream with atomics, several ranges of K to one element in the hardware's order,
+        so two runs agree to 32-bit rounding of the stream only; ``True`` keeps every sum
+        in a fixed order (some 10 % slower decoding), and the same requests scheduled the
+        same way then give the same bits."""
+        self.model = DecoderModel.from_folder(model_dir, dtype, reproducible=reproducible)
         limit = max_model_len or self.model.spec.max_position or 8192
         if max_model_len is None:
             limit = min(limit, 8192)

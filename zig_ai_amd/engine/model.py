@@ -107,11 +107,13 @@ class DecoderModel:
 
     # ------------------------------------------------------------- construction
     @classmethod
-    def from_folder(cls, model_dir: str, dtype="bfloat16", device: Optional[torch.device] = None):
+    def from_folder(cls, model_dir: str, dtype="bfloat16", device: Optional[torch.device] = None,
+                    reproducible: bool = False):
+        """``reproducible``: every sum in a fixed order (see ``Runtime.stream_additions``)."""
         device = device or require_gpu()
         config = load_config(model_dir)
         spec = config.to_spec()
-        rt = parts.Runtime(device=device, dtype=run_dtype(dtype))
+        rt = parts.Runtime(device=device, dtype=run_dtype(dtype), stream_additions=not reproducible)
         tensors = load_tensors(model_dir, spec, rt.dtype, device)
         model = cls(spec, tensors, rt)
         model.config = config

@@ -72,6 +72,11 @@ class Runtime:
 
     device: torch.device
     dtype: torch.dtype
+    # Whether parts may add their result to the residual stream themselves.  Several
+    # ranges of K then add to one element with atomics, in the hardware's order: faster,
+    # and reproducible to 32-bit rounding only.  False keeps every sum in a fixed order
+    # (bitwise the same result for the same step, run after run).
+    stream_additions: bool = True
 
 
 class Part:

@@ -46,7 +46,9 @@ def apply_normed(norm, part, residual: torch.Tensor, pending: Optional[torch.Ten
     x = norm.deferred(residual) if pending is None else None
     if x is None:
         x = norm.add_forward(residual, pending)
-    return part.forward(x, *args, stream=residual)
+    runtime = getattr(part, "runtime", None)
+    adds = runtime is None or getattr(runtime, "stream_additions", True)
+    return part.forward(x, *args, stream=residual if adds else None)
 
 
 register_arrangement(PreNormResidualBlock.kind, PreNormResidualBlock)
