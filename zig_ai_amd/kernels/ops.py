@@ -237,9 +237,9 @@ def normed_rows_fusable(rows: int, width: int) -> bool:
 def _takes_normed_rows(x, weight: torch.Tensor, M: int, K: int) -> bool:
     """Whether the product's kernel runs the norm itself.  Every workgroup reads the rows
     in 32-bit, which costs more the more rows there are (measured at K = 2048 against the
-    norm kernel followed by the product: 1 to 2 us saved per product up to 8 rows, about
-    even at 16), unless a workgroup walks many row groups with them (the output head:
-    5 to 7 us saved up to 16 rows)."""
+    norm kernel followed by the product: 2 to 2.6 us saved per product up to 8 rows, even
+    at 16), unless a workgroup walks many row groups with them (the gate|up projection:
+    2.7 us saved at 16 rows; the output head: 5 to 7 us)."""
     return (isinstance(x, NormedRows) and x.dtype == torch.bfloat16
             and weight.dtype == torch.bfloat16 and normed_rows_pay(M, weight.shape[0], K))
 
