@@ -10,12 +10,15 @@
 // No device code here.  What a call costs on the host matters for steps of a few
 // hundred tokens, which issue some sixty of these products: the descriptors and the
 // algorithm the library's heuristic names for a shape are made once per (device,
-// M, N, K, output type, P) and kept, so a later call is one hipblasLtMatmul.
+// M, N, K, output type, P) and kept, so a later call is one hipblasLtMatmul, or, for
+// operands seen before, one launch of a prepared instance (see InstanceKey).
 // The same shape therefore always runs the same kernel, recorded in a graph or not.
 #include <hip/hip_runtime.h>
+#include <hipblaslt/hipblaslt-ext.hpp>
 #include <hipblaslt/hipblaslt.h>
 
 #include <map>
+#include <memory>
 #include <mutex>
 #include <string>
 #include <tuple>
@@ -36,9 +39,22 @@ struct Plan {
 
 using Key = std::tuple<int, int, int, int, int, int>;   // device, M, N, K, output type, P
 
+// A product on given operands, with its kernel arguments made: issuing it again is one
+// launch (some 6 us less on the host than hipblasLtMatmul, which derives the arguments
+// at every call; making an instance costs some 12 us more than one such call).  Steps of
+// the same shape get the same addresses from the tensor library's allocator, so the
+// products of a loop over equal steps (portions of a long prompt, decode batches that
+// are not replayed from a graph) are found again.  An instance is made when a shape and
+// its operands are seen for the second time (an entry without one marks the first); a
+// table that has grown to kMaxInstances is emptied.
+using InstanceKey = std::tuple<Key, const void*, const void*, void*, void*>;   // shape, x, w, y, workspace
+constexpr size_t kMaxInstances = 8192;
+
 std::mutex g_lock;
 std::map<int, hipblasLtHandle_t> g_handles;
 std::map<Key, Plan> g_plans;
+std::map<InstanceKey, std::unique_ptr<hipblaslt_ext::Gemm>> g_instances;
+const float kOne = 1.0f, kZero = 0.0f;
 thread_local std::string g_error;
 
 int fail(int code, const std::string& what) {
@@ -142,11 +158,30 @@ ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int
   }
   if (!plan.usable || plan.workspace > workspace_bytes)
     return fail(ZA_ERR_UNSUPPORTED, "za_lt_matmul: the library names no algorithm for this shape");
-  const float one = 1.0f, zero = 0.0f;
-  const hipblasStatus_t s = hipblasLtMatmul(handle, plan.op, &one, w, plan.a, x, plan.b, &zero, y, plan.c,
-                                            y, plan.c, &plan.algo, workspace, workspace_bytes, stream);
+  hipblaslt_ext::Gemm* instance = nullptr;
+  {
+    std::lock_guard<std::mutex> guard(g_lock);
+    const InstanceKey ikey(Key(device, M, N, K, out_f32, P), x, w, y, workspace);
+    auto it = g_instances.find(ikey);
+    if (it == g_instances.end()) {
+      if (g_instances.size() >= kMaxInstances) g_instances.clear();
+      g_instances.emplace(ikey, nullptr);          // seen once
+    } else {
+      if (!it->second) {
+        std::unique_ptr<hipblaslt_ext::Gemm> made(new hipblaslt_ext::Gemm(
+            handle, plan.op, &kOne, w, plan.a, x, plan.b, &kZero, y, plan.c, y, plan.c));
+        hipblasLtMatmulAlgo_t algo = plan.algo;
+        if (made->initialize(algo, workspace) == HIPBLAS_STATUS_SUCCESS) it->second = std::move(made);
+      }
+      instance = it->second.get();                 // null: the plain call below
+    }
+  }
+  const hipblasStatus_t s =
+      instance ? instance->run(stream)
+               : hipblasLtMatmul(handle, plan.op, &kOne, w, plan.a, x, plan.b, &kZero, y, plan.c, y,
+                                 plan.c, &plan.algo, workspace, workspace_bytes, stream);
   if (s != HIPBLAS_STATUS_SUCCESS)
     return fail((int)s > 0 ? (int)s : ZA_ERR_ARG,
-                "hipblasLtMatmul failed with hipBLAS status " + std::to_string((int)s));
+                "the library's product failed with hipBLAS status " + std::to_string((int)s));
   return 0;
 }
