@@ -257,6 +257,36 @@ def test_library_product_again_on_the_same_operands():
         assert rel_err(o.linear(x, w, out_dtype=torch.float32), -2 * expect) < F32_TOL
 
 
+def test_library_products_when_the_table_of_instances_is_full():
+    """With room for four prepared instances and twelve shapes called in turn, the table
+    is emptied again and again (after the device has finished): every result is right."""
+    import os
+    import subprocess
+    import sys
+    code = (
+        "import torch\n"
+        "from zig_ai_amd.kernels import ops\n"
+        "dev = torch.device('cuda', 0)\n"
+        "g = torch.Generator().manual_seed(3)\n"
+        "w = torch.randn(64, 256, generator=g).to(torch.bfloat16)\n"
+        "xs = [torch.randn(17 + i, 256, generator=g).to(torch.bfloat16) for i in range(12)]\n"
+        "wd, xd = w.to(dev), [x.to(dev) for x in xs]\n"
+        "worst = 0.0\n"
+        "for turn in range(6):\n"
+        "    for x, xg in zip(xs, xd):\n"
+        "        y = ops.linear(xg, wd, out_dtype=torch.float32).double().cpu()\n"
+        "        e = x.double() @ w.double().T\n"
+        "        worst = max(worst, float((y - e).abs().max() / e.abs().max()))\n"
+        "print('worst', worst)\n")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for limit in ("4", "0"):
+        env = dict(os.environ, ZIG_AI_GEMM_INSTANCES=limit, PYTHONPATH=root)
+        out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True,
+                             timeout=300)
+        assert out.returncode == 0, out.stderr[-2000:]
+        assert float(out.stdout.split()[-1]) < F32_TOL, out.stdout
+
+
 def _normed_operands(x: torch.Tensor, weight: torch.Tensor, eps: float):
     """What the decode kernels make of a norm handed to them: the operands
     bf16(x * weight) and the row's scale, which multiplies the 32-bit sums."""

@@ -17,6 +17,7 @@
 #include <hipblaslt/hipblaslt-ext.hpp>
 #include <hipblaslt/hipblaslt.h>
 
+#include <cstdlib>
 #include <map>
 #include <memory>
 #include <mutex>
@@ -46,9 +47,17 @@ using Key = std::tuple<int, int, int, int, int, int>;   // device, M, N, K, outp
 // products of a loop over equal steps (portions of a long prompt, decode batches that
 // are not replayed from a graph) are found again.  An instance is made when a shape and
 // its operands are seen for the second time (an entry without one marks the first); a
-// table that has grown to kMaxInstances is emptied.
+// table that has grown to max_instances() is emptied, after the device has finished what
+// was issued.
 using InstanceKey = std::tuple<Key, const void*, const void*, void*, void*>;   // shape, x, w, y, workspace
-constexpr size_t kMaxInstances = 8192;
+// (ZIG_AI_GEMM_INSTANCES overrides the size of the table; 0 switches the instances off)
+size_t max_instances() {
+  static const size_t limit = [] {
+    const char* v = std::getenv("ZIG_AI_GEMM_INSTANCES");
+    return v ? (size_t)std::strtoul(v, nullptr, 10) : (size_t)8192;
+  }();
+  return limit;
+}
 
 std::mutex g_lock;
 std::map<int, hipblasLtHandle_t> g_handles;
@@ -164,8 +173,16 @@ ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int
     const InstanceKey ikey(Key(device, M, N, K, out_f32, P), x, w, y, workspace);
     auto it = g_instances.find(ikey);
     if (it == g_instances.end()) {
-      if (g_instances.size() >= kMaxInstances) g_instances.clear();
-      g_instances.emplace(ikey, nullptr);          // seen once
+      if (g_instances.size() >= max_instances()) {
+        // Instances may own memory that products already issued still read: the table is
+        // emptied only once the device has finished them, and never while a stream is
+        // being recorded (then it simply stays full until the next call outside).
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &capturing) == hipSuccess &&
+            capturing == hipStreamCaptureStatusNone && hipDeviceSynchronize() == hipSuccess)
+          g_instances.clear();
+      }
+      if (g_instances.size() < max_instances()) g_instances.emplace(ikey, nullptr);   // seen once
     } else {
       if (!it->second) {
         std::unique_ptr<hipblaslt_ext::Gemm> made(new hipblaslt_ext::Gemm(
