@@ -286,6 +286,47 @@ def test_reproducible_decoding_at_real_layer_sizes():
     check(run(False), expect, "bfloat16", "with additions to the stream")
 
 
+def test_a_decode_step_at_real_layer_sizes_runs_no_norm_kernel(monkeypatch):
+    """What the fused forms are for: in a bfloat16 step of a few tokens every norm runs
+    inside the projection that follows it and every mixer and feed-forward adds to the
+    stream itself, so the norm kernel and the stacks of partial sums do not appear; in a
+    step of many tokens, and with ``reproducible``, they do."""
+    from zig_ai_amd.engine import DecoderModel, ModelRunner, StepEntry
+    from zig_ai_amd.kernels import ops
+    folder = eu.model_folder(REAL_2L, 7, torch.bfloat16, std=0.02, norm_init="around_one")
+    calls = {"norm": 0, "stacks": 0}
+    norm_kernel, linear = ops.add_rmsnorm, ops.linear
+
+    def counting_norm(*a, **kw):
+        calls["norm"] += 1
+        return norm_kernel(*a, **kw)
+
+    def counting_linear(*a, **kw):
+        y = linear(*a, **kw)
+        if y is not None and y.dim() == 3:
+            calls["stacks"] += 1
+        return y
+
+    monkeypatch.setattr(ops, "add_rmsnorm", counting_norm)
+    monkeypatch.setattr(ops, "linear", counting_linear)
+    for reproducible in (False, True):
+        model = DecoderModel.from_folder(folder, "bfloat16", reproducible=reproducible)
+        runner = ModelRunner(model, page_size=16, num_pages=8, num_slots=2, use_graphs=False)
+        runner.admit("a")
+        runner.admit("b")
+        for tokens, few in (([list(range(20)), list(range(30, 47))], False), ([[5], [6]], True)):
+            calls.update(norm=0, stacks=0)
+            runner.step([StepEntry("a", tokens[0], [len(tokens[0]) - 1]),
+                         StepEntry("b", tokens[1], [len(tokens[1]) - 1])])
+            if few and not reproducible:
+                assert calls == {"norm": 0, "stacks": 0}, calls
+            else:
+                # two layers: four norms and the final one (the first is handed over and
+                # run by the projection's binding, which this count does not see);
+                # out_proj / w2 leave stacks
+                assert calls["norm"] >= 4 and calls["stacks"] >= 2, calls
+
+
 def test_graph_replays_with_library_products():
     """Decode batches beyond 16 rows send their projections to the GEMM library (K in
     ranges as a batched product where N is small, 32-bit logits): such steps are
