@@ -323,6 +323,11 @@ def test_gemm_bf16_decode_rows_normalised_by_the_kernel(M, N, K):
             assert rel_err(out, scale * (a @ w.double().T) + b.double()) < F32_TOL
         separate = o.linear(normed.materialise(), w.to(dev()), b.to(dev()), out_dtype=torch.float32)
         assert rel_err(out, separate.double()) < BF16_TOL
+        # both at once: the norm on the way in, the sum added to a stream on the way out
+        base = rand((M, N), torch.float32, 49)
+        stream_out = base.clone().to(dev())
+        assert o.linear(normed, w.to(dev()), b.to(dev()), accumulate=stream_out) is None
+        assert rel_err(stream_out, base.double() + out.double().cpu()) < F32_TOL
         exact = plain.rms_norm(x.double(), nw.double(), eps) @ w.double().T + b.double()
         assert rel_err(out, exact) < BF16_TOL
 
