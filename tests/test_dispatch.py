@@ -1,0 +1,39 @@
+"""Which kernel a projection goes to is decided on the host from its sizes alone; the
+decisions are checked here without a GPU."""
+
+import pytest
+
+from zig_ai_amd.kernels import ops
+
+
+@pytest.mark.parametrize("M,N,K,plan", [
+    (8, 2048, 2048, 4),          # few outputs: K in ranges until some 512 workgroups run
+    (8, 2048, 8192, 4),
+    (1, 64, 4096, 8),
+    (8, 6144, 12288, 2),         # a wide model: outputs alone fill the chip, K is too long
+    (3, 8192, 28672, 4),
+    (16, 5136, 9216, 2),
+    (2, 48, 8200, 0),            # no cut of 8200 is a multiple of 32: the product comes back
+    (17, 2048, 2048, 0),         # more than a decode batch
+    (8, 2048, 2052, 0),          # rows that do not start on 16-byte boundaries
+])
+def test_how_a_decode_product_reaches_the_stream(M, N, K, plan):
+    assert ops.accumulate_plan(M, N, K, False) == plan
+
+
+def test_every_plan_fits_the_kernel():
+    """Whatever the sizes, a plan's ranges are what the decode kernel takes: no longer than a
+    workgroup covers, and a multiple of 32 when K is cut."""
+    for N in (16, 100, 2048, 5136, 6144, 8192, 65536, 200000):
+        for K in range(8, 70000, 8):
+            plan = ops.accumulate_plan(8, N, K, False)
+            if plan == 0:
+                continue
+            assert (K + plan - 1) // plan <= ops.ROWS16_MAX_K_PER_WORKGROUP, (N, K, plan)
+            assert plan == 1 or K % (plan * 32) == 0, (N, K, plan)
+
+
+def test_the_kernel_that_runs_the_norm_covers_k_alone():
+    assert ops.accumulate_plan(8, 2048, 2048, True) == 1
+    assert ops.normed_rows_pay(8, 2048, 2048) and not ops.normed_rows_pay(8, 2048, 4608)
+    assert not ops.normed_rows_pay(16, 2048, 2048) and ops.normed_rows_pay(16, 16384, 2048)

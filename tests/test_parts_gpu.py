@@ -116,6 +116,32 @@ def test_swiglu_part(dtype, T):
     assert rel_err(out, expect) < TOL[dtype]
 
 
+@pytest.mark.parametrize("T", [1, 8, 16])
+@pytest.mark.parametrize("adds", [False, True])
+def test_swiglu_part_of_a_wide_model(T, adds):
+    """Hidden 6144 with a feed-forward of 12288 in bfloat16, a decode batch: K is longer
+    than one workgroup of the decode kernel covers and there are more outputs than fill
+    the chip, whether the part adds to the stream itself or hands its product back."""
+    from zig_ai_amd.parts import lookup
+    cls = lookup("feed_forward", "swiglu")
+    H, I = 6144, 12288
+    params = {"hidden_size": H, "intermediate_size": I}
+    w = {"gate.weight": rnd((I, H), 7, 0.02), "up.weight": rnd((I, H), 8, 0.02),
+         "down.weight": rnd((H, I), 9, 0.02)}
+    part = cls(params, place(w, cls.tensor_rules(params), torch.bfloat16), runtime(torch.bfloat16))
+    x = rnd((T, H), 10).to(torch.bfloat16)
+    wd = {k: v.to(torch.bfloat16).double() for k, v in w.items()}
+    expect = plain.swiglu_ffn(x.double(), wd["gate.weight"], wd["up.weight"], wd["down.weight"])
+    if adds:
+        stream0 = rnd((T, H), 11)
+        stream = stream0.to(dev())
+        assert part.forward(x.to(dev()), None, stream=stream) is None
+        assert rel_err(stream, stream0.double() + expect) < TOL[torch.bfloat16]
+    else:
+        out = total(part.forward(x.to(dev()), None))
+        assert rel_err(out, expect) < TOL[torch.bfloat16]
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("bias", [False, True])
 def test_short_conv_part(dtype, bias):

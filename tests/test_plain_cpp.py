@@ -262,7 +262,14 @@ def test_kernel_attention_path_against_twin(dtype, nh, nkv, d, rot, adjacent, pa
     through their twins, both on caches of their own with the same block table:
     portions of prompts, then further portions beside a decoded token, then decoded
     tokens only.  Queries, every element of both caches, and the outputs agree."""
-    from zig_ai_amd.engine.batch import _make_items
+    def work_items(counts, rows_per_item):
+        seq, row0, cnt, first = [], [], [], 0
+        for s, n in enumerate(counts):
+            for lo in range(0, n, rows_per_item):
+                seq.append(s); row0.append(first + lo); cnt.append(min(rows_per_item, n - lo))
+            first += n
+        return seq, row0, cnt
+
     steps = [[(0, 0, 37), (1, 0, 70)], [(0, 37, 1), (1, 70, 45), (2, 0, 9)], [(0, 38, 1), (1, 115, 1), (2, 9, 1)]]
     ends = [39, 116, 10]
     eps = 1e-5
@@ -306,7 +313,7 @@ def test_kernel_attention_path_against_twin(dtype, nh, nkv, d, rot, adjacent, pa
         kinds = ["plain"] + (["mfma"] if mfma else []) + (["decode"] if mfma and max(counts) == 1 else [])
         for kind in kinds:
             rows = {"plain": 32, "mfma": 128, "decode": 16}[kind] // G
-            item_seq, row0, cnt = (i32(x).to(dev()) for x in _make_items(counts, max(1, rows)))
+            item_seq, row0, cnt = (i32(x).to(dev()) for x in work_items(counts, max(1, rows)))
             fn = {"plain": ops().paged_attention, "mfma": ops().paged_attention_mfma,
                   "decode": ops().paged_attention_decode_mfma}[kind]
             got = fn(got_q, gpu_cache, step_table, i32(pos).to(dev()), item_seq, row0, cnt,

@@ -328,14 +328,37 @@ def _library_matmul(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtyp
     return out
 
 
+ROWS16_MAX_K_PER_WORKGROUP = 8192      # what one workgroup of the decode kernel covers
+
+
 def _accumulate_splits(N: int, K: int) -> int:
     """Into how many ranges K is cut when a decode batch's product is added to the
-    stream with atomics: until some 512 workgroups stream the weight."""
+    stream with atomics: until some 512 workgroups stream the weight, and at least so
+    many that one workgroup's range fits the kernel.  0: no cut fits (the caller then
+    takes the ordinary path and lets the next norm add the product)."""
     groups = (N + 15) // 16
     for split in (8, 4, 2):
-        if groups * split <= 640 and K % (split * 32) == 0 and K // split >= 512:
+        if groups * split <= 640 and K % (split * 32) == 0 and K // split >= 512 \
+                and K // split <= ROWS16_MAX_K_PER_WORKGROUP:
             return split
-    return 1
+    if K <= ROWS16_MAX_K_PER_WORKGROUP:
+        return 1
+    # a wide model: more workgroups than the chip wants, rather than a range too long
+    for split in (2, 4, 8, 16):
+        if K % (split * 32) == 0 and (K + split - 1) // split <= ROWS16_MAX_K_PER_WORKGROUP:
+            return split
+    return 0
+
+
+def accumulate_plan(M: int, N: int, K: int, normed: bool) -> int:
+    """How a decode batch's product reaches the stream: the number of ranges of K whose
+    partial products are added there with atomics, or 0 when the kernel that adds takes
+    no such product (the product then comes back and the caller adds it)."""
+    if M > 16 or K % 8:
+        return 0
+    if normed:
+        return 1            # the kernel that runs the norm covers K with one workgroup
+    return _accumulate_splits(N, K)
 
 
 def linear(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
@@ -371,22 +394,28 @@ def linear(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
             normed = x
         else:
             x = x.materialise()
-    if accumulate is not None and not (
-            M <= 16 and weight.dtype == torch.bfloat16 and K % 8 == 0 and not force_tiled
-            and (normed is not None or x.dtype == torch.bfloat16)):
-        accumulate = None
+    if normed is not None and accumulate is not None \
+            and normed.residual.untyped_storage().data_ptr() == accumulate.untyped_storage().data_ptr():
+        # workgroups would read rows of the stream while others add to them
+        normed, x = None, x.materialise()
+    splits = 1
+    if accumulate is not None:
+        if weight.dtype == torch.bfloat16 and not force_tiled \
+                and (normed is not None or x.dtype == torch.bfloat16):
+            splits = accumulate_plan(M, N, K, normed is not None)
+        else:
+            splits = 0
+        if splits == 0:
+            accumulate, splits = None, 1
     if normed is not None or accumulate is not None:
         _need(weight, "weight", torch.bfloat16, (N, K))
         if bias is not None:
             _need(bias, "bias", torch.float32, (N,))
         if normed is None:
             _need(x, "x", torch.bfloat16)
-        splits = 1
         if accumulate is not None:
             _need(accumulate, "accumulate", torch.float32, (M, N))
             out, out_code = accumulate, 0
-            if normed is None:
-                splits = _accumulate_splits(N, K)
         else:
             out_dtype = out_dtype or normed.dtype
             out = torch.empty((M, N), dtype=out_dtype, device=weight.device)
