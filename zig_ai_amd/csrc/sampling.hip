@@ -14,8 +14,12 @@
 //     listed tokens by the factor given for each (pipeline.zig:61-68).
 #include <math.h>
 #include <stdint.h>
+#include <stdio.h>
+
+#include <mutex>
 
 #include "common.h"
+#include "no_alloc.h"
 
 #define SM_THREADS 1024
 
@@ -578,6 +582,83 @@ extern "C" int za_argmax(const float* logits, int n_rows, int vocab, int* out, f
     return za_launch_status();
   }
   if (!part_v || !part_i || chunks > 65535) return ZA_ERR_ARG;
+  hipLaunchKernelGGL(argmax_chunk_kernel, dim3(n_rows, chunks), dim3(SM_THREADS), 0, stream,
+                     logits, vocab, part_v, part_i);
+  int rc = za_launch_status();
+  if (rc != 0) return rc;
+  hipLaunchKernelGGL(argmax_merge_kernel, dim3(n_rows), dim3(64), 0, stream, part_v, part_i,
+                     chunks, out);
+  return za_launch_status();
+}
+
+// ---------------------------------------------- greedy choice without allocation
+// The workspace of the chunked argmax for callers that cannot allocate (no_alloc.h):
+// ZA_ARGMAX_NO_ALLOC_MAX_PARTIALS maxima (32-bit floats), then as many indices.  Host
+// code never uses the array's name as an address (it is a stand-in there): the device
+// address is asked for once per device and kept.
+static __device__ __align__(256) unsigned char scratch[ZA_ARGMAX_NO_ALLOC_MAX_PARTIALS * 8];
+
+#define ZA_NO_ALLOC_MAX_DEVICES 64
+static void* scratch_of_device[ZA_NO_ALLOC_MAX_DEVICES];     // null until asked for
+static std::mutex scratch_lock;
+static thread_local char no_alloc_error[192];
+
+extern "C" const char* za_no_alloc_last_error(void) { return no_alloc_error; }
+
+// The current device's copy of `scratch`, or null with the reason in no_alloc_error.
+static void* scratch_address() {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess || device < 0 || device >= ZA_NO_ALLOC_MAX_DEVICES) {
+    snprintf(no_alloc_error, sizeof no_alloc_error,
+             "za_argmax_no_alloc: no current device below %d (hipGetDevice: %s)",
+             ZA_NO_ALLOC_MAX_DEVICES, hipGetErrorString(e));
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> hold(scratch_lock);
+  if (!scratch_of_device[device]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      snprintf(no_alloc_error, sizeof no_alloc_error,
+               "za_argmax_no_alloc: hipGetSymbolAddress on device %d: %s", device,
+               hipGetErrorString(e));
+      return nullptr;
+    }
+    scratch_of_device[device] = ptr;
+  }
+  return scratch_of_device[device];
+}
+
+extern "C" int za_argmax_no_alloc(const float* logits, int n_rows, int vocab, int* out,
+                                  int chunks, hipStream_t stream) {
+  no_alloc_error[0] = 0;
+  if (n_rows == 0) return 0;
+  if (n_rows < 0 || vocab <= 0 || !logits || !out || chunks < 1) {
+    snprintf(no_alloc_error, sizeof no_alloc_error,
+             "za_argmax_no_alloc: bad argument (n_rows %d, vocab %d, chunks %d, logits %p, out %p)",
+             n_rows, vocab, chunks, (const void*)logits, (void*)out);
+    return ZA_ERR_ARG;
+  }
+  if (chunks == 1) {                       // one workgroup a row: no partial results at all
+    hipLaunchKernelGGL(argmax_kernel, dim3(n_rows), dim3(SM_THREADS), 0, stream, logits, vocab,
+                       out);
+    return za_launch_status();
+  }
+  if (chunks > 65535 || (long long)n_rows * chunks > ZA_ARGMAX_NO_ALLOC_MAX_PARTIALS) {
+    snprintf(no_alloc_error, sizeof no_alloc_error,
+             "za_argmax_no_alloc: %d rows in %d chunks need %lld partial results, the array "
+             "holds %d (and a row at most 65535 chunks)",
+             n_rows, chunks, (long long)n_rows * chunks, ZA_ARGMAX_NO_ALLOC_MAX_PARTIALS);
+    return ZA_ERR_UNSUPPORTED;
+  }
+  void* base = scratch_address();
+  if (!base) return ZA_ERR_ARG;
+  float* part_v = reinterpret_cast<float*>(base);
+  int* part_i = reinterpret_cast<int*>(reinterpret_cast<unsigned char*>(base) +
+                                       (size_t)ZA_ARGMAX_NO_ALLOC_MAX_PARTIALS * sizeof(float));
+  // every entry the merge reads (n_rows * chunks of each) is written by the chunk kernel
+  // of this call: what an earlier call left is never read
   hipLaunchKernelGGL(argmax_chunk_kernel, dim3(n_rows, chunks), dim3(SM_THREADS), 0, stream,
                      logits, vocab, part_v, part_i);
   int rc = za_launch_status();

@@ -38,6 +38,7 @@ HIPCC_FLAGS = [
 ]
 
 EXTRA_FLAGS = {"blaslt": ["-lhipblaslt"]}   # host code around the GEMM library, no kernels
+EXTRA_HEADERS = {"sampling": ["no_alloc.h"]}    # headers a source includes beside common.h
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
@@ -95,7 +96,8 @@ def _writable_lib_dir() -> str:
 def source_digest(name: str) -> str:
     h = hashlib.sha256()
     host = name in HOST_SOURCES
-    for path in ([] if host else [os.path.join(CSRC_DIR, "common.h")]) + [_source_of(name)]:
+    headers = ([] if host else ["common.h"]) + EXTRA_HEADERS.get(name, [])
+    for path in [os.path.join(CSRC_DIR, h) for h in headers] + [_source_of(name)]:
         with open(path, "rb") as f:
             h.update(f.read())
     h.update(" ".join((CXX_FLAGS if host else HIPCC_FLAGS) + EXTRA_FLAGS.get(name, [])).encode())
