@@ -16,11 +16,85 @@ from __future__ import annotations
 import json
 import math
 import os
+from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence
 
 import torch
 
 DT = torch.float64
+
+
+# ------------------------------------------------ where a bfloat16 run rounds
+def bf(x: torch.Tensor) -> torch.Tensor:
+    """Round to bfloat16 (nearest even) and widen again."""
+    return x.to(torch.bfloat16).to(x.dtype)
+
+
+@dataclass
+class Rounding:
+    """Where a bfloat16 run of the model stores bfloat16 between its 32-bit sums, so that
+    the plain implementation can round at the same places (sums, norms, softmax, the
+    residual stream and the logits stay wide).  Always rounded: a norm's output, the
+    opening projections' outputs (q|k|v, B|C|x), q and k after the rotation, the
+    attention's output, the convolution's gated output, the SwiGLU's output.  What depends
+    on how a token was run is given per position (one boolean per row, ``True`` for the
+    form that a step of few tokens takes):
+
+      late_norm[key]   the product applies the row's scale itself:
+                       y = scale * (bf(x * w) @ W^T)  instead of  bf(x * scale * w) @ W^T;
+                       keys (layer, "mixer"), (layer, "feed_forward") and "head"
+      wide_gate        the SwiGLU gate is applied to the unrounded gate and up products
+      wide_close[key]  the closing product (out_proj, w2) is added to the stream as the
+                       32-bit sum it is, not rounded first; keys (layer, "mixer"),
+                       (layer, "feed_forward")
+
+    ``probabilities``: the attention rounds its probabilities for the second product
+    (the sum they are divided by stays unrounded).  A missing key means ``False``
+    everywhere."""
+
+    late_norm: Dict[object, torch.Tensor] = field(default_factory=dict)
+    wide_gate: Optional[torch.Tensor] = None
+    wide_close: Dict[object, torch.Tensor] = field(default_factory=dict)
+    probabilities: bool = True
+
+    @staticmethod
+    def _rows(mask: Optional[torch.Tensor], n: int) -> torch.Tensor:
+        return torch.zeros(n, dtype=torch.bool) if mask is None else mask.to(torch.bool)
+
+
+def by_row(mask: torch.Tensor, when_true, when_false) -> torch.Tensor:
+    """Rows of ``when_true()`` where ``mask`` holds and of ``when_false()`` elsewhere; each
+    is called with the row indices it has to produce and only if there are any."""
+    yes, no = mask.nonzero().flatten(), (~mask).nonzero().flatten()
+    if yes.numel() == 0:
+        return when_false(no)
+    if no.numel() == 0:
+        return when_true(yes)
+    a, b = when_true(yes), when_false(no)
+    out = torch.empty((mask.numel(),) + tuple(a.shape[1:]), dtype=a.dtype)
+    out[yes], out[no] = a, b
+    return out
+
+
+def normed_product(x: torch.Tensor, norm_w: torch.Tensor, eps: float, W: torch.Tensor,
+                   bias: Optional[torch.Tensor], rounding: Optional[Rounding],
+                   late: Optional[torch.Tensor]) -> torch.Tensor:
+    """``rms_norm(x) @ W^T + bias`` (norm.zig:6-33, then the projection), unrounded
+    result; with ``rounding`` the operand is rounded where a bfloat16 run rounds it."""
+    def add_bias(y):
+        return y if bias is None else y + bias
+    if rounding is None:
+        return add_bias(rms_norm(x, norm_w, eps) @ W.T)
+
+    def early(rows):
+        return add_bias(bf(rms_norm(x[rows], norm_w, eps)) @ W.T)
+
+    def late_form(rows):
+        xr = x[rows]
+        scale = 1.0 / torch.sqrt((xr * xr).sum(dim=-1, keepdim=True) / xr.shape[-1] + eps)
+        return add_bias((bf(xr * norm_w) @ W.T) * scale)
+
+    return by_row(Rounding._rows(late, x.shape[0]), late_form, early)
 
 
 # ------------------------------------------------------------------ the parts
@@ -32,8 +106,8 @@ def rms_norm(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
 
 def rope_inv_freq(rotary_dim: int, theta: float, dtype=DT) -> torch.Tensor:
     """rope.zig:29-32: freq_i = 1 / base^(2i / dim), i < dim/2."""
-    i = torch.arange(0, rotary_dim // 2, dtype=dtype)
-    return 1.0 / torch.pow(torch.tensor(theta, dtype=dtype), 2.0 * i / rotary_dim)
+    i = torch.arange(0, rotary_dim // 2, dtype=DT)
+    return (1.0 / torch.pow(torch.tensor(theta, dtype=DT), 2.0 * i / rotary_dim)).to(dtype)
 
 
 def apply_rope(x: torch.Tensor, positions: torch.Tensor, theta: float,
@@ -68,7 +142,7 @@ def kv_head_of(h: int, num_heads: int, num_kv_heads: int) -> int:
 
 def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                      positions: Optional[torch.Tensor] = None, window: int = 0,
-                     scale: Optional[float] = None) -> torch.Tensor:
+                     scale: Optional[float] = None, round_probabilities: bool = False) -> torch.Tensor:
     """q: [T, nh, d]; k, v: [T, nkv, d] (the whole sequence).  hybrid_attn.zig:571-608:
     s = q.k / sqrt(d), keys after the query masked, two-pass softmax, weighted
     sum of values.  ``window`` > 0 also masks keys at distance >= window."""
@@ -85,9 +159,19 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
         if window > 0:
             mask = mask | (dist >= window)
         s = s.masked_fill(mask, float("-inf"))
-        p = torch.exp(s - s.max(dim=-1, keepdim=True).values)
-        p = p / p.sum(dim=-1, keepdim=True)
-        out[:, h, :] = p @ v[:, g, :]
+        if round_probabilities:
+            # A bfloat16 run on the matrix cores rounds the unnormalised probabilities for
+            # the second product and divides by their unrounded sum.  It takes them
+            # relative to the row's maximum rounded up to a whole number on the base-2
+            # scale, p = 2^(s log2(e) - ceil(max)): the same softmax (the common factor
+            # cancels), and the one form in which the rounded values do not depend on the
+            # order in which the keys are visited.
+            t = s * math.log2(math.e)
+            p = torch.exp2(t - torch.ceil(t.max(dim=-1, keepdim=True).values))
+            out[:, h, :] = (bf(p) @ v[:, g, :]) / p.sum(dim=-1, keepdim=True)
+        else:
+            p = torch.exp(s - s.max(dim=-1, keepdim=True).values)
+            out[:, h, :] = (p / p.sum(dim=-1, keepdim=True)) @ v[:, g, :]
     return out
 
 
@@ -97,16 +181,46 @@ def attention_mixer(x: torch.Tensor, w: Dict[str, torch.Tensor], positions: torc
     """hybrid_attn.zig:286-640: projections (no bias), per-head RMSNorm of q and k
     (371-382, before the rotation, not on v), RoPE, causal softmax attention,
     output projection."""
-    T = x.shape[0]
-    q = (x @ w["q_proj"].T).view(T, num_heads, head_dim)
-    k = (x @ w["k_proj"].T).view(T, num_kv_heads, head_dim)
-    v = (x @ w["v_proj"].T).view(T, num_kv_heads, head_dim)
-    q = rms_norm(q, w["q_norm"], eps)
-    k = rms_norm(k, w["k_norm"], eps)
-    q = apply_rope(q, positions, theta)
-    k = apply_rope(k, positions, theta)
-    o = causal_attention(q, k, v, positions, window)
-    return o.reshape(T, num_heads * head_dim) @ w["out_proj"].T
+    qkv = x @ torch.cat([w["q_proj"], w["k_proj"], w["v_proj"]]).T
+    return attention_core(qkv, w, positions, num_heads, num_kv_heads, head_dim, eps, theta,
+                          window) @ w["out_proj"].T
+
+
+def attention_inputs(qkv: torch.Tensor, w: Dict[str, torch.Tensor], positions: torch.Tensor,
+                     num_heads: int, num_kv_heads: int, head_dim: int, eps: float, theta: float,
+                     rounding: Optional[Rounding] = None):
+    """The projected q|k|v rows as heads: q and k normalised per head and rotated
+    (hybrid_attn.zig:362-396), v as it is.  With ``rounding`` q and k are rounded after the
+    rotation (they are stored so)."""
+    T = qkv.shape[0]
+    nq, nk = num_heads * head_dim, num_kv_heads * head_dim
+    q = qkv[:, :nq].reshape(T, num_heads, head_dim)
+    k = qkv[:, nq:nq + nk].reshape(T, num_kv_heads, head_dim)
+    v = qkv[:, nq + nk:].reshape(T, num_kv_heads, head_dim)
+    q = apply_rope(rms_norm(q, w["q_norm"], eps), positions, theta)
+    k = apply_rope(rms_norm(k, w["k_norm"], eps), positions, theta)
+    if rounding is not None:
+        q, k = bf(q), bf(k)
+    return q, k, v
+
+
+def attention_core(qkv: torch.Tensor, w: Dict[str, torch.Tensor], positions: torch.Tensor,
+                   num_heads: int, num_kv_heads: int, head_dim: int, eps: float, theta: float,
+                   window: int = 0, rounding: Optional[Rounding] = None) -> torch.Tensor:
+    """From the projected q|k|v rows to the attention's output ``[T, heads * head_dim]``
+    (hybrid_attn.zig:362-608).  With ``rounding``: the probabilities are rounded if the
+    run rounds them, and the output."""
+    q, k, v = attention_inputs(qkv, w, positions, num_heads, num_kv_heads, head_dim, eps, theta,
+                               rounding)
+    return attention_output(q, k, v, positions, window, rounding)
+
+
+def attention_output(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, positions: torch.Tensor,
+                     window: int = 0, rounding: Optional[Rounding] = None) -> torch.Tensor:
+    o = causal_attention(q, k, v, positions, window,
+                         round_probabilities=rounding is not None and rounding.probabilities)
+    o = o.reshape(q.shape[0], q.shape[1] * q.shape[2])
+    return bf(o) if rounding is not None else o
 
 
 def causal_depthwise_conv(u: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
@@ -130,13 +244,17 @@ def short_conv_mixer(x: torch.Tensor, w: Dict[str, torch.Tensor]) -> torch.Tenso
     z = x @ w["in_proj"].T
     if "in_proj_bias" in w:
         z = z + w["in_proj_bias"]
-    H = x.shape[1]
-    B, C, xx = z[:, :H], z[:, H:2 * H], z[:, 2 * H:]
-    c = causal_depthwise_conv(B * xx, w["conv"], w.get("conv_bias"))
-    y = (C * c) @ w["out_proj"].T
+    y = short_conv_core(z, w) @ w["out_proj"].T
     if "out_proj_bias" in w:
         y = y + w["out_proj_bias"]
     return y
+
+
+def short_conv_core(z: torch.Tensor, w: Dict[str, torch.Tensor]) -> torch.Tensor:
+    """From the projected B|C|x rows to the gated convolution's output ``[T, H]``."""
+    H = z.shape[1] // 3
+    B, C, xx = z[:, :H], z[:, H:2 * H], z[:, 2 * H:]
+    return C * causal_depthwise_conv(B * xx, w["conv"], w.get("conv_bias"))
 
 
 def swiglu_ffn(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor,
@@ -206,36 +324,107 @@ class PlainLfm2:
                 out[local] = w[p + name]
         return out
 
-    def hidden_states(self, tokens: Sequence[int], position_offset: int = 0,
-                      upto_layer: Optional[int] = None) -> torch.Tensor:
-        """hybrid_layer.zig:366-492: h = x + mixer(norm1(x)); y = h + ffn(norm2(h))."""
+    def attention_qkv(self, i: int, x: torch.Tensor, positions: torch.Tensor,
+                      rounding: Optional[Rounding] = None):
+        """Layer ``i``'s queries, keys and values ``[T, heads, head_dim]`` from the stream:
+        what the attention reads (the queries) and what goes into the cache."""
+        lw = self.layer_weights(i)
+        w_qkv = torch.cat([lw["q_proj"], lw["k_proj"], lw["v_proj"]])
+        late = rounding.late_norm.get((i, "mixer")) if rounding is not None else None
+        qkv = normed_product(x, self.w[f"model.layers.{i}.operator_norm.weight"], self.eps, w_qkv,
+                             None, rounding, late)
+        if rounding is not None:
+            qkv = bf(qkv)
+        return attention_inputs(qkv, lw, positions, self.nh, self.nkv, self.d, self.eps,
+                                self.theta, rounding)
+
+    def layer(self, i: int, x: torch.Tensor, positions: torch.Tensor,
+              rounding: Optional[Rounding] = None,
+              attention_output_given: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """One decoder block on the whole sequence's stream ``x [T, H]``
+        (hybrid_layer.zig:366-492): h = x + mixer(norm1(x)); y = h + ffn(norm2(h)).
+        With ``rounding`` the same formulas, rounded to bfloat16 where such a run stores
+        bfloat16 (see ``Rounding``).  ``attention_output_given`` ``[T, heads * head_dim]``
+        stands in for the attention's output (tests that look at the rest of the block
+        alone)."""
         w = self.w
-        x = embedding(tokens, w["model.embed_tokens.weight"])
-        positions = torch.arange(len(tokens)) + position_offset
-        n_layers = len(self.kinds) if upto_layer is None else upto_layer
-        for i in range(n_layers):
-            p = f"model.layers.{i}."
+        p = f"model.layers.{i}."
+        lw = self.layer_weights(i)
+        if rounding is None:
             n1 = rms_norm(x, w[p + "operator_norm.weight"], self.eps)
-            lw = self.layer_weights(i)
-            if self.kinds[i] == "attention":
+            if self.kinds[i] == "attention" and attention_output_given is not None:
+                m = attention_output_given.to(x.dtype) @ lw["out_proj"].T
+            elif self.kinds[i] == "attention":
                 m = attention_mixer(n1, lw, positions, self.nh, self.nkv, self.d, self.eps,
                                     self.theta)
             else:
                 m = short_conv_mixer(n1, lw)
             h = x + m
             n2 = rms_norm(h, w[p + "ffn_norm.weight"], self.eps)
-            f = swiglu_ffn(n2, w[p + "feed_forward.w1.weight"], w[p + "feed_forward.w3.weight"],
-                           w[p + "feed_forward.w2.weight"])
-            x = h + f
+            return h + swiglu_ffn(n2, w[p + "feed_forward.w1.weight"],
+                                  w[p + "feed_forward.w3.weight"], w[p + "feed_forward.w2.weight"])
+        r = rounding
+        T = x.shape[0]
+
+        def closing(y, key):
+            wide = Rounding._rows(r.wide_close.get(key), T)
+            return torch.where(wide[:, None], y, bf(y))
+
+        late = r.late_norm.get((i, "mixer"))
+        if self.kinds[i] == "attention":
+            if attention_output_given is not None:
+                o = attention_output_given.to(x.dtype)
+            else:
+                q, k, v = self.attention_qkv(i, x, positions, r)
+                o = attention_output(q, k, v, positions, 0, r)
+            m = o @ lw["out_proj"].T
+        else:
+            z = bf(normed_product(x, w[p + "operator_norm.weight"], self.eps, lw["in_proj"],
+                                  lw.get("in_proj_bias"), r, late))
+            m = bf(short_conv_core(z, lw)) @ lw["out_proj"].T
+            if "out_proj_bias" in lw:
+                m = m + lw["out_proj_bias"]
+        h = x + closing(m, (i, "mixer"))
+        w_gu = torch.cat([w[p + "feed_forward.w1.weight"], w[p + "feed_forward.w3.weight"]])
+        gu = normed_product(h, w[p + "ffn_norm.weight"], self.eps, w_gu, None, r,
+                            r.late_norm.get((i, "feed_forward")))
+        gu = torch.where(Rounding._rows(r.wide_gate, T)[:, None], gu, bf(gu))
+        inter = gu.shape[1] // 2
+        g, u = gu[:, :inter], gu[:, inter:]
+        a = bf(g * (1.0 / (1.0 + torch.exp(-g))) * u)
+        return h + closing(a @ w[p + "feed_forward.w2.weight"].T, (i, "feed_forward"))
+
+    def embed(self, tokens: Sequence[int]) -> torch.Tensor:
+        return embedding(tokens, self.w["model.embed_tokens.weight"])
+
+    def hidden_states(self, tokens: Sequence[int], position_offset: int = 0,
+                      upto_layer: Optional[int] = None,
+                      rounding: Optional[Rounding] = None) -> torch.Tensor:
+        x = self.embed(tokens)
+        positions = torch.arange(len(tokens)) + position_offset
+        n_layers = len(self.kinds) if upto_layer is None else upto_layer
+        for i in range(n_layers):
+            x = self.layer(i, x, positions, rounding)
         return x
 
-    def logits(self, tokens: Sequence[int]) -> torch.Tensor:
+    def head(self, x: torch.Tensor, rounding: Optional[Rounding] = None,
+             late: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Final RMSNorm, then the output projection (tied: the embedding table;
-        gguf_model.zig:47-54, main.zig:870-877)."""
-        x = self.hidden_states(tokens)
-        n = rms_norm(x, self.w["model.embedding_norm.weight"], self.eps)
-        head = self.w["model.embed_tokens.weight"] if self.tied else self.w["lm_head.weight"]
-        return n @ head.T
+        gguf_model.zig:47-54, main.zig:870-877) of the rows ``x`` of the stream."""
+        table = self.w["model.embed_tokens.weight"] if self.tied else self.w["lm_head.weight"]
+        return normed_product(x, self.w["model.embedding_norm.weight"], self.eps, table, None,
+                              rounding, late)
+
+    def logits(self, tokens: Sequence[int], rows: Optional[Sequence[int]] = None,
+               rounding: Optional[Rounding] = None) -> torch.Tensor:
+        """Logits of all positions, or of ``rows``."""
+        x = self.hidden_states(tokens, rounding=rounding)
+        late = rounding.late_norm.get("head") if rounding is not None else None
+        if rows is not None:
+            idx = torch.as_tensor(list(rows), dtype=torch.long)
+            x = x[idx]
+            late = late[idx] if late is not None else None
+        return self.head(x, rounding, late)
 
     def greedy(self, prompt: Sequence[int], n_new: int) -> List[int]:
         toks = list(prompt)

@@ -56,6 +56,19 @@ TINY_F = {
     "tie_embedding": False, "max_position_embeddings": 2048,
 }
 
+# a wide, deep one: five layers, four of them attention on the matrix cores, width 1536 (the
+# decode kernels that run the norm themselves take it).  Of 3,000 configurations drawn at
+# random this one had the largest end-to-end deviation in bfloat16 (2.6e-2 of the largest
+# logit, with 6.7e-6 in 32-bit: rounding, not logic).
+TINY_G = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "hidden_size": 1536, "num_hidden_layers": 5, "num_attention_heads": 4,
+    "num_key_value_heads": 2, "head_dim": 64, "vocab_size": 417,
+    "layer_types": ["full_attention", "full_attention", "full_attention", "conv", "full_attention"],
+    "intermediate_size": 176, "rope_theta": 1000000.0, "norm_eps": 1e-6, "conv_L_cache": 3,
+    "conv_bias": False, "tie_embedding": False, "max_position_embeddings": 4096,
+}
+
 # two layers at the sizes of the LFM2-1.2B shape: the kernels' large-size paths
 REAL_2L = {
     "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
@@ -66,6 +79,10 @@ REAL_2L = {
     "conv_L_cache": 3, "conv_bias": False, "tie_embedding": True,
     "max_position_embeddings": 128000,
 }
+
+# three layers (ShortConv, attention, ShortConv) at the same sizes, for whole requests of
+# hundreds of tokens under every way of cutting them
+REAL_3L = dict(REAL_2L, num_hidden_layers=3, layer_types=["conv", "full_attention", "conv"])
 
 # widths that are multiples of neither 8 nor 16: fine in 32-bit, refused in bfloat16
 TINY_E = {

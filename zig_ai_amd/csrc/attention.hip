@@ -199,10 +199,12 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
   }
 }
 
+// `base2`: the partial maxima are whole numbers on the base-2 scale (what the matrix-core
+// kernels keep), so a partial result's weight 2^(m_z - m) is an exact power of two.
 template <typename T>
 __global__ void __launch_bounds__(64)
 attention_combine_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-                         T* __restrict__ out, int d, int nsplit) {
+                         T* __restrict__ out, int d, int nsplit, int base2) {
   const size_t row = blockIdx.x;  // token * nh + head
   const int lane = threadIdx.x;
   float mx = -INFINITY;
@@ -215,7 +217,7 @@ attention_combine_kernel(const float* __restrict__ part_acc, const float* __rest
     const float mz = part_ml[(row * nsplit + z) * 2];
     const float lz = part_ml[(row * nsplit + z) * 2 + 1];
     if (!(mz > -INFINITY)) continue;
-    const float w = expf(mz - mx);
+    const float w = base2 ? ldexpf(1.0f, (int)(mz - mx)) : expf(mz - mx);
     total += lz * w;
     const float* pa = part_acc + (row * nsplit + z) * d;
 #pragma unroll
@@ -243,7 +245,13 @@ attention_combine_kernel(const float* __restrict__ part_acc, const float* __rest
 // eight light waves are faster.)  Per tile of 64 keys:
 //   S^T = K Q^T   (keys as the rows of the first operand, 16 query rows as columns; a
 //                  lane ends up with the scores of ONE query row for 16 keys)
-//   p   = 2^(S^T * scale * log2(e) - m)  in 32-bit, running maximum and sum per lane
+//   p   = 2^(S^T * scale * log2(e) - m)  in 32-bit, running maximum and sum per lane;
+//                  m is the running maximum ROUNDED UP TO A WHOLE NUMBER, so every
+//                  rescaling factor 2^(m_old - m_new) is an exact power of two: the
+//                  probabilities' rounding to bfloat16 for the second product is then the
+//                  same whatever the order of tiles, ranges and waves (scaling by a power
+//                  of two commutes with rounding), and a row's result does not depend on
+//                  how its keys were cut beyond the order of 32-bit additions
 //   O^T += V^T P^T  (P^T goes from the accumulator registers straight into the second
 //                  operand: the matrix core does not care in which order the 32 keys of
 //                  a step are numbered as long as both operands agree, so V^T is stored
@@ -508,9 +516,10 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
 #pragma unroll
           for (int i = 0; i < 4; ++i) tmax = fmaxf(tmax, s[c][jb][i]);
         tmax = quad_max(tmax);
-        const float m_new = fmaxf(m[c], tmax * scale_log2e);   // the factor is positive
+        const float m_new = fmaxf(m[c], ceilf(tmax * scale_log2e));   // the factor is positive
         const float m_use = m_new > -INFINITY ? m_new : 0.f;
-        const float alpha = __builtin_amdgcn_exp2f(m[c] - m_use);   // m = -inf gives 0
+        // (nothing is accumulated yet while m is -inf: any finite factor does)
+        const float alpha = m[c] > -INFINITY ? ldexpf(1.0f, (int)(m[c] - m_use)) : 1.0f;
         float psum = 0.f;
 #pragma unroll
         for (int jb = 0; jb < 4; ++jb)
@@ -558,14 +567,13 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
     if (row_valid[c]) {
       const size_t orow = (size_t)tok[c] * nh + head[c];
       if (nsplit > 1) {
-        // unnormalised accumulator, and (maximum, sum) with the maximum turned back
-        // from the base-2 scale into the natural one the merge kernel works in
+        // unnormalised accumulator, and (maximum, sum), the maximum on the base-2 scale
         float* pa = part_acc + (orow * nsplit + z) * D;
 #pragma unroll
         for (int db = 0; db < DBLK; ++db)
           *reinterpret_cast<f32x4_t*>(pa + db * 16 + grp * 4) = o[c][db];
         if (grp == 0) {
-          part_ml[(orow * nsplit + z) * 2] = m[c] * 0.69314718055994531f;
+          part_ml[(orow * nsplit + z) * 2] = m[c];
           part_ml[(orow * nsplit + z) * 2 + 1] = l[c];
         }
         continue;
@@ -601,7 +609,7 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
                                    const int* __restrict__ wi_seq, const int* __restrict__ wi_row0,
                                    const int* __restrict__ wi_count, float* __restrict__ part_acc,
                                    float* __restrict__ part_ml, int nh, int nkv, int page_size,
-                                   float scale, int window, int keys_per_split, int nsplit) {
+                                   float scale_log2e, int window, int keys_per_split, int nsplit) {
   constexpr int KSTEPS = D / 32;
   constexpr int DBLK = D / 16;
   __shared__ float mg_m[NWV][16], mg_l[NWV][16];
@@ -765,20 +773,22 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
         const int kp = tile0 + (jb >> 1) * 32 + grp * 8 + (jb & 1) * 4 + i;
         bool valid = kp <= pos_row && kp >= lo && kp <= range_hi;
         if (window > 0 && kp <= pos_row - window) valid = false;
-        const float v = valid ? s[jb][i] * scale : -INFINITY;
+        const float v = valid ? s[jb][i] * scale_log2e : -INFINITY;
         s[jb][i] = v;
         tmax = fmaxf(tmax, v);
       }
     tmax = quad_max(tmax);
-    const float m_new = fmaxf(m, tmax);
+    // the running maximum as a whole number on the base-2 scale: every rescaling factor
+    // is an exact power of two (see paged_attention_mfma_kernel)
+    const float m_new = fmaxf(m, ceilf(tmax));
     const float m_use = m_new > -INFINITY ? m_new : 0.f;
-    const float alpha = expf(m - m_use);
+    const float alpha = m > -INFINITY ? ldexpf(1.0f, (int)(m - m_use)) : 1.0f;
     float psum = 0.f;
 #pragma unroll
     for (int jb = 0; jb < 4; ++jb)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float p = expf(s[jb][i] - m_use);
+        const float p = __builtin_amdgcn_exp2f(s[jb][i] - m_use);
         s[jb][i] = p;
         psum += p;
       }
@@ -831,7 +841,7 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
     float wgt[NWV], total = 0.f;
 #pragma unroll
     for (int w = 0; w < NWV; ++w) {
-      wgt[w] = expf(mg_m[w][r16] - mu);
+      wgt[w] = mg_m[w][r16] > -INFINITY ? ldexpf(1.0f, (int)(mg_m[w][r16] - mu)) : 0.f;
       total += mg_l[w][r16] * wgt[w];
     }
     const size_t orow = (size_t)tok * nh + head;
@@ -911,10 +921,10 @@ extern "C" int za_paged_attention(const void* q, void* out, const void* kv, cons
   dim3 grid((unsigned)((size_t)n_tokens * nh)), block(64);
   if (dtype == 0)
     hipLaunchKernelGGL((attention_combine_kernel<float>), grid, block, 0, stream, part_acc,
-                       part_ml, (float*)out, d, nsplit);
+                       part_ml, (float*)out, d, nsplit, 0);
   else
     hipLaunchKernelGGL((attention_combine_kernel<bf16_t>), grid, block, 0, stream, part_acc,
-                       part_ml, (bf16_t*)out, d, nsplit);
+                       part_ml, (bf16_t*)out, d, nsplit, 0);
   return za_launch_status();
 }
 
@@ -947,7 +957,7 @@ static int launch_attention_mfma(const void* q, void* out, const void* kv, const
   if (rc != 0 || nsplit == 1) return rc;
   dim3 cgrid((unsigned)((size_t)n_tokens * nh)), cblock(64);
   hipLaunchKernelGGL((attention_combine_kernel<bf16_t>), cgrid, cblock, 0, stream, part_acc,
-                     part_ml, (bf16_t*)out, D, nsplit);
+                     part_ml, (bf16_t*)out, D, nsplit, 1);
   return za_launch_status();
 }
 
@@ -1014,22 +1024,22 @@ extern "C" int za_paged_attention_decode_mfma(const void* q, void* out, const vo
     hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<64, 8>), grid, dim3(512), 0, stream,
                        (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
                        positions, wi_seq, wi_row0, wi_count, part_acc, part_ml, nh, nkv,
-                       page_size, scale, window, keys_per_split, nsplit);
+                       page_size, scale * 1.44269504088896341f, window, keys_per_split, nsplit);
   } else if (d == 64) {
     hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<64, 4>), grid, block, 0, stream,
                        (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
                        positions, wi_seq, wi_row0, wi_count, part_acc, part_ml, nh, nkv,
-                       page_size, scale, window, keys_per_split, nsplit);
+                       page_size, scale * 1.44269504088896341f, window, keys_per_split, nsplit);
   } else {
     hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<128, 4>), grid, block, 0, stream,
                        (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
                        positions, wi_seq, wi_row0, wi_count, part_acc, part_ml, nh, nkv,
-                       page_size, scale, window, keys_per_split, nsplit);
+                       page_size, scale * 1.44269504088896341f, window, keys_per_split, nsplit);
   }
   int rc = za_launch_status();
   if (rc != 0 || nsplit == 1) return rc;
   dim3 cgrid((unsigned)((size_t)n_tokens * nh)), cblock(64);
   hipLaunchKernelGGL((attention_combine_kernel<bf16_t>), cgrid, cblock, 0, stream, part_acc,
-                     part_ml, (bf16_t*)out, d, nsplit);
+                     part_ml, (bf16_t*)out, d, nsplit, 1);
   return za_launch_status();
 }

@@ -57,6 +57,9 @@ class StepContext:
     host: Optional[np.ndarray] = None
     offsets: Dict[str, Tuple[int, int]] = field(default_factory=dict)
     table_width: int = 0
+    # diagnostics: when a dict, the part that is running may leave copies of its
+    # intermediate tensors in it by name (token rows first); see DecoderModel.forward
+    taps: Optional[Dict[str, torch.Tensor]] = None
 
     def attention_items(self, rows_per_item: int):
         """Work items of at most ``rows_per_item`` consecutive query rows of one

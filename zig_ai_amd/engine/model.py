@@ -162,13 +162,30 @@ class DecoderModel:
         return [cache.view(call.cache, call.writes_cache) for call in self.schedule]
 
     # ------------------------------------------------------------------ forward
-    def forward(self, step: StepContext, views: Sequence[CacheView]) -> torch.Tensor:
+    def forward(self, step: StepContext, views: Sequence[CacheView],
+                taps: Optional[List[Dict[str, torch.Tensor]]] = None) -> torch.Tensor:
         """Run the step's tokens through every run-order entry and return 32-bit
-        logits ``[R, vocab]`` for ``step.logit_rows``."""
+        logits ``[R, vocab]`` for ``step.logit_rows``.  ``taps`` (diagnostics, as the
+        reference's per-layer dumps, /root/reference/src/main.zig:854-860): a list that
+        receives one dictionary for the embedding and one per run-order entry, with
+        ``"stream"``, the 32-bit residual stream ``[T, width]`` after it, and whatever the
+        entry's parts left under ``step.taps`` (the attention mixer: its queries, the
+        keys and values it stored, its output); all copies that later kernels do not
+        touch."""
         residual = self.embedding.forward(step.token_ids)
         pending = None
+        if taps is not None:
+            taps.append({"stream": residual.clone()})
         for call, view in zip(self.schedule, views):
+            step.taps = {} if taps is not None else None
             residual, pending = self.blocks[call.layer].forward(residual, pending, step, view)
+            if taps is not None:
+                now = residual.clone()
+                if pending is not None:
+                    now += (pending.sum(dim=0) if pending.dim() == 3 else pending).float()
+                step.taps["stream"] = now
+                taps.append(step.taps)
+        step.taps = None
         if step.n_logit_rows == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32,
                                device=self.runtime.device)

@@ -14,7 +14,7 @@ written for several sequences (``num_seqs``, ``block_tables[seq]``:
 
 from __future__ import annotations
 
-from typing import Callable, Hashable, List, Sequence
+from typing import Callable, Hashable, List, Optional, Sequence
 
 import torch
 
@@ -61,14 +61,17 @@ class ModelRunner:
         return build_step(entries, self.cache, self.device, self.model.spec.vocab_size,
                           self.model.item_granularities, self.model.spec.max_position)
 
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry],
+             taps: Optional[list] = None) -> torch.Tensor:
         """Logits ``[R, vocab]`` (32-bit) at the wanted places, in the order of the
-        entries and of each entry's ``want``."""
-        if self.graphs is not None and entries and all(len(e.tokens) == 1 for e in entries):
+        entries and of each entry's ``want``.  ``taps``: see ``DecoderModel.forward``
+        (such a step is never replayed from a graph)."""
+        if taps is None and self.graphs is not None and entries \
+                and all(len(e.tokens) == 1 for e in entries):
             logits = self._graph_step(entries)
         else:
             ctx = self.prepare(entries)
-            logits = self.model.forward(ctx, self.views)
+            logits = self.model.forward(ctx, self.views, taps)
         self.cache.commit_many([e.request for e in entries], [len(e.tokens) for e in entries])
         self.steps_run += 1
         return logits

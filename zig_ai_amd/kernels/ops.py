@@ -74,6 +74,19 @@ class KernelError(RuntimeError):
     pass
 
 
+# Diagnostics: when this is a list, every projection and attention call appends a record
+# of the form it took (which of several equivalent kernels ran, and so where values were
+# rounded to the storage type on the way): ``{"op", "M", "N", "K", ...}``.  Steps replayed
+# from a HIP graph call nothing here and leave no records.
+form_log: Optional[list] = None
+
+
+def _note(op: str, **fields) -> None:
+    if form_log is not None:
+        fields["op"] = op
+        form_log.append(fields)
+
+
 def _fn(lib: str, name: str):
     key = (lib, name)
     f = _functions.get(key)
@@ -429,6 +442,8 @@ def linear(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
             _ptr(weight), _ptr(bias), _ptr(out), out_code, M, N, K, splits,
             1 if accumulate is not None else 0, _stream())
         _check(rc, "gemm_bf16_rows16_stream", f"M={M} N={N} K={K} splits={splits}")
+        _note("linear", M=M, N=N, K=K, norm_in_product=normed is not None,
+              added_to_stream=accumulate is not None, partial_sums=1, out=out.dtype)
         return None if accumulate is not None else out
     _need(x, "x", (torch.float32, torch.bfloat16))
     _need(weight, "weight", (torch.float32, torch.bfloat16), (N, K))
@@ -440,6 +455,8 @@ def linear(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
         rc = _fn("gemm", "za_gemm_f32")(_ptr(x), _code(x.dtype), _ptr(weight), _ptr(bias), _ptr(out),
                                         _code(out_dtype), M, N, K, _stream())
         _check(rc, "gemm_f32", f"M={M} N={N} K={K}")
+        _note("linear", M=M, N=N, K=K, norm_in_product=False, added_to_stream=False,
+              partial_sums=1, out=out.dtype)
         return out
     if x.dtype != torch.bfloat16:
         raise KernelError("a bfloat16 weight needs bfloat16 activations")
@@ -457,17 +474,23 @@ def linear(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
         rc = _fn("gemm", "za_gemm_bf16_rows16")(_ptr(x), _ptr(weight), _ptr(bias), _ptr(stack),
                                                 0, M, N, K, splits, 0, _stream())
         _check(rc, "gemm_bf16_rows16", f"M={M} N={N} K={K} splits={splits}")
+        _note("linear", M=M, N=N, K=K, norm_in_product=False, added_to_stream=False,
+              partial_sums=splits, out=stack.dtype)
         return stack
     if library:
         # (with ranges of K: one batched product, [P, M, K/P] x [P, K/P, N])
         out = _library_matmul(x, weight, out_dtype, splits)
         if out is not None:
+            _note("linear", M=M, N=N, K=K, norm_in_product=False, added_to_stream=False,
+                  partial_sums=splits, out=out.dtype)
             return out
     out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     rc = _fn("gemm", "za_gemm_bf16")(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out),
                                      _code(out_dtype), M, N, K, 1 if force_tiled else 0,
                                      _stream())
     _check(rc, "gemm_bf16", f"M={M} N={N} K={K}")
+    _note("linear", M=M, N=N, K=K, norm_in_product=False, added_to_stream=False, partial_sums=1,
+          out=out.dtype)
     return out
 
 
@@ -502,6 +525,7 @@ def linear_swiglu(x, gate_up_weight: torch.Tensor) -> torch.Tensor:
         normed.eps if normed is not None else 0.0,
         _ptr(gate_up_weight), _ptr(out), M, I, K, _stream())
     _check(rc, "linear_swiglu", f"M={M} I={I} K={K}")
+    _note("linear_swiglu", M=M, N=2 * I, K=K, norm_in_product=normed is not None)
     return out
 
 
@@ -608,6 +632,7 @@ def paged_attention(q: torch.Tensor, kv_cache: torch.Tensor, block_table: torch.
         _ptr(part_acc), _ptr(part_ml), _code(q.dtype), nh, nkv, d, page_size, float(scale),
         int(window), int(keys_per_split), int(nsplit), _stream())
     _check(rc, "paged_attention")
+    _note("attention", kernel="plain", rows=T, dtype=q.dtype, nsplit=int(nsplit))
     return out
 
 
@@ -667,6 +692,7 @@ def paged_attention_mfma(q: torch.Tensor, kv_cache: torch.Tensor, block_table: t
         _ptr(part_acc), _ptr(part_ml), nh, nkv, d, page_size, float(scale), int(window),
         int(keys_per_split), int(nsplit), _stream())
     _check(rc, "paged_attention_mfma")
+    _note("attention", kernel="mfma", rows=T, dtype=q.dtype, nsplit=int(nsplit))
     return out
 
 
@@ -722,6 +748,7 @@ def paged_attention_decode_mfma(q: torch.Tensor, kv_cache: torch.Tensor,
         _ptr(part_acc), _ptr(part_ml), nh, nkv, d, page_size, float(scale), int(window),
         int(keys_per_split), int(nsplit), _stream())
     _check(rc, "paged_attention_decode_mfma")
+    _note("attention", kernel="decode_mfma", rows=T, dtype=q.dtype, nsplit=int(nsplit))
     return out
 
 

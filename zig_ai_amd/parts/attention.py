@@ -178,8 +178,24 @@ class GroupedQueryAttention(Mixer):
             o = ops.paged_attention(q, cache.kv, step.block_tables[cache.group], step.positions,
                                     item_seq, item_row0, item_count, n_items, self.scale,
                                     self.window, keys, nsplit)
+        if getattr(step, "taps", None) is not None:
+            self._leave_taps(step, cache, q, o)
         return ops.linear(o.view(T, nh * d), self.w_out, self.b_out, partial_ok=True,
                           accumulate=stream)
+
+    def _leave_taps(self, step, cache, q: torch.Tensor, o: torch.Tensor) -> None:
+        """Diagnostics: the queries, the keys and values of the step's tokens as they lie in
+        the cache now (read back through the tokens' places), and the attention's output."""
+        step.taps["q"] = q.clone()
+        step.taps["o"] = o.clone()
+        if not cache.writes:
+            return
+        page_size = cache.kv.shape[3]
+        place = step.slot_mapping[cache.group].long()
+        page, offset = place // page_size, place % page_size
+        step.taps["k"] = cache.kv[page, 0, :, offset, :]
+        values = cache.kv[:, 1].reshape(cache.kv.shape[0], self.num_kv_heads, self.head_dim, page_size)
+        step.taps["v"] = values[page, :, :, offset]
 
 
 register_mixer(GroupedQueryAttention.kind, GroupedQueryAttention)
