@@ -11,7 +11,14 @@ one decode step of the whole batch through the engine's own step function and
 greedy sampler, issued as generation issues them (the tokens of a step reach the
 next one on the device; the host reads them every 8 steps).  Prints ONE JSON line: decoded tokens per second as ``value``,
 a 2,048-token prefill under ``prefill``, the decode step against the HBM
-roofline under ``roofline``, and batch 1 / batch 64 decoding under ``points``.
+roofline under ``roofline``, and batch 1 / batch 64 decoding under ``points`` (tokens per
+second) with their step times, bytes and fractions under ``points_detail``.  Further keys:
+``prefill_chunked_512`` (the same 2,048 tokens in four steps of 512, the reference's
+``-ub 512``, /root/reference/src/main.zig:57-61), and ``calibration``: what this GPU
+does at best, measured here (a kernel that only reads 1 GiB; matrix-core instructions
+issued back to back), with every fraction also given against those (``frac_measured``).
+The model is ``DecoderModel.from_random(cfg, seed=0)``: the tensors that
+``write_random_model(cfg, folder, seed=0)`` stores, drawn on the device.
 """
 
 import argparse
@@ -213,7 +220,11 @@ def main() -> int:
         torch.cuda.empty_cache()
         return dt, ctx_mid
 
-    # ---- prefill of 2,048 tokens, one request, one step
+    # ---- what this GPU does at best
+    calibration = {"read_GBps": ops.measured_read_bandwidth() / 1e9,
+                   "mfma_bf16_TFLOPs": ops.measured_mfma_rate() / 1e12}
+
+    # ---- prefill of 2,048 tokens, one request: in one step, and in four steps of 512
     T = 2048
     if args.phase == "decode":
         dt, ctx_mid = decode_run(args.batch, args.prompt_len, args.steps, args.warmup)
@@ -221,49 +232,71 @@ def main() -> int:
                           "ms_per_step": dt / args.steps * 1e3,
                           "value": args.batch * args.steps / dt, "unit": "tokens/s"}), flush=True)
         return 0
-    runner = ModelRunner(model, page_size=page, num_pages=4 * (T // page + 1), num_slots=4)
-    for r in range(2):                                  # warm-up
-        runner.admit(("w", r))
-        runner.step([StepEntry(("w", r), tokens(T), [T - 1])])
-        runner.release(("w", r))
-    torch.cuda.synchronize()
-    reps = 3
-    t0 = time.perf_counter()
-    for r in range(reps):
-        runner.admit(("p", r))
-        runner.step([StepEntry(("p", r), tokens(T), [T - 1])])
-        runner.release(("p", r))
-    torch.cuda.synchronize()
-    prefill_s = (time.perf_counter() - t0) / reps
-    del runner
-    torch.cuda.empty_cache()
     n_attn = sum(1 for k in cfg["layer_types"] if k != "conv")
     qdim = cfg["num_attention_heads"] * (cfg["hidden_size"] // cfg["num_attention_heads"])
     prefill_flops = 2.0 * T * matmul_params(model) + n_attn * 2.0 * T * T * qdim \
         + 2.0 * vocab * cfg["hidden_size"]
-    prefill = {"value": T / prefill_s, "tokens": T, "ms": prefill_s * 1e3,
-               "frac": prefill_flops / prefill_s / PEAK_FLOPS["bf16"]}
+
+    def prefill_run(portion, reps=3):
+        runner = ModelRunner(model, page_size=page, num_pages=4 * (T // page + 1), num_slots=4)
+
+        def one(name):
+            runner.admit(name)
+            toks = tokens(T)
+            for lo in range(0, T, portion):
+                hi = min(T, lo + portion)
+                runner.step([StepEntry(name, toks[lo:hi], [hi - lo - 1] if hi == T else [])])
+            runner.release(name)
+
+        for r in range(2):                                  # warm-up
+            one(("w", r))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for r in range(reps):
+            one(("p", r))
+        torch.cuda.synchronize()
+        seconds = (time.perf_counter() - t0) / reps
+        del runner
+        torch.cuda.empty_cache()
+        rate = prefill_flops / seconds
+        return {"value": T / seconds, "tokens": T, "ms": seconds * 1e3,
+                "frac": rate / PEAK_FLOPS["bf16"],
+                "frac_measured": rate / (calibration["mfma_bf16_TFLOPs"] * 1e12)}
+
+    prefill = prefill_run(T)
     if args.phase == "prefill":
         print(json.dumps({"phase": "prefill", **prefill}), flush=True)
         return 0
+    prefill_chunked = prefill_run(512)
 
     # ---- the headline: batch 8 decoding from a 2,048-token context
+    hd = cfg["hidden_size"] // cfg["num_attention_heads"]
+    kv_bytes_per_token = n_attn * 2 * cfg["num_key_value_heads"] * hd * 2
+    weight_bytes = count_bytes(model)
+
+    def against_memory(batch, seconds_per_step, ctx):
+        """A decode step against the memory it has to read: every weight once and the
+        cache of the live requests."""
+        step_bytes = weight_bytes + batch * kv_bytes_per_token * ctx
+        rate = step_bytes / seconds_per_step
+        return {"ms_per_step": seconds_per_step * 1e3, "bytes": step_bytes,
+                "achieved_GBps": rate / 1e9, "frac": rate / HBM_BYTES_PER_S,
+                "frac_measured": rate / (calibration["read_GBps"] * 1e9)}
+
     dt, ctx_mid = decode_run(args.batch, args.prompt_len, args.steps, args.warmup)
     ms_per_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
-    hd = cfg["hidden_size"] // cfg["num_attention_heads"]
-    kv_bytes_per_token = n_attn * 2 * cfg["num_key_value_heads"] * hd * 2
-    step_bytes = count_bytes(model) + args.batch * kv_bytes_per_token * ctx_mid
-    achieved = step_bytes / (dt / args.steps)
-    roofline = {"bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_BYTES_PER_S / 1e9,
-                "unit": "GB/s", "frac": achieved / HBM_BYTES_PER_S}
+    headline = against_memory(args.batch, dt / args.steps, ctx_mid)
+    roofline = {"bound": "hbm", "achieved": headline["achieved_GBps"], "peak": HBM_BYTES_PER_S / 1e9,
+                "unit": "GB/s", "frac": headline["frac"], "frac_measured": headline["frac_measured"]}
 
-    points = {}
+    points, points_detail = {}, {}
     if not args.no_points:
         for b in (1, 64):
             steps = max(16, args.steps // 2)
-            d, _ = decode_run(b, args.prompt_len, steps, 4)
+            d, ctx = decode_run(b, args.prompt_len, steps, 4)
             points[f"decode_b{b}"] = b * steps / d
+            points_detail[f"decode_b{b}"] = against_memory(b, d / steps, ctx)
 
     line = {
         "metric": f"decode tok/s @ batch {args.batch} (LFM2-{args.shape.upper()} shape, context "
@@ -285,6 +318,8 @@ def main() -> int:
             "page_size": page, "weights_GB": count_bytes(model) / 1e9,
         },
         "prefill": prefill, "roofline": roofline, "points": points,
+        "points_detail": points_detail, "prefill_chunked_512": prefill_chunked,
+        "calibration": calibration,
     }
     print(json.dumps(line), flush=True)
     return 0

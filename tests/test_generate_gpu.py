@@ -18,15 +18,22 @@ pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def folder_for(cfg, seed, dtype=torch.float32):
-    return eu.model_folder(cfg, seed, dtype, **eu.sharp_kwargs())
+def folder_for(cfg, seed, dtype=torch.float32, weights="sharp"):
+    """``sharp``: the weights under which faults show (see ``engine_util.sharp_kwargs``).
+    ``as written``: what the workloads' definitions say, every matrix N(0, 0.02), with norm
+    weights of 1 (tiny-A) or drawn like everything else (``all normal``, tiny-B)."""
+    if weights == "sharp":
+        return eu.model_folder(cfg, seed, dtype, **eu.sharp_kwargs())
+    return eu.model_folder(cfg, seed, dtype, std=0.02,
+                           norm_init="ones" if weights == "as written" else "normal")
 
 
-def test_greedy_generation_tiny_a():
+@pytest.mark.parametrize("weights", ["sharp", "as written"])
+def test_greedy_generation_tiny_a(weights):
     """The tiny-A workload: prompts of 5/17/33 tokens, 16 greedy tokens each,
-    page size 4, in 32-bit: the same tokens as the plain implementation."""
+    page size 4, in 32-bit, seed 0: the same tokens as the plain implementation."""
     from zig_ai_amd.engine import Engine
-    folder = folder_for(TINY_A, 0)
+    folder = folder_for(TINY_A, 0, weights=weights)
     oracle = plain.PlainLfm2(folder)
     prompts = [eu.random_tokens(n, 256, 200 + n) for n in (5, 17, 33)]
     engine = Engine(folder, dtype="float32", page_size=4, num_pages=64, max_num_seqs=4)
@@ -57,6 +64,8 @@ def follow_sampling(oracle, prompt, tokens, params, number):
 
 @pytest.mark.parametrize("params", [
     dict(temperature=0.7, seed=1234),
+    dict(temperature=0.7, seed=1234, weights="as written"),
+    dict(temperature=0.7, seed=1234, weights="all normal"),
     dict(temperature=1.3, top_k=20, seed=7),
     dict(temperature=0.9, top_p=0.8, seed=8),
     dict(temperature=0.8, top_k=50, top_p=0.9, repetition_penalty=1.3, seed=9),
@@ -67,7 +76,8 @@ def test_sampled_generation_tiny_b(params):
     16, temperature 0.7 with a fixed sampling seed, page size 8; and the sampler's
     other options."""
     from zig_ai_amd.engine import Engine
-    folder = folder_for(TINY_B, 1)
+    params = dict(params)
+    folder = folder_for(TINY_B, 1, weights=params.pop("weights", "sharp"))
     oracle = plain.PlainLfm2(folder)
     prompts = [eu.random_tokens(n, 512, 300 + n) for n in (1, 8, 31, 64, 100)]
     engine = Engine(folder, dtype="float32", page_size=8, num_pages=128, max_num_seqs=8,
@@ -182,23 +192,27 @@ def test_command_line_diagnostics(tmp_path):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_trace_run(dtype, tmp_path):
-    """bin/trace_run on a mixed trace with a pool so small that pages are used
-    again; every wanted row against the plain implementation."""
+@pytest.mark.parametrize("kind", ["whole", "bulk", "portions", "mixed"])
+def test_trace_run(dtype, kind, tmp_path):
+    """bin/trace_run on the same requests whole, with the last 32 tokens one by one, in
+    portions of changing size, and mixed with a pool so small that pages are used again;
+    every wanted row, found through index.json, against the plain implementation."""
     import numpy as np
     store = torch.float32 if dtype == "float32" else torch.bfloat16
     folder = folder_for(TINY_B, 1, store)
     oracle = plain.PlainLfm2(folder)
     lengths = [70, 33, 100, 18, 64, 90]
     prompts = [eu.random_tokens(n, 512, 500 + i) for i, n in enumerate(lengths)]
-    schedule = eu.mixed(lengths, seed=4, max_live=4)
-    lines, wanted = [], []
+    schedule = {"whole": eu.whole(lengths), "bulk": eu.bulk_then_single(lengths, 32),
+                "portions": eu.changing_portions(lengths, 2),
+                "mixed": eu.mixed(lengths, seed=4, max_live=4)}[kind]
+    lines, wanted = [], {}
     for step, (entries, ends) in enumerate(schedule):
         rec = {"step": step, "entries": [], "end": [f"r{i}" for i in ends]}
         for i, a, b in entries:
             want = [k for k in range(b - a) if (a + k) % 3 != 1]        # not every place
             rec["entries"].append({"id": f"r{i}", "tokens": prompts[i][a:b], "want": want})
-            wanted.append((step, i, [a + k for k in want]))
+            wanted.setdefault(f"r{i}", []).extend(a + k for k in want)
         lines.append(json.dumps(rec))
     out_dir = tmp_path / "out"
     proc = subprocess.run(
@@ -207,24 +221,53 @@ def test_trace_run(dtype, tmp_path):
         input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=600)
     assert proc.returncode == 0, proc.stderr[-3000:]
     assert proc.stdout.split() == [w for s in range(len(schedule)) for w in ("done", str(s))]
-    expect = [oracle.logits(p) for p in prompts]
-    tol = 1e-4 if dtype == "float32" else 2.5e-2
-    by_step = {}
-    for step, i, places in wanted:
-        by_step.setdefault(step, []).append((i, places))
-    for step, items in by_step.items():
-        rows = sum(len(p) for _, p in items)
-        path = out_dir / f"{step}.f32"
-        if rows == 0:
-            assert not path.exists()
-            continue
-        data = torch.from_numpy(np.fromfile(path, dtype="<f4").reshape(rows, 512))
-        r = 0
-        for i, places in items:
-            if places:
-                err = eu.rel_err(data[r:r + len(places)], expect[i][places])
-                assert err < tol, f"step {step} request {i}: {err:.3e}"
-            r += len(places)
+    with open(out_dir / "index.json") as f:
+        index = json.load(f)
+    assert {r: [p for p, _, _ in rows] for r, rows in index.items()} == wanted
+    tol = 1e-4 if dtype == "float32" else 4e-2
+    files = {}
+    for i, p in enumerate(prompts):
+        expect = oracle.logits(p)
+        got = []
+        for place, step, row in index[f"r{i}"]:
+            if step not in files:
+                files[step] = torch.from_numpy(np.fromfile(out_dir / f"{step}.f32", dtype="<f4").reshape(-1, 512))
+            got.append(files[step][row])
+        err = eu.rel_err(torch.stack(got), expect[[place for place, _, _ in index[f"r{i}"]]])
+        assert err < tol, f"request {i}: {err:.3e}"
+    for step, (entries, _) in enumerate(schedule):       # a step that wants nothing writes nothing
+        rows = sum(1 for i, a, b in entries for k in range(a, b) if k % 3 != 1)
+        assert (out_dir / f"{step}.f32").exists() == (rows > 0)
+        if rows:
+            assert files[step].shape[0] == rows
+
+
+def test_trace_run_with_random_weights(tmp_path):
+    """``--config FILE --random-weights --seed S`` replays on the model that the random model
+    writer stores for that configuration and seed."""
+    import numpy as np
+    from zig_ai_amd.weights import write_random_model
+    cfg_path = tmp_path / "cfg.json"
+    cfg_path.write_text(json.dumps(TINY_A))
+    folder = str(tmp_path / "model")
+    write_random_model(TINY_A, folder, seed=9, dtype=torch.float32)
+    prompt = eu.random_tokens(21, 256, 77)
+    trace = json.dumps({"step": 0, "entries": [{"id": "a", "tokens": prompt[:13], "want": [12]}], "end": []}) \
+        + "\n" + json.dumps({"step": 1, "entries": [{"id": "a", "tokens": prompt[13:], "want": [0, 7]}],
+                             "end": ["a"]}) + "\n"
+    proc = subprocess.run(
+        [os.path.join(ROOT, "bin", "trace_run"), "--config", str(cfg_path), "--random-weights",
+         "--seed", "9", "--dtype", "float32", "--out", str(tmp_path / "out"), "--max-tokens", "64"],
+        input=trace, capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    expect = plain.PlainLfm2(folder).logits(prompt)
+    got = torch.cat([torch.from_numpy(np.fromfile(tmp_path / "out" / f"{s}.f32", dtype="<f4").reshape(-1, 256))
+                     for s in (0, 1)])
+    assert eu.rel_err(got, expect[[12, 13, 20]]) < 1e-4
+    assert json.load(open(tmp_path / "out" / "index.json")) == {"a": [[12, 0, 0], [13, 1, 0], [20, 1, 1]]}
+    bad = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--dtype", "float32", "--out",
+                          str(tmp_path / "o2"), "--max-tokens", "64"], input="", capture_output=True, text=True)
+    assert bad.returncode != 0 and "--model" in bad.stderr
 
 
 def test_an_engine_used_again_and_again_keeps_nothing():

@@ -107,6 +107,58 @@ def test_random_model_is_reproducible_and_loads(tmp_path):
                        loaded[("layer", 0, "mixer")]["q_proj.weight"].float())
 
 
+def test_random_values_are_keyed_by_seed_name_and_index(tmp_path):
+    """A value is a function of (seed, tensor name, element index): the known answer of the
+    generator's round function, prefixes and chunks agree, and a tensor does not change
+    when the model around it does (more layers: other tensors are drawn before it)."""
+    from zig_ai_amd.weights import random_init as ri
+    # Philox-4x32-10, counter 0, key 0: the generator's published known answer
+    words = ri._philox(torch.zeros(1, dtype=torch.int64), (0, 0))
+    assert [int(w[0]) for w in words] == [0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8]
+    a = ri.keyed_normal(7, "x.weight", 1003)
+    assert torch.equal(a[:99], ri.keyed_normal(7, "x.weight", 99))
+    assert torch.equal(a, ri.keyed_normal(7, "x.weight", 1003, chunk=64))
+    assert not torch.equal(a, ri.keyed_normal(8, "x.weight", 1003))
+    assert not torch.equal(a, ri.keyed_normal(7, "y.weight", 1003))
+    big = ri.keyed_normal(1, "t", 400000)
+    assert abs(float(big.mean())) < 0.01 and abs(float(big.std()) - 1) < 0.01
+    assert abs(float((big.abs() > 2).float().mean()) - 0.0455) < 0.003
+    deeper = dict(TINY_A, num_hidden_layers=5,
+                  layer_types=["full_attention"] + TINY_A["layer_types"])
+    d1, d2 = str(tmp_path / "a"), str(tmp_path / "b")
+    write_random_model(TINY_A, d1, seed=3, dtype=torch.float32)
+    write_random_model(deeper, d2, seed=3, dtype=torch.float32)
+    c1, c2 = Checkpoint(d1), Checkpoint(d2)
+    for name in ("model.embed_tokens.weight", "model.layers.1.conv.in_proj.weight",
+                 "model.layers.3.feed_forward.w2.weight"):
+        assert torch.equal(c1.tensor(name), c2.tensor(name)), name
+
+
+@pytest.mark.gpu
+def test_a_random_model_drawn_on_the_gpu_is_the_folder(tmp_path):
+    """``DecoderModel.from_random`` (what the benchmark builds) holds the tensors that the
+    random model writer stores for the same configuration and seed, drawn on the CPU."""
+    from zig_ai_amd.engine import DecoderModel
+    from zig_ai_amd.weights import random_init as ri
+    folder = str(tmp_path / "m")
+    tensors = ri.random_tensors(config_from_dict(TINY_B).to_spec(), 11, torch.bfloat16,
+                                norm_init="around_one", device="cpu")
+    ri.write_random_model(TINY_B, folder, seed=11, dtype=torch.bfloat16, norm_init="around_one")
+    stored = Checkpoint(folder)
+    for name, t in tensors.items():
+        assert torch.equal(stored.tensor(name), t), name
+    drawn = DecoderModel.from_random(TINY_B, seed=11, dtype="bfloat16", norm_init="around_one")
+    loaded = DecoderModel.from_folder(folder, "bfloat16")
+    for a, b in zip(drawn.blocks, loaded.blocks):
+        for part in ("mixer", "feed_forward", "mixer_norm", "feed_forward_norm"):
+            pa, pb = getattr(a, part), getattr(b, part)
+            for key, value in vars(pa).items():
+                if isinstance(value, torch.Tensor):
+                    assert torch.equal(value, getattr(pb, key)), (part, key)
+    assert torch.equal(drawn.embedding.weight, loaded.embedding.weight)
+    assert torch.equal(drawn.head.weight, loaded.head.weight)
+
+
 def test_kept_precision():
     bf, f32, f16 = torch.bfloat16, torch.float32, torch.float16
     assert keep_dtype(bf, "matrix", bf) == bf

@@ -122,31 +122,30 @@ class DecoderModel:
     @classmethod
     def from_random(cls, config, seed: int = 0, dtype="bfloat16",
                     device: Optional[torch.device] = None, std: float = 0.02,
-                    norm_init: str = "ones"):
-        """A model with random weights drawn on the device, for benchmarks: the same
-        distributions as the random model writer, without the trip through a file.
-        ``config`` is a typed configuration or a config.json dictionary."""
+                    norm_init: str = "ones", reproducible: bool = False,
+                    role_std: Optional[Mapping[str, float]] = None):
+        """The model that ``write_random_model(config, folder, seed, ...)`` followed by
+        ``from_folder`` gives, without the trip through a file: every tensor is drawn on the
+        device by the same keyed generator (a value depends on seed, tensor name and element
+        index only) and kept as the loader would keep it.  ``config`` is a typed
+        configuration or a config.json dictionary."""
         from ..config import config_from_dict
         from ..weights.loader import expected_tensors, keep_dtype
+        from ..weights.random_init import deviation_of, random_tensor
         device = device or require_gpu()
         if isinstance(config, Mapping):
             config = config_from_dict(config)
         spec = config.to_spec()
-        rt = parts.Runtime(device=device, dtype=run_dtype(dtype))
-        gen = torch.Generator(device=device)
-        gen.manual_seed(int(seed))
+        rt = parts.Runtime(device=device, dtype=run_dtype(dtype), stream_additions=not reproducible)
         tensors: Dict[Any, Dict[str, torch.Tensor]] = {}
         for exp in expected_tensors(spec):
-            shape = exp.rule.shapes[0]
-            if exp.rule.role == "norm" and norm_init == "ones":
-                t = torch.ones(shape, dtype=torch.float32, device=device)
-            else:
-                t = torch.empty(shape, dtype=torch.float32, device=device)
-                t.normal_(0.0, std, generator=gen)
-                if exp.rule.role == "norm" and norm_init == "around_one":
-                    t += 1.0
-            tensors.setdefault(exp.owner, {})[exp.local] = t.to(
-                keep_dtype(rt.dtype, exp.rule.role, rt.dtype))
+            stored = random_tensor(seed, exp.names[0], exp.rule.stored_shape or exp.rule.shapes[0],
+                                   exp.rule.role, rt.dtype,
+                                   deviation_of(exp.names[0], exp.rule.role, std, role_std or {}),
+                                   norm_init, device)
+            kept = keep_dtype(stored.dtype, exp.rule.role, rt.dtype)
+            tensors.setdefault(exp.owner, {})[exp.local] = \
+                stored.reshape(exp.rule.shapes[0]).to(kept).contiguous()
         model = cls(spec, tensors, rt)
         model.config = config
         return model

@@ -64,6 +64,8 @@ _SIGNATURES = {
                                 c_void_p, c_int, c_void_p],
     ("sampling", "za_repetition_penalty"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                                             c_void_p],
+    ("calibrate", "za_read_stream"): [c_void_p, c_size_t, c_int, c_void_p, c_void_p],
+    ("calibrate", "za_mfma_loop"): [c_int, c_int, c_void_p, c_void_p],
     ("blaslt", "za_lt_matmul"): [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                  c_void_p, c_size_t, c_void_p],
 }
@@ -868,3 +870,44 @@ def repetition_penalty_(logits: torch.Tensor, rows: torch.Tensor, tokens: torch.
     rc = _fn("sampling", "za_repetition_penalty")(_ptr(logits), logits.shape[1], _ptr(rows),
                                                   _ptr(tokens), _ptr(factors), n, _stream())
     _check(rc, "repetition_penalty")
+
+
+# ------------------------------------------------------------ measured ceilings
+def measured_read_bandwidth(n_bytes: int = 1 << 30, repeats: int = 5) -> float:
+    """Bytes per second of a kernel that only reads ``n_bytes`` of device memory (more than
+    any cache holds), the best of ``repeats`` runs; see csrc/calibrate.hip."""
+    n_bytes = n_bytes // 16 * 16
+    device = torch.device("cuda", torch.cuda.current_device())
+    src = torch.zeros((n_bytes,), dtype=torch.uint8, device=device)
+    sink = torch.zeros((1,), dtype=torch.float32, device=device)
+    fn = _fn("calibrate", "za_read_stream")
+    best = 0.0
+    for i in range(repeats + 1):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        _check(fn(_ptr(src), n_bytes, 256 * 16, _ptr(sink), _stream()), "read_stream")
+        stop.record()
+        stop.synchronize()
+        if i:                                   # (the first run also loads the kernel)
+            best = max(best, n_bytes / (start.elapsed_time(stop) * 1e-3))
+    return best
+
+
+def measured_mfma_rate(repeats: int = 3) -> float:
+    """bfloat16 flop per second of matrix-core instructions issued back to back from
+    registers by every compute unit; see csrc/calibrate.hip."""
+    device = torch.device("cuda", torch.cuda.current_device())
+    sink = torch.zeros((1,), dtype=torch.float32, device=device)
+    fn = _fn("calibrate", "za_mfma_loop")
+    blocks, iters = 256 * 8, 20000
+    flops = blocks * 4 * iters * 8 * 16384.0
+    best = 0.0
+    for i in range(repeats + 1):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        _check(fn(blocks, iters, _ptr(sink), _stream()), "mfma_loop")
+        stop.record()
+        stop.synchronize()
+        if i:
+            best = max(best, flops / (start.elapsed_time(stop) * 1e-3))
+    return best
