@@ -119,7 +119,7 @@ def count_bytes(model):
     add(model.head.weight)
     add(model.final_norm.weight)
     for b in model.blocks:
-        for part in (b.mixer_norm, b.mixer, b.feed_forward_norm, b.feed_forward):
+        for part in b.parts.values():
             for v in vars(part).values():
                 if hasattr(v, "data_ptr"):
                     add(v)

@@ -82,7 +82,8 @@ def test_a_norm_that_cannot_defer_runs():
 def test_block_with_parts_that_add_to_the_stream_leaves_nothing_pending():
     for adds in (True, False):
         residual = torch.ones(2, 3)
-        block = PreNormResidualBlock(Norm(True), StreamPart(adds), Norm(True), StreamPart(adds))
+        block = PreNormResidualBlock({"mixer_norm": Norm(True), "mixer": StreamPart(adds),
+                                      "feed_forward_norm": Norm(True), "feed_forward": StreamPart(adds)})
         out, pending = block.forward(residual, None, "step", "cache")
         assert out is residual
         # h = x + (2x + 1) = 4; y = h + (2h + 1) = 13

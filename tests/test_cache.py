@@ -10,9 +10,9 @@ from zig_ai_amd.parts import PagedNeed, StateNeed
 
 
 def manager(num_pages=16, page_size=4, num_slots=4, window=0, extra=None):
-    needs = {0: StateNeed((8, 3)), 1: PagedNeed(2, 16, 0), 2: StateNeed((8, 3)), 3: PagedNeed(2, 16, 0)}
+    needs = {0: StateNeed((8, 3)), 1: PagedNeed.kv(2, 16, 0), 2: StateNeed((8, 3)), 3: PagedNeed.kv(2, 16, 0)}
     if window:
-        needs[4] = PagedNeed(2, 16, window)
+        needs[4] = PagedNeed.kv(2, 16, window)
     needs.update(extra or {})
     return CacheManager(needs, page_size, num_pages, num_slots, allocate=False)
 
@@ -51,7 +51,7 @@ def test_block_table_growth_like_the_reference():
     test_paged_attention_gpu.zig:51,294: 5 tokens at page 4 -> 2 pages, 7 -> 2, 9 -> 3;
     40 at 16 -> 3; 4096 at 16 -> 256."""
     for tokens, page, want in [(5, 4, 2), (7, 4, 2), (9, 4, 3), (40, 16, 3), (4096, 16, 256)]:
-        m = CacheManager({0: PagedNeed(1, 16)}, page, 300, 1, allocate=False)
+        m = CacheManager({0: PagedNeed.kv(1, 16)}, page, 300, 1, allocate=False)
         m.admit("r")
         m.reserve("r", tokens)
         assert len(m.table("r", 0)) == want
@@ -73,7 +73,7 @@ def test_groups_and_views():
     assert m.groups[0].cache_ids == [1, 3] and m.groups[1].cache_ids == [4]
     assert m.view(1).kind == "paged" and m.view(1).group == 0 and m.view(4).group == 1
     assert m.view(0).kind == "state" and m.view(7).kind == "none"
-    assert m.floats_per_slot == 2 * 8 * 3
+    assert m.bytes_per_slot == 2 * 8 * 3 * 4
 
 
 def test_reserve_is_all_or_nothing():
@@ -180,7 +180,7 @@ def test_scattered_pools_hand_out_every_page_once():
     books stay right when pages come back."""
     orders = []
     for _ in range(2):
-        m = CacheManager({0: PagedNeed(1, 16)}, 4, 257, 2, allocate=False, scatter_pages=True)
+        m = CacheManager({0: PagedNeed.kv(1, 16)}, 4, 257, 2, allocate=False, scatter_pages=True)
         m.admit("r")
         m.reserve("r", 257 * 4)
         order = m.table("r", 0)
@@ -196,7 +196,7 @@ def test_scattered_pools_hand_out_every_page_once():
     assert orders[0] != list(range(257))
     runs = sum(1 for a, b in zip(orders[0], orders[0][1:]) if b == a + 1)
     assert runs < 16                                   # no long stretches in address order
-    plain = CacheManager({0: PagedNeed(1, 16)}, 4, 257, 2, allocate=False)
+    plain = CacheManager({0: PagedNeed.kv(1, 16)}, 4, 257, 2, allocate=False)
     plain.admit("r")
     plain.reserve("r", 40)
     assert plain.table("r", 0) == list(range(10))      # the default: 0, 1, 2 ...

@@ -17,9 +17,9 @@ CPU = torch.device("cpu")
 
 
 def manager(num_pages=40, page_size=4, num_slots=4, window=0):
-    needs = {0: StateNeed((8, 3)), 1: PagedNeed(2, 16, 0), 3: PagedNeed(2, 16, 0)}
+    needs = {0: StateNeed((8, 3)), 1: PagedNeed.kv(2, 16, 0), 3: PagedNeed.kv(2, 16, 0)}
     if window:
-        needs[4] = PagedNeed(2, 16, window)
+        needs[4] = PagedNeed.kv(2, 16, window)
     return CacheManager(needs, page_size, num_pages, num_slots, allocate=False)
 
 

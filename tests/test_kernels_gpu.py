@@ -332,6 +332,31 @@ def test_gemm_bf16_decode_rows_normalised_by_the_kernel(M, N, K):
         assert rel_err(out, exact) < BF16_TOL
 
 
+def test_a_product_that_reads_and_adds_to_the_same_stream():
+    """``linear(NormedRows(stream), W[H, H], accumulate=stream)``: workgroups would read rows
+    of the stream while others add to them; the norm is run first instead, and the result is
+    stream + norm(stream as it was) W^T."""
+    o = ops()
+    H = 2048
+    x0 = rand((8, H), torch.float32, 90)
+    nw = rand((H,), torch.float32, 91, 0.2) + 1
+    w = rand((H, H), torch.bfloat16, 92, 0.05)
+    stream = x0.to(dev())
+    normed = o.NormedRows(stream, nw.to(dev()), 1e-5, torch.bfloat16)
+    assert o.linear(normed, w.to(dev()), accumulate=stream) is None
+    a = plain.rms_norm(x0.double(), nw.double(), 1e-5).to(torch.bfloat16).double()
+    assert rel_err(stream, x0.double() + a @ w.double().T) < 1e-4
+    # with another tensor to add to, the kernel runs the norm itself
+    other = torch.zeros((8, H), dtype=torch.float32, device=dev())
+    o.form_log = []
+    try:
+        o.linear(o.NormedRows(x0.to(dev()), nw.to(dev()), 1e-5, torch.bfloat16), w.to(dev()), accumulate=other)
+        assert o.form_log[-1]["norm_in_product"] and o.form_log[-1]["added_to_stream"]
+    finally:
+        o.form_log = None
+    assert rel_err(other, a @ w.double().T) < BF16_TOL
+
+
 def test_normed_rows_beyond_the_fused_kernel_run_the_norm_kernel():
     """More than 16 rows, a K no workgroup covers, 32-bit weights: the norm runs as a
     kernel of its own and the product is the usual one."""

@@ -202,7 +202,7 @@ def test_attention_part(dtype, nh, nkv, d, window):
          "v_proj.weight": rnd((nkv * d, H), 21, 0.2), "out_proj.weight": rnd((H, nh * d), 22, 0.2),
          "q_norm.weight": rnd((d,), 23, 0.2) + 1, "k_norm.weight": rnd((d,), 24, 0.2) + 1}
     need = cls.cache_need(params)
-    assert (need.num_kv_heads, need.head_dim, need.window) == (nkv, d, window)
+    assert need.is_kv and (need.planes[0], need.window) == ((nkv, d), window)
     part = cls(params, place(w, cls.tensor_rules(params), dtype), runtime(dtype))
     cache = CacheManager({0: need}, 8, 16, 2, device=dev(), dtype=dtype)
     view = cache.view(0)
@@ -237,11 +237,11 @@ def test_block_arrangement(dtype, T):
           "out_proj.weight": rnd((H, H), 34, 0.2)}
     fw = {"gate.weight": rnd((I, H), 35, 0.2), "up.weight": rnd((I, H), 36, 0.2), "down.weight": rnd((H, I), 37, 0.2)}
     mp, fp, npar = {"hidden_size": H, "kernel_size": L, "bias": False}, {"hidden_size": H, "intermediate_size": I}, {"width": H, "eps": eps}
-    block = lookup("arrangement", "pre_norm_residual")(
-        norm_cls(npar, place({"weight": n1w}, norm_cls.tensor_rules(npar), dtype), rt),
-        mix_cls(mp, place(mw, mix_cls.tensor_rules(mp), dtype), rt),
-        norm_cls(npar, place({"weight": n2w}, norm_cls.tensor_rules(npar), dtype), rt),
-        ffn_cls(fp, place(fw, ffn_cls.tensor_rules(fp), dtype), rt))
+    block = lookup("arrangement", "pre_norm_residual")({
+        "mixer_norm": norm_cls(npar, place({"weight": n1w}, norm_cls.tensor_rules(npar), dtype), rt),
+        "mixer": mix_cls(mp, place(mw, mix_cls.tensor_rules(mp), dtype), rt),
+        "feed_forward_norm": norm_cls(npar, place({"weight": n2w}, norm_cls.tensor_rules(npar), dtype), rt),
+        "feed_forward": ffn_cls(fp, place(fw, ffn_cls.tensor_rules(fp), dtype), rt)})
     cache = CacheManager({0: mix_cls.cache_need(mp)}, 4, 4, 1, device=dev(), dtype=dtype)
     cache.admit("r")
     x = rnd((T, H), 38)

@@ -11,7 +11,7 @@ from zig_ai_amd.parts import PagedNeed, StateNeed
 
 
 def make(num_pages=16, page_size=4, num_slots=4, **kw):
-    cache = CacheManager({0: StateNeed((4, 3)), 1: PagedNeed(1, 16)}, page_size, num_pages,
+    cache = CacheManager({0: StateNeed((4, 3)), 1: PagedNeed.kv(1, 16)}, page_size, num_pages,
                          num_slots, allocate=False)
     return cache, Scheduler(cache, **kw)
 
@@ -178,7 +178,7 @@ def run_differential(seed):
                   chunk_size=rng.randint(2, 12), max_model_len=rng.choice([0, 0, 30]))
     needs = {0: StateNeed((4, 3))}
     for g, w in enumerate(windows):
-        needs[1 + g] = PagedNeed(1, 16, w)
+        needs[1 + g] = PagedNeed.kv(1, 16, w)
     cache = CacheManager(needs, page_size, num_pages, num_slots, allocate=False)
     sched = Scheduler(cache, **limits)
     pcache = PlainCache(windows, num_pages, page_size, num_slots)

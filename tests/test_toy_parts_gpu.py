@@ -95,7 +95,7 @@ class ToyConfig:
                            {k + ".weight": (p + "ffn." + k + ".weight",) for k in ("gate", "up", "down")})
             n1 = PartSpec("rms_norm", {"width": H, "eps": 1e-5}, {"weight": (p + "norm1.weight",)})
             n2 = PartSpec("rms_norm", {"width": H, "eps": 1e-5}, {"weight": (p + "norm2.weight",)})
-            layers.append(LayerSpec(mixer, ffn, n1, n2))
+            layers.append(LayerSpec.pre_norm(mixer, ffn, n1, n2))
         schedule = tuple(LayerCall(*c) for c in d["schedule"])
         return ModelSpec("ToyForCausalLM", H, V,
                          PartSpec("token_embedding", {"vocab_size": V, "hidden_size": H},
@@ -282,7 +282,7 @@ class RoutedConfig:
             ffn = PartSpec("toy_top_one_experts", {"hidden_size": H, "intermediate_size": I, "experts": E}, names)
             n1 = PartSpec("rms_norm", {"width": H, "eps": 1e-5}, {"weight": (p + "norm1.weight",)})
             n2 = PartSpec("rms_norm", {"width": H, "eps": 1e-5}, {"weight": (p + "norm2.weight",)})
-            layers.append(LayerSpec(mixer, ffn, n1, n2))
+            layers.append(LayerSpec.pre_norm(mixer, ffn, n1, n2))
         schedule = tuple(LayerCall(i, i) for i in range(len(layers)))
         return ModelSpec("ToyRoutedForCausalLM", H, V,
                          PartSpec("token_embedding", {"vocab_size": V, "hidden_size": H},
@@ -370,3 +370,206 @@ def test_toy_routing_and_position_parts_step_through_the_engine():
         got = eu.run_schedule(runner, prompts, schedule)
         for g, e in zip(got, expect):
             assert eu.rel_err(g, e) < 1e-4
+
+
+# ---------- another arrangement (four norms, two mixers), a mixer that pages ONE vector
+def sandwich_classes():
+    from zig_ai_amd.kernels import ops
+    from zig_ai_amd.parts import (Mixer, PagedNeed, StateNeed, TensorRule, register_arrangement,
+                                  register_mixer)
+
+    class LatentMemoryMixer(Mixer):
+        """Attention over one small vector per token: c[t] = x[t] Wd^T is all that is kept
+        (ONE plane of ``latent`` elements per token, in 32-bit whatever the run's type);
+        y[t] = softmax_j<=t(q[t] . c[j] / sqrt(latent)) c[j] Wu^T with q[t] = x[t] Wq^T."""
+        kind = "toy_latent_memory"
+        kernel_sources = ("gemm",)
+
+        @classmethod
+        def tensor_rules(cls, params):
+            H, r = int(params["width"]), int(params["latent"])
+            return {"down.weight": TensorRule(((r, H),)), "q.weight": TensorRule(((r, H),)),
+                    "up.weight": TensorRule(((H, r),))}
+
+        @classmethod
+        def cache_need(cls, params):
+            return PagedNeed(((1, int(params["latent"])),), dtype=torch.float32)
+
+        def __init__(self, params, tensors, runtime):
+            super().__init__(params, tensors, runtime)
+            self.latent = int(params["latent"])
+            self.down, self.q, self.up = (tensors[k + ".weight"] for k in ("down", "q", "up"))
+
+        def forward(self, x, step, cache):
+            (plane,) = cache.planes                       # [pages, 1, page_size, latent]
+            assert plane.dtype == torch.float32 and cache.kv is None
+            page_size = plane.shape[2]
+            c = ops.linear(x, self.down, out_dtype=torch.float32)
+            q = ops.linear(x, self.q, out_dtype=torch.float32)
+            place = step.slot_mapping[cache.group].long()
+            plane[place // page_size, 0, place % page_size] = c
+            out = torch.empty((x.shape[0], self.latent), dtype=torch.float32, device=x.device)
+            row = 0
+            table = step.block_tables[cache.group]
+            for s, (n, ctx) in enumerate(zip(step.seq_lens_host, step.ctx_lens_host)):
+                total = ctx + n
+                pages = table[s, : (total + page_size - 1) // page_size].long()
+                memory = plane[pages, 0].reshape(-1, self.latent)[:total]
+                scores = q[row:row + n] @ memory.T / self.latent ** 0.5
+                seen = torch.arange(total, device=x.device)[None, :] <= \
+                    (ctx + torch.arange(n, device=x.device))[:, None]
+                weights = torch.softmax(scores.masked_fill(~seen, float("-inf")), dim=-1)
+                out[row:row + n] = weights @ memory
+                row += n
+            return ops.linear(out.to(x.dtype), self.up)
+
+    class FadingGate(Mixer):
+        """A factor 1 / (1 + t / 8) for the request's t-th token: the count of tokens seen
+        is its state, one 32-bit INTEGER per request."""
+        kind = "toy_fading_gate"
+
+        @classmethod
+        def cache_need(cls, params):
+            return StateNeed((1,), dtype=torch.int32)
+
+        def forward(self, x, step, cache):
+            assert cache.state.dtype == torch.int32
+            factor = torch.empty((x.shape[0], 1), dtype=torch.float32, device=x.device)
+            row = 0
+            for n, slot in zip(step.seq_lens_host, step.slots_host):
+                seen = int(cache.state[slot, 0])
+                t = seen + torch.arange(n, device=x.device, dtype=torch.float32)
+                factor[row:row + n, 0] = 1.0 / (1.0 + t / 8.0)
+                cache.state[slot, 0] = seen + n
+                row += n
+            return factor
+
+    class SandwichBlock:
+        """Norms before AND after each of mixer and feed-forward, and a second mixer whose
+        output scales the first one's:
+            h = x + post1(mixer(pre1(x)) * gate(pre1(x)));  y = h + post2(ffn(pre2(h)))"""
+        kind = "toy_sandwich"
+        slots = {"pre_mixer_norm": "norm", "mixer": "mixer", "gate": "mixer",
+                 "post_mixer_norm": "norm", "pre_feed_forward_norm": "norm",
+                 "feed_forward": "feed_forward", "post_feed_forward_norm": "norm"}
+
+        def __init__(self, parts):
+            self.parts = dict(parts)
+
+        def forward(self, residual, pending, step, cache):
+            p = self.parts
+            n1 = p["pre_mixer_norm"].add_forward(residual, pending)
+            m = p["mixer"].forward(n1, step, cache["mixer"]).float() \
+                * p["gate"].forward(n1, step, cache["gate"])
+            residual += p["post_mixer_norm"].forward(m).float()
+            f = p["feed_forward"].forward(p["pre_feed_forward_norm"].forward(residual), step)
+            if f.dim() == 3:
+                f = f.sum(dim=0)
+            return residual, p["post_feed_forward_norm"].forward(f.float())
+
+    register_mixer(LatentMemoryMixer.kind, LatentMemoryMixer)
+    register_mixer(FadingGate.kind, FadingGate)
+    register_arrangement(SandwichBlock.kind, SandwichBlock)
+
+
+class SandwichConfig:
+    def __init__(self, data):
+        self.data = dict(data)
+
+    @classmethod
+    def from_dict(cls, data):
+        return cls(data)
+
+    def to_dict(self):
+        return dict(self.data)
+
+    def to_spec(self):
+        from zig_ai_amd.config.spec import LayerCall, LayerSpec, ModelSpec, PartSpec
+        d = self.data
+        H, V = d["width"], d["vocab_size"]
+
+        def norm(name):
+            return PartSpec("rms_norm", {"width": H, "eps": 1e-5}, {"weight": (name,)})
+
+        layers = []
+        for i in range(d["layers"]):
+            p = f"layers.{i}."
+            layers.append(LayerSpec({
+                "pre_mixer_norm": norm(p + "pre1.weight"),
+                "mixer": PartSpec("toy_latent_memory", {"width": H, "latent": d["latent"]},
+                                  {k + ".weight": (p + k + ".weight",) for k in ("down", "q", "up")}),
+                "gate": PartSpec("toy_fading_gate", {}),
+                "post_mixer_norm": norm(p + "post1.weight"),
+                "pre_feed_forward_norm": norm(p + "pre2.weight"),
+                "feed_forward": PartSpec("swiglu", {"hidden_size": H, "intermediate_size": d["ffn"]},
+                                         {k + ".weight": (p + "ffn." + k + ".weight",)
+                                          for k in ("gate", "up", "down")}),
+                "post_feed_forward_norm": norm(p + "post2.weight"),
+            }, "toy_sandwich"))
+        return ModelSpec("ToySandwichForCausalLM", H, V,
+                         PartSpec("token_embedding", {"vocab_size": V, "hidden_size": H},
+                                  {"weight": ("embed.weight",)}),
+                         tuple(layers), tuple(LayerCall(i, i) for i in range(d["layers"])),
+                         norm("norm.weight"),
+                         PartSpec("linear_head", {"vocab_size": V, "hidden_size": H, "tied": True}, {}))
+
+
+SANDWICH = {"architectures": ["ToySandwichForCausalLM"], "width": 56, "vocab_size": 91, "ffn": 80,
+            "latent": 24, "layers": 3}
+
+
+def sandwich_oracle(folder, tokens):
+    from safetensors.torch import load_file
+    w = {k: v.double() for k, v in load_file(folder + "/model.safetensors").items()}
+    d = SANDWICH
+    T, r = len(tokens), d["latent"]
+    x = w["embed.weight"][torch.tensor(tokens)]
+    factor = 1.0 / (1.0 + torch.arange(T, dtype=torch.float64) / 8.0)
+    for i in range(d["layers"]):
+        p = f"layers.{i}."
+        n1 = plain.rms_norm(x, w[p + "pre1.weight"], 1e-5)
+        c, q = n1 @ w[p + "down.weight"].T, n1 @ w[p + "q.weight"].T
+        scores = (q @ c.T / r ** 0.5).masked_fill(torch.ones(T, T).triu(1).bool(), float("-inf"))
+        m = (torch.softmax(scores, dim=-1) @ c) @ w[p + "up.weight"].T * factor[:, None]
+        h = x + plain.rms_norm(m, w[p + "post1.weight"], 1e-5)
+        f = plain.swiglu_ffn(plain.rms_norm(h, w[p + "pre2.weight"], 1e-5), w[p + "ffn.gate.weight"],
+                             w[p + "ffn.up.weight"], w[p + "ffn.down.weight"])
+        x = h + plain.rms_norm(f, w[p + "post2.weight"], 1e-5)
+    return plain.rms_norm(x, w["norm.weight"], 1e-5) @ w["embed.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_another_arrangement_and_a_mixer_that_pages_one_vector(dtype):
+    """A block of another shape (norms before and after both parts: four norms; two
+    mixers) and a mixer that keeps ONE vector per token in pages, of a storage type of
+    its own, beside a mixer whose state is an integer: all defined here, registered from
+    outside, built from a model folder by the framework's loader and random model writer
+    (which ask the arrangement for its parts' names), and stepped whole, in portions and
+    mixed, with pages used again."""
+    from zig_ai_amd.config import register_architecture
+    from zig_ai_amd.engine import DecoderModel, ModelRunner
+    sandwich_classes()
+    register_architecture("ToySandwichForCausalLM", SandwichConfig)
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    folder = eu.model_folder(SANDWICH, 17, store, std=0.2, norm_init="around_one", role_std={"norm": 0.2})
+    model = DecoderModel.from_folder(folder, dtype)
+    assert not model.graph_safe
+    # per layer a paged entry and a state entry, named (cache, part)
+    assert len(model.cache_needs) == 6 and (0, "mixer") in model.cache_needs
+    lengths = [37, 5, 22, 14]
+    prompts = [eu.random_tokens(n, 91, 800 + n) for n in lengths]
+    expect = [sandwich_oracle(folder, p) for p in prompts]
+    tol = 1e-4 if dtype == "float32" else 4e-2
+    for schedule in (eu.whole(lengths), eu.changing_portions(lengths, 4),
+                     eu.mixed(lengths, seed=6, max_live=2, decode_tail=6)):
+        pages = eu.peak_tokens(lengths, schedule, round_to=4) // 4
+        runner = ModelRunner(model, page_size=4, num_pages=pages, num_slots=2)
+        group = runner.cache.groups[0]
+        assert group.dtype == torch.float32 and group.kv is None
+        assert group.elements_per_page() == 4 * 24 and len(group.cache_ids) == 3
+        got = eu.run_schedule(runner, prompts, schedule)
+        for g, e in zip(got, expect):
+            assert eu.rel_err(g, e) < tol
+        stats = runner.cache.stats()
+        assert stats["requests"] == 0 and stats["slots_high_water"] <= 2
+    assert stats["pages_reused"] > 0

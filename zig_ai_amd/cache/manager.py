@@ -3,7 +3,8 @@ with one block table per request and group, and one slot of fixed-size state
 per request for the mixers that carry state.
 
 Groups.  Mixers declare what they need (``PagedNeed`` or ``StateNeed``).  Paged
-needs with the same (kv heads, head size, window) form a *group*: its layers
+needs that are equal (the same planes per token, window and storage type) form a
+*group*: its layers
 share one block table per request (page ``p`` names the same place in every
 layer's plane of the group's tensor) and the group has a pool of pages of its
 own, because a group that keeps every key and a group that keeps a window of
@@ -17,10 +18,14 @@ Life of a request: ``admit`` (takes a slot, zeroes its state), then per step
 tokens are in the cache; pages wholly behind a group's window go back to the
 pool), finally ``release`` (every page and the slot go back).
 
-Device memory: per group ``kv[layer, page, 2, kv_head, page_size * head_dim]``,
-where a page's keys lie as ``[offset][head_dim]`` and its values turned round as
-``[head_dim][offset]`` (the order the attention kernels' second product reads);
-state ``slots[slot, floats]`` in 32-bit with one view per state entry.
+Device memory: per group one tensor ``[layer, page, elements of a page]``; a page
+holds the group's planes one after the other, plane ``p`` as ``[heads_p, page_size,
+width_p]``, and every layer sees it as one view per plane.  For keys and values (two
+planes of one size) that is the tensor ``kv[page, 2, kv_head, page_size, head_dim]``
+the attention kernels take, where a page's keys lie as ``[offset][head_dim]`` and
+the kernels store its values turned round as ``[head_dim][offset]`` (the order
+their second product reads).  State: ``slots[slot, bytes]`` with one typed view per
+state entry (32-bit floats unless the need says otherwise).
 """
 
 from __future__ import annotations
@@ -44,17 +49,43 @@ FREED = -1   # block-table entry of a page that was given back (behind the windo
 class PagedGroup:
     index: int
     need: PagedNeed
-    cache_ids: List[int]
+    cache_ids: List[Hashable]
     pool: Pool
     page_size: int
-    kv: Optional[torch.Tensor] = None      # [layers, pages, 2, kv_heads, page_size, head_dim]
+    dtype: torch.dtype = torch.bfloat16
+    memory: Optional[torch.Tensor] = None      # [layers, pages, elements of a page]
 
-    def layer_of(self, cache_id: int) -> int:
+    def layer_of(self, cache_id) -> int:
         return self.cache_ids.index(cache_id)
 
-    def bytes_per_page(self, element_size: int) -> int:
-        n = self.need
-        return len(self.cache_ids) * 2 * n.num_kv_heads * self.page_size * n.head_dim * element_size
+    def elements_per_page(self) -> int:
+        return self.need.elements_per_token() * self.page_size
+
+    def bytes_per_page(self, element_size: Optional[int] = None) -> int:
+        size = torch.empty((), dtype=self.dtype).element_size() if element_size is None else element_size
+        return len(self.cache_ids) * self.elements_per_page() * size
+
+    @property
+    def kv(self) -> Optional[torch.Tensor]:
+        """Keys and values of every layer, ``[layers, pages, 2, kv_heads, page_size,
+        head_dim]``; only for a group of two equal planes."""
+        if self.memory is None or not self.need.is_kv:
+            return None
+        heads, width = self.need.planes[0]
+        return self.memory.view(len(self.cache_ids), self.pool.size, 2, heads, self.page_size, width)
+
+    def plane_views(self, layer: int) -> List[torch.Tensor]:
+        """One view ``[pages, heads, page_size, width]`` per plane of ``layer``."""
+        if self.memory is None:
+            return []
+        mem = self.memory[layer]
+        per_page = self.elements_per_page()
+        out, offset = [], 0
+        for heads, width in self.need.planes:
+            n = heads * self.page_size * width
+            out.append(mem[:, offset:offset + n].unflatten(1, (heads, self.page_size, width)))
+            offset += n
+        return out
 
 
 @dataclass
@@ -62,7 +93,8 @@ class CacheView:
     """What a mixer sees of the cache for one entry of the run order."""
     kind: str                      # "paged" | "state" | "none"
     group: int = -1                # paged: index of the group (selects table and slots)
-    kv: Optional[torch.Tensor] = None        # paged: [pages, 2, kv_heads, page_size, head_dim]
+    kv: Optional[torch.Tensor] = None        # paged, keys and values: [pages, 2, kv_heads, page_size, head_dim]
+    planes: Optional[List[torch.Tensor]] = None   # paged: per plane [pages, heads, page_size, width]
     state: Optional[torch.Tensor] = None     # state: [slots, *shape]
     writes: bool = True
 
@@ -71,12 +103,12 @@ class CacheManager:
     """Groups, tables and slots are kept by the host library; this class owns the
     device memory, names the requests and translates failures into exceptions."""
 
-    def __init__(self, needs: Mapping[int, object], page_size: int, num_pages, num_slots: int,
+    def __init__(self, needs: Mapping[Hashable, object], page_size: int, num_pages, num_slots: int,
                  device: Optional[torch.device] = None, dtype: torch.dtype = torch.bfloat16,
                  allocate: bool = True, scatter_pages: bool = False):
         """``needs``: cache id -> PagedNeed | StateNeed | None.  ``num_pages``: an int
-        (every group gets that many) or a mapping from group key
-        ``(kv_heads, head_dim, window)`` to a count.  ``scatter_pages``: fresh pools hand
+        (every group gets that many) or a mapping from the group's ``PagedNeed`` to a
+        count.  ``scatter_pages``: fresh pools hand
         their pages out in a fixed pseudo-random order rather than 0, 1, 2 ..., so that
         requests filled one after the other do not lie a constant distance apart."""
         if page_size <= 0:
@@ -87,32 +119,33 @@ class CacheManager:
         self._lib = host.lib()
         self.handles = host.Handles()
         self._pinned: set = set()      # names a scheduler still knows: their handles are kept
-        self._group_of: Dict[int, int] = {}
-        by_key: Dict[Tuple[int, int, int], int] = {}
+        self._group_of: Dict[Hashable, int] = {}
+        by_key: Dict[PagedNeed, int] = {}
         group_needs: List[PagedNeed] = []
-        group_ids: List[List[int]] = []
+        group_ids: List[List[Hashable]] = []
         group_pages: List[int] = []
-        state_entries: List[Tuple[int, StateNeed]] = []
-        for cid in sorted(needs):
-            need = needs[cid]
+        state_entries: List[Tuple[Hashable, StateNeed]] = []
+        for cid, need in needs.items():
             if need is None:
                 continue
             if isinstance(need, PagedNeed):
-                key = (need.num_kv_heads, need.head_dim, need.window)
-                if key not in by_key:
-                    count = num_pages[key] if isinstance(num_pages, Mapping) else int(num_pages)
+                if not need.planes or any(h <= 0 or w <= 0 for h, w in need.planes):
+                    raise ValueError(f"cache entry {cid!r}: a paged need has planes of positive "
+                                     f"sizes, got {need.planes!r}")
+                if need not in by_key:
+                    count = num_pages[need] if isinstance(num_pages, Mapping) else int(num_pages)
                     if count < 0:
                         raise ValueError(f"a pool cannot have {count} pages")
-                    by_key[key] = len(group_needs)
+                    by_key[need] = len(group_needs)
                     group_needs.append(need)
                     group_ids.append([])
                     group_pages.append(count)
-                group_ids[by_key[key]].append(cid)
-                self._group_of[cid] = by_key[key]
+                group_ids[by_key[need]].append(cid)
+                self._group_of[cid] = by_key[need]
             elif isinstance(need, StateNeed):
                 state_entries.append((cid, need))
             else:
-                raise TypeError(f"cache need of entry {cid} is {need!r}")
+                raise TypeError(f"cache need of entry {cid!r} is {need!r}")
         if num_slots < 0:
             raise ValueError(f"a pool cannot have {num_slots} slots")
         G = len(group_needs)
@@ -125,29 +158,30 @@ class CacheManager:
         self.groups: List[PagedGroup] = [
             PagedGroup(g, group_needs[g], group_ids[g],
                        Pool(0, "page", _attach=(self._lib.za_cache_pool(self._ptr, g), self.handles)),
-                       page_size)
+                       page_size, group_needs[g].dtype or dtype)
             for g in range(G)]
         self.slots = Pool(0, "slot", _attach=(self._lib.za_cache_pool(self._ptr, -1), self.handles))
-        self._state_layout: Dict[int, Tuple[int, Tuple[int, ...]]] = {}
+        # a slot is a row of bytes; every state entry has its own 16-byte aligned window of it
+        self._state_layout: Dict[Hashable, Tuple[int, int, Tuple[int, ...], torch.dtype]] = {}
         offset = 0
         for cid, need in state_entries:
             n = 1
             for s in need.shape:
                 n *= int(s)
-            self._state_layout[cid] = (offset, tuple(int(s) for s in need.shape))
-            offset += n
-        self.floats_per_slot = offset
+            nbytes = n * torch.empty((), dtype=need.dtype).element_size()
+            self._state_layout[cid] = (offset, nbytes, tuple(int(s) for s in need.shape), need.dtype)
+            offset += (nbytes + 15) // 16 * 16
+        self.bytes_per_slot = offset
         self.slot_memory: Optional[torch.Tensor] = None
         if allocate:
             if device is None:
                 raise ValueError("a device is needed to allocate the cache")
             for grp in self.groups:
-                n = grp.need
-                grp.kv = torch.zeros((len(grp.cache_ids), grp.pool.size, 2, n.num_kv_heads,
-                                      page_size, n.head_dim), dtype=dtype, device=device)
-            if self.floats_per_slot:
-                self.slot_memory = torch.zeros((num_slots, self.floats_per_slot),
-                                               dtype=torch.float32, device=device)
+                grp.memory = torch.zeros((len(grp.cache_ids), grp.pool.size, grp.elements_per_page()),
+                                         dtype=grp.dtype, device=device)
+            if self.bytes_per_slot:
+                self.slot_memory = torch.zeros((num_slots, self.bytes_per_slot),
+                                               dtype=torch.uint8, device=device)
         self._n_groups = G
         self._scratch = (ctypes.c_int * max(G, 1))()
 
@@ -162,31 +196,32 @@ class CacheManager:
         return self._ptr
 
     @staticmethod
-    def bytes_per_page_index(needs: Mapping[int, object], page_size: int, element_size: int) -> int:
+    def bytes_per_page_index(needs: Mapping[Hashable, object], page_size: int,
+                             run_dtype: torch.dtype) -> int:
         """Device bytes that ONE more page in every group costs (all groups are given
         the same number of pages when ``num_pages`` is a single number)."""
         total = 0
         for need in needs.values():
             if isinstance(need, PagedNeed):
-                total += 2 * need.num_kv_heads * page_size * need.head_dim * element_size
+                size = torch.empty((), dtype=need.dtype or run_dtype).element_size()
+                total += need.elements_per_token() * page_size * size
         return total
 
     # ------------------------------------------------------------------ views
-    def view(self, cache_id: int, writes: bool = True) -> CacheView:
+    def view(self, cache_id, writes: bool = True) -> CacheView:
         if cache_id in self._group_of:
             grp = self.groups[self._group_of[cache_id]]
-            kv = grp.kv[grp.layer_of(cache_id)] if grp.kv is not None else None
-            return CacheView("paged", group=grp.index, kv=kv, writes=writes)
+            layer = grp.layer_of(cache_id)
+            kv = grp.kv[layer] if grp.kv is not None else None
+            return CacheView("paged", group=grp.index, kv=kv, planes=grp.plane_views(layer),
+                             writes=writes)
         if cache_id in self._state_layout:
-            off, shape = self._state_layout[cache_id]
+            off, nbytes, shape, dtype = self._state_layout[cache_id]
             st = None
             if self.slot_memory is not None:
-                n = 1
-                for s in shape:
-                    n *= s
                 # A window of every slot's row: contiguous within a slot, slots spaced by
                 # the whole row.
-                st = self.slot_memory[:, off:off + n].unflatten(1, shape)
+                st = self.slot_memory[:, off:off + nbytes].view(dtype).unflatten(1, shape)
             return CacheView("state", state=st, writes=writes)
         return CacheView("none", writes=writes)
 

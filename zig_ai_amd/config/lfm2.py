@@ -239,7 +239,7 @@ class Lfm2Config:
                                                    g + "attn_norm.weight")})
             ffn_norm = PartSpec("rms_norm", {"width": H, "eps": self.norm_eps},
                                 {"weight": names(p + "ffn_norm.weight", g + "ffn_norm.weight")})
-            layers.append(LayerSpec(mixer, ffn, mixer_norm, ffn_norm, "pre_norm_residual"))
+            layers.append(LayerSpec.pre_norm(mixer, ffn, mixer_norm, ffn_norm))
 
         embedding = PartSpec("token_embedding", {"vocab_size": self.vocab_size, "hidden_size": H},
                              {"weight": ("model.embed_tokens.weight", "token_embd.weight")})

@@ -38,14 +38,28 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """A decoder block: two norms, a token mixer and a feed-forward, and the
-    name of the arrangement that wires them together."""
+    """A decoder block: its parts by name, and the name of the arrangement that wires
+    them together.  The arrangement says which names it has and of which family each
+    is (``slots``); the usual block has a mixer, a feed-forward and a norm before each
+    (``LayerSpec.pre_norm``), another may have four norms, no feed-forward, or two
+    mixers."""
 
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
+    parts: Mapping[str, PartSpec]
     arrangement: str = "pre_norm_residual"
+
+    @classmethod
+    def pre_norm(cls, mixer: PartSpec, feed_forward: PartSpec, mixer_norm: PartSpec,
+                 feed_forward_norm: PartSpec, arrangement: str = "pre_norm_residual") -> "LayerSpec":
+        return cls({"mixer_norm": mixer_norm, "mixer": mixer,
+                    "feed_forward_norm": feed_forward_norm, "feed_forward": feed_forward},
+                   arrangement)
+
+    def __getattr__(self, name: str) -> PartSpec:
+        # a part by its name, as an attribute: layer.mixer, layer.feed_forward_norm
+        parts = object.__getattribute__(self, "parts")
+        if name in parts:
+            return parts[name]
+        raise AttributeError(name)
 
 
 @dataclass(frozen=True)

@@ -53,12 +53,17 @@ class Engine:
         limit = max_model_len or self.model.spec.max_position or 8192
         if max_model_len is None:
             limit = min(limit, 8192)
+        if 0 < self.model.spec.max_position < limit:
+            # positions beyond the model's own limit would stop a step in the middle of a
+            # call of generate(), and every request of the call with it
+            raise ValueError(f"max_model_len {limit} exceeds the model's max_position_embeddings "
+                             f"{self.model.spec.max_position}")
         self.max_model_len = limit
         if num_pages is None:
             per_request = (limit + page_size - 1) // page_size
             num_pages = max_num_seqs * per_request
-            element = 4 if self.model.runtime.dtype == torch.float32 else 2
-            per_page = CacheManager.bytes_per_page_index(self.model.cache_needs, page_size, element)
+            per_page = CacheManager.bytes_per_page_index(self.model.cache_needs, page_size,
+                                                         self.model.runtime.dtype)
             if per_page:
                 free, _ = torch.cuda.mem_get_info(self.model.runtime.device)
                 fit = int(free * memory_fraction) // per_page

@@ -37,6 +37,20 @@ def require_gpu() -> torch.device:
     return torch.device("cuda", torch.cuda.current_device())
 
 
+def arrangement_slots(arrangement, layer) -> Dict[str, str]:
+    """The names and families of the parts an arrangement wires (its ``slots``), checked
+    against the parts the layer's description gives."""
+    slots = dict(getattr(arrangement, "slots", None) or {})
+    if not slots:
+        raise ValueError(f"arrangement {layer.arrangement!r} declares no parts (``slots``)")
+    missing = [n for n in slots if n not in layer.parts]
+    unknown = [n for n in layer.parts if n not in slots]
+    if missing or unknown:
+        raise ValueError(f"arrangement {layer.arrangement!r} wires {sorted(slots)}; the layer "
+                         f"lacks {missing} and has {unknown} besides")
+    return slots
+
+
 class DecoderModel:
     def __init__(self, spec: ModelSpec, tensors: Mapping[Any, Mapping[str, torch.Tensor]],
                  runtime: parts.Runtime):
@@ -55,16 +69,16 @@ class DecoderModel:
         self.embedding = make("embedding", spec.embedding, ("embedding",))
         note(self.embedding)
         self.blocks = []
-        self.mixer_classes = []
+        self.mixer_slots: List[List[str]] = []      # per layer: the names of its mixers
         for i, layer in enumerate(spec.layers):
-            mixer_norm = make("norm", layer.mixer_norm, ("layer", i, "mixer_norm"))
-            mixer = make("mixer", layer.mixer, ("layer", i, "mixer"))
-            ffn_norm = make("norm", layer.feed_forward_norm, ("layer", i, "feed_forward_norm"))
-            ffn = make("feed_forward", layer.feed_forward, ("layer", i, "feed_forward"))
-            for p in (mixer_norm, mixer, ffn_norm, ffn):
-                note(p)
             arrangement = parts.lookup("arrangement", layer.arrangement)
-            self.blocks.append(arrangement(mixer_norm, mixer, ffn_norm, ffn))
+            slots = arrangement_slots(arrangement, layer)
+            built = {name: make(family, layer.parts[name], ("layer", i, name))
+                     for name, family in slots.items()}
+            for p in built.values():
+                note(p)
+            self.blocks.append(arrangement(built))
+            self.mixer_slots.append([n for n, family in slots.items() if family == "mixer"])
         self.final_norm = make("norm", spec.final_norm, ("final_norm",))
         self.head = make("head", spec.lm_head, ("lm_head",))
         note(self.final_norm)
@@ -74,28 +88,33 @@ class DecoderModel:
         if getattr(self.head, "weight", None) is None:
             raise ValueError("the output head has no weight")
 
+        # Cache entries: a run-order entry's mixer uses the entry named by ``call.cache``;
+        # a block with several mixers has one entry per mixer, ``(call.cache, name)``.
         self.schedule: Sequence[LayerCall] = spec.resolved_schedule()
-        self.cache_needs: Dict[int, object] = {}
+        self.cache_needs: Dict[Any, object] = {}
         for call in self.schedule:
             layer = spec.layers[call.layer]
-            need = parts.lookup("mixer", layer.mixer.kind).cache_need(layer.mixer.params)
-            if call.cache in self.cache_needs and self.cache_needs[call.cache] != need:
-                raise ValueError(
-                    f"run-order entries sharing cache {call.cache} need different caches: "
-                    f"{self.cache_needs[call.cache]} and {need}")
-            self.cache_needs[call.cache] = need
-        writers = {c.cache for c in self.schedule if c.writes_cache}
+            for key, name in self.cache_keys(call):
+                part = layer.parts[name]
+                need = parts.lookup("mixer", part.kind).cache_need(part.params)
+                if key in self.cache_needs and self.cache_needs[key] != need:
+                    raise ValueError(
+                        f"run-order entries sharing cache {key} need different caches: "
+                        f"{self.cache_needs[key]} and {need}")
+                self.cache_needs[key] = need
+        writers = {key for c in self.schedule if c.writes_cache for key, _ in self.cache_keys(c)}
         for call in self.schedule:
-            if self.cache_needs[call.cache] is not None and call.cache not in writers:
-                raise ValueError(f"cache {call.cache} is read but no run-order entry writes it")
+            for key, _ in self.cache_keys(call):
+                if self.cache_needs[key] is not None and key not in writers:
+                    raise ValueError(f"cache {key} is read but no run-order entry writes it")
+        every = [self.embedding, self.final_norm, self.head]
+        for b in self.blocks:
+            every += list(b.parts.values())
         self.item_granularities = sorted({
-            g for b in self.blocks for g in getattr(b.mixer, "item_granularities", ())})
+            g for p in every for g in getattr(p, "item_granularities", ())})
         self.kernel_sources = sorted(sources)
         # A step may be recorded into a HIP graph only if no part looks at the step's
         # numbers on the host while it runs.
-        every = [self.embedding, self.final_norm, self.head]
-        for b in self.blocks:
-            every += [b.mixer_norm, b.mixer, b.feed_forward_norm, b.feed_forward]
         self.graph_safe = all(getattr(p, "graph_safe", False) for p in every)
         # Compile what this model's parts use (and the host library), together, before
         # the first step.
@@ -156,9 +175,25 @@ class DecoderModel:
                             device=self.runtime.device, dtype=self.runtime.dtype,
                             scatter_pages=scatter_pages)
 
-    def cache_views(self, cache: CacheManager) -> List[CacheView]:
-        """One view per run-order entry."""
-        return [cache.view(call.cache, call.writes_cache) for call in self.schedule]
+    def cache_keys(self, call: LayerCall):
+        """``[(cache entry, mixer's name)]`` of one run-order entry."""
+        names = self.mixer_slots[call.layer]
+        if len(names) == 1:
+            return [(call.cache, names[0])]
+        return [((call.cache, name), name) for name in names]
+
+    def cache_views(self, cache: CacheManager) -> List[Any]:
+        """Per run-order entry what its block's ``forward`` receives as ``cache``: the
+        mixer's view, or for a block with several mixers (or none) a dictionary from
+        the mixers' names to their views."""
+        out = []
+        for call in self.schedule:
+            keys = self.cache_keys(call)
+            if len(keys) == 1 and keys[0][0] == call.cache:
+                out.append(cache.view(call.cache, call.writes_cache))
+            else:
+                out.append({name: cache.view(key, call.writes_cache) for key, name in keys})
+        return out
 
     # ------------------------------------------------------------------ forward
     def forward(self, step: StepContext, views: Sequence[CacheView],

@@ -79,8 +79,8 @@ class GroupedQueryAttention(Mixer):
 
     @classmethod
     def cache_need(cls, params: Mapping[str, Any]):
-        return PagedNeed(int(params["num_kv_heads"]), int(params["head_dim"]),
-                         int(params.get("window") or 0))
+        return PagedNeed.kv(int(params["num_kv_heads"]), int(params["head_dim"]),
+                            int(params.get("window") or 0))
 
     def __init__(self, params, tensors, runtime: Runtime):
         super().__init__(params, tensors, runtime)

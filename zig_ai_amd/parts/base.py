@@ -10,7 +10,8 @@ never learns which model it is in.  Five families exist:
                      partial sums that the following norm adds up)
   norm               ``forward(x) -> y`` and ``add_forward(residual, delta) -> y``
   position encoding  used by mixers: a rotation table, or ``apply(q, k, positions)``
-  arrangement        wires two norms, a mixer and a feed-forward into a block
+  arrangement        wires a block's parts (it declares their names and families;
+                     two norms, a mixer and a feed-forward in the usual block)
 
 plus the embedding and the output head.  All ``forward`` functions take packed
 token rows ``[T, width]``: the tokens of every request in the step, one after
@@ -47,20 +48,41 @@ class TensorRule:
 # ---------------------------------------------------------------- cache needs
 @dataclass(frozen=True)
 class PagedNeed:
-    """Keys and values per token: ``num_kv_heads * head_dim`` of each.  With
-    ``window > 0`` only the last ``window`` positions are ever read, so older
-    pages can be given back."""
+    """What a mixer keeps per token, in pages: one or more *planes*, each ``heads``
+    vectors of ``width`` elements per token.  Keys and values are two planes of
+    ``(num_kv_heads, head_dim)`` (``PagedNeed.kv``); a mixer that keeps one latent
+    vector per token has one plane ``(1, width)``; planes may differ in size.  With
+    ``window > 0`` only the last ``window`` positions are ever read, so older pages
+    can be given back.  ``dtype``: what the planes store (``None``: the run's storage
+    type)."""
 
-    num_kv_heads: int
-    head_dim: int
+    planes: Tuple[Tuple[int, int], ...]
     window: int = 0
+    dtype: Optional[torch.dtype] = None
+
+    @classmethod
+    def kv(cls, num_kv_heads: int, head_dim: int, window: int = 0,
+           dtype: Optional[torch.dtype] = None) -> "PagedNeed":
+        plane = (int(num_kv_heads), int(head_dim))
+        return cls((plane, plane), int(window), dtype)
+
+    @property
+    def is_kv(self) -> bool:
+        """Two planes of the same size: keys and values, which the attention kernels
+        read as one tensor ``[pages, 2, heads, page_size, width]``."""
+        return len(self.planes) == 2 and self.planes[0] == self.planes[1]
+
+    def elements_per_token(self) -> int:
+        return sum(h * w for h, w in self.planes)
 
 
 @dataclass(frozen=True)
 class StateNeed:
-    """Per-request state of fixed size (32-bit floats), zero for a new request."""
+    """Per-request state of fixed size, zero for a new request; 32-bit floats unless
+    ``dtype`` says otherwise."""
 
     shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
 
 
 # ------------------------------------------------------------------- runtime
@@ -101,7 +123,9 @@ class Mixer(Part):
     # ``Norm.deferred`` returned (a norm that has not run yet, which the kernels of
     # ``ops.linear`` / ``ops.linear_swiglu`` can run themselves), and a keyword
     # ``stream``: the 32-bit residual stream, to which it may add its result itself;
-    # it then returns ``None``.
+    # it then returns ``None``.  What is handed over IS the stream (a norm that has not
+    # run reads its rows when the first projection runs): a part must be done with ``x``
+    # before it adds anything to ``stream``, or the norm would see the sum.
     takes_stream = False
 
     @classmethod

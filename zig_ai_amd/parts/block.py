@@ -1,4 +1,6 @@
-"""Arrangements: how two norms, a mixer and a feed-forward form a block.
+"""Arrangements: how a block's parts are wired.  An arrangement declares its parts
+(``slots``: name -> family; the model builds each from the layer's ``PartSpec`` of that
+name and hands them over as a dictionary) and runs them in ``forward``.
 
 ``pre_norm_residual`` is the reference's decoder block
 (/root/reference/src/transformer/hybrid_layer.zig:366-492):
@@ -24,12 +26,15 @@ from .base import register_arrangement
 
 class PreNormResidualBlock:
     kind = "pre_norm_residual"
+    slots = {"mixer_norm": "norm", "mixer": "mixer", "feed_forward_norm": "norm",
+             "feed_forward": "feed_forward"}
 
-    def __init__(self, mixer_norm, mixer, feed_forward_norm, feed_forward):
-        self.mixer_norm = mixer_norm
-        self.mixer = mixer
-        self.feed_forward_norm = feed_forward_norm
-        self.feed_forward = feed_forward
+    def __init__(self, parts):
+        self.parts = dict(parts)
+        self.mixer_norm = parts["mixer_norm"]
+        self.mixer = parts["mixer"]
+        self.feed_forward_norm = parts["feed_forward_norm"]
+        self.feed_forward = parts["feed_forward"]
 
     def forward(self, residual: torch.Tensor, pending: Optional[torch.Tensor], step,
                 cache) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:

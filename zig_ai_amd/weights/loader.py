@@ -52,13 +52,6 @@ class Expected:
     rule: parts_base.TensorRule
 
 
-_FAMILY_OF_SLOT = {
-    "mixer": "mixer", "feed_forward": "feed_forward", "mixer_norm": "norm",
-    "feed_forward_norm": "norm", "embedding": "embedding", "final_norm": "norm",
-    "lm_head": "head",
-}
-
-
 def _part_expectations(owner: Owner, family: str, part: PartSpec) -> Iterator[Expected]:
     cls = parts_base.lookup(family, part.kind)
     rules = cls.tensor_rules(part.params)
@@ -80,9 +73,13 @@ def expected_tensors(spec: ModelSpec) -> List[Expected]:
     out: List[Expected] = []
     out += _part_expectations(("embedding",), "embedding", spec.embedding)
     for i, layer in enumerate(spec.layers):
-        for slot in ("mixer_norm", "mixer", "feed_forward_norm", "feed_forward"):
-            out += _part_expectations(("layer", i, slot), _FAMILY_OF_SLOT[slot],
-                                      getattr(layer, slot))
+        # the arrangement names the layer's parts and says of which family each is
+        slots = getattr(parts_base.lookup("arrangement", layer.arrangement), "slots", {})
+        for name, family in slots.items():
+            if name not in layer.parts:
+                raise KeyError(f"layer {i}: arrangement {layer.arrangement!r} wires a part "
+                               f"{name!r} that the layer's description does not give")
+            out += _part_expectations(("layer", i, name), family, layer.parts[name])
     out += _part_expectations(("final_norm",), "norm", spec.final_norm)
     out += _part_expectations(("lm_head",), "head", spec.lm_head)
     return out
