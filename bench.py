@@ -66,7 +66,7 @@ SHAPES = {
 }
 
 
-def serve(cfg, name, n_requests, new_tokens) -> int:
+def serve(cfg, name, n_requests, new_tokens, portion_graphs=False) -> int:
     """Requests with prompts of 128 to 2,048 tokens through the scheduler, the step
     function and the sampler (temperature 0.7), all admitted at once."""
     import random
@@ -83,7 +83,8 @@ def serve(cfg, name, n_requests, new_tokens) -> int:
     with tempfile.TemporaryDirectory(prefix="zigai_bench_") as folder:
         write_random_model(config_from_dict(cfg), folder, seed=0, dtype=torch.bfloat16)
         engine = Engine(folder, dtype="bfloat16", page_size=16, max_num_seqs=64,
-                        max_num_batched_tokens=4096, chunk_size=2048, max_model_len=4096)
+                        max_num_batched_tokens=4096, chunk_size=2048, max_model_len=4096,
+                        portion_graphs=portion_graphs)
         # warm-up: every kind of step once (more than 16 rows of logits among them),
         # so that no library loads its kernels inside the timed run
         engine.generate([p[:64] for p in prompts[:20]], max_new_tokens=4, temperature=0.7, seed=3,
@@ -156,6 +157,8 @@ def main() -> int:
     ap.add_argument("--new-tokens", type=int, default=256, help="new tokens per request of "
                     "--workload serve")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points")
+    ap.add_argument("--portion-graphs", action="store_true",
+                    help="--workload serve: also record steps with prompt portions")
     ap.add_argument("--phase", choices=["all", "prefill", "decode"], default="all",
                     help="measure only one phase (for profiling); the JSON line then holds "
                          "only that phase")
@@ -171,7 +174,7 @@ def main() -> int:
     torch.cuda.set_device(0)
     cfg = dict(SHAPES[args.shape])
     if args.workload == "serve":
-        return serve(cfg, args.shape.upper(), args.requests, args.new_tokens)
+        return serve(cfg, args.shape.upper(), args.requests, args.new_tokens, args.portion_graphs)
     full_layers = cfg["num_hidden_layers"]
     if args.layers is not None and args.layers < full_layers:
         cfg["num_hidden_layers"] = args.layers

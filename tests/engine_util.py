@@ -247,7 +247,7 @@ def run_schedule(runner, prompts, schedule, wants=None, forms=None, streams=None
         for i in list(streams):
             streams[i] = [{name: torch.cat(parts) if isinstance(parts, list) else parts
                            for name, parts in named.items()} for named in streams[i]]
-    return [torch.cat(got[i]) for i in range(len(prompts))]
+    return [torch.cat(got[i]) if got[i] else torch.empty((0, 0)) for i in range(len(prompts))]
 
 
 def layer_errors(oracle, prompt, taps, rounding, logits, rows=None):

@@ -161,14 +161,16 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
         s = s.masked_fill(mask, float("-inf"))
         if round_probabilities:
             # A bfloat16 run on the matrix cores rounds the unnormalised probabilities for
-            # the second product and divides by their unrounded sum.  It takes them
+            # the second product and divides by the sum of the rounded values (the weights
+            # that reach the values then add up to one).  It takes them
             # relative to the row's maximum rounded up to a whole number on the base-2
             # scale, p = 2^(s log2(e) - ceil(max)): the same softmax (the common factor
             # cancels), and the one form in which the rounded values do not depend on the
             # order in which the keys are visited.
             t = s * math.log2(math.e)
             p = torch.exp2(t - torch.ceil(t.max(dim=-1, keepdim=True).values))
-            out[:, h, :] = (bf(p) @ v[:, g, :]) / p.sum(dim=-1, keepdim=True)
+            p = bf(p)
+            out[:, h, :] = (p @ v[:, g, :]) / p.sum(dim=-1, keepdim=True)
         else:
             p = torch.exp(s - s.max(dim=-1, keepdim=True).values)
             out[:, h, :] = (p / p.sum(dim=-1, keepdim=True)) @ v[:, g, :]

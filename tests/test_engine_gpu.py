@@ -260,6 +260,40 @@ def test_graph_replays_between_other_work(dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prompt_portions_replayed_from_graphs(dtype):
+    """Prompts cut into portions of one size, as a serving loop cuts them: from the second
+    time a shape is seen the step is recorded, then replayed, also beside decoded tokens of
+    another request and with other requests' steps and synchronisations between the
+    replays.  Every replay gives what the same step gives when it is issued kernel by
+    kernel, and both give the plain implementation's logits."""
+    from zig_ai_amd.engine import ModelRunner
+    model, expect, prompts = setup("D", dtype)          # 150, 9, 66 and 40 tokens
+    lengths = LENGTHS["D"]
+    schedule = []
+    for i, n in enumerate(lengths):                      # each alone, 32 tokens at a time
+        for a in range(0, n, 32):
+            schedule.append(([(i, a, min(n, a + 32))], [i] if a + 32 >= n else []))
+    # and two together: portions of 32 of one beside single tokens of the other
+    both = [([(0, 0, 32), (2, 0, 32)], [])]
+    for k in range(1, 4):
+        both.append(([(0, 32 * k, 32 * k + 32), (2, 31 + k, 32 + k)], []))
+    both.append(([(0, 128, 150), (2, 35, 66)], [0, 2]))
+    recorded = ModelRunner(model, page_size=8, num_pages=64, num_slots=4, portion_graphs=True)
+    eager = ModelRunner(model, page_size=8, num_pages=64, num_slots=4)
+    for sched, which in ((schedule, range(4)), (both, (0, 2)), (schedule, range(4))):
+        got = eu.run_schedule(recorded, prompts, sched)
+        same = eu.run_schedule(eager, prompts, sched)
+        for i in which:
+            assert eu.rel_err(got[i], expect[i]) < TOL[dtype]
+            assert eu.rel_err(got[i], same[i].double()) < SAME_STEPS[dtype]
+        torch.cuda.synchronize()
+    g = recorded.graphs
+    assert g.portion_captures >= 3 and g.portion_replays >= 12
+    assert eager.graphs.portion_replays == 0
+    recorded.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_first_tokens(dtype):
     """The very first positions: one token alone, two, three (shorter than the
     convolution), each as its own request."""

@@ -62,6 +62,9 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--no-graph", action="store_true",
                     help="launch decode steps kernel by kernel instead of replaying HIP graphs "
                          "(the reference's NOGRAPH)")
+    ap.add_argument("--portion-graphs", action="store_true",
+                    help="also record steps with prompt portions into HIP graphs, from the second "
+                         "time a shape (tokens per request, table width) is seen")
     ap.add_argument("--dump-logits", default=None, metavar="DIR",
                     help="write the logits every token is drawn from to DIR/<step>.f32, "
                          "[rows, vocab] little-endian 32-bit (the reference's DUMP_LOGITS)")
@@ -167,7 +170,8 @@ def run(args) -> int:
     engine = Engine(args.model, dtype=args.dtype, page_size=args.page_size,
                     num_pages=args.num_pages, max_num_seqs=args.max_num_seqs,
                     max_num_batched_tokens=args.batch_size, chunk_size=args.ubatch_size,
-                    max_model_len=args.max_model_len, use_graphs=not args.no_graph, reproducible=args.reproducible,
+                    max_model_len=args.max_model_len, use_graphs=not args.no_graph, portion_graphs=args.portion_graphs,
+                    reproducible=args.reproducible,
                     on_step=on_step if (args.dump_logits or args.verbose or args.profile) else None)
     load_s = time.perf_counter() - load_start
     start = time.perf_counter()

@@ -245,7 +245,10 @@ attention_combine_kernel(const float* __restrict__ part_acc, const float* __rest
 // eight light waves are faster.)  Per tile of 64 keys:
 //   S^T = K Q^T   (keys as the rows of the first operand, 16 query rows as columns; a
 //                  lane ends up with the scores of ONE query row for 16 keys)
-//   p   = 2^(S^T * scale * log2(e) - m)  in 32-bit, running maximum and sum per lane;
+//   p   = 2^(S^T * scale * log2(e) - m)  in 32-bit, running maximum per lane; p is rounded
+//                  to bfloat16 for the second product, and the sum that normalises the
+//                  result is the sum of those rounded values (so the weights that reach
+//                  the values add up to one), taken by the matrix core as well;
 //                  m is the running maximum ROUNDED UP TO A WHOLE NUMBER, so every
 //                  rescaling factor 2^(m_old - m_new) is an exact power of two: the
 //                  probabilities' rounding to bfloat16 for the second product is then the
@@ -384,12 +387,15 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
   const int wave_hi = wave_active ? positions[row0 + wave_last_tok] : -1;
   const int wave_lo = wave_active ? positions[row0 + wave_first_row / G] : 0;
 
-  f32x4_t o[NS][DBLK];
-  float m[NS], l[NS];
+  f32x4_t o[NS][DBLK], lsum[NS];
+  float m[NS];
+  bf16x8_t ones8;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ones8[i] = (bf16_t)1.0f;
 #pragma unroll
   for (int c = 0; c < NS; ++c) {
     m[c] = -INFINITY;
-    l[c] = 0.f;
+    lsum[c] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int db = 0; db < DBLK; ++db) o[c][db] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
   }
@@ -399,7 +405,9 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
   // tile) for head-dimension elements vdd0 + v * (NT / 16).  What does not change from
   // tile to tile is folded into two base pointers.
   const int krow0 = tid / VEC_PER_ROW, vkr = tid & 15, vdd0 = tid >> 4;
-  const size_t page_stride = (size_t)2 * nkv * page_size * D;
+  // (elements of one page, keys and values of all heads: below 2^32, the host checks;
+  // page * stride is then ONE 32 x 32 -> 64-bit multiply-add per load)
+  const unsigned page_stride = 2u * (unsigned)nkv * (unsigned)page_size * (unsigned)D;
   const bf16_t* kbase = kv + (size_t)gkv * page_size * D + (tid % VEC_PER_ROW) * 8;
   const bf16_t* vbase = kv + ((size_t)nkv + gkv) * page_size * D + (size_t)vdd0 * page_size;
   const int vstep = (NT / 16) * page_size;   // elements between a thread's value pieces
@@ -424,12 +432,12 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
 #pragma unroll
     for (int v = 0; v < KVEC; ++v) {
       const int off = page_offset(tile0 + krow0 + v * KROWS, page_size, ps_shift);
-      const int page = kpg[v] < 0 ? 0 : kpg[v];
-      kreg[v] = *reinterpret_cast<const bf16x8_t*>(kbase + (size_t)page * page_stride + off * D);
+      const unsigned page = kpg[v] < 0 ? 0u : (unsigned)kpg[v];
+      kreg[v] = *reinterpret_cast<const bf16x8_t*>(kbase + ((size_t)page * page_stride + (unsigned)(off * D)));
     }
     const int off = page_offset(tile0 + vkr * 4, page_size, ps_shift);
-    const int page = vpg < 0 ? 0 : vpg;
-    const bf16_t* src = vbase + (size_t)page * page_stride + off;
+    const unsigned page = vpg < 0 ? 0u : (unsigned)vpg;
+    const bf16_t* src = vbase + ((size_t)page * page_stride + (unsigned)off);
 #pragma unroll
     for (int v = 0; v < VVEC; ++v)
       vreg[v] = *reinterpret_cast<const bf16x4_t*>(src + v * vstep);
@@ -500,13 +508,21 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
 #pragma unroll
       for (int c = 0; c < NS; ++c) {
         if (needs_mask) {
+          // key jb * 16 + grp * 4 + i of the tile counts for this lane's row if it lies in
+          // [first, last]; both bounds are taken relative to the lane's own keys once, so
+          // that an element costs two comparisons with constants
+          int last = pos_row[c] < hi ? pos_row[c] : hi;
+          int first = lo;
+          if (window > 0 && pos_row[c] - window + 1 > first) first = pos_row[c] - window + 1;
+          last -= tile0 + grp * 4;
+          first -= tile0 + grp * 4;
+          const bool below = __any(first > 0);   // does any lane have keys before its first?
 #pragma unroll
           for (int jb = 0; jb < 4; ++jb)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-              const int kp = tile0 + jb * 16 + grp * 4 + i;
-              bool valid = kp <= pos_row[c] && kp >= lo && kp <= hi;
-              if (window > 0 && kp <= pos_row[c] - window) valid = false;
+              bool valid = jb * 16 + i <= last;
+              if (below) valid = valid && jb * 16 + i >= first;
               if (!valid) s[c][jb][i] = -INFINITY;
             }
         }
@@ -520,32 +536,32 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
         const float m_use = m_new > -INFINITY ? m_new : 0.f;
         // (nothing is accumulated yet while m is -inf: any finite factor does)
         const float alpha = m[c] > -INFINITY ? ldexpf(1.0f, (int)(m[c] - m_use)) : 1.0f;
-        float psum = 0.f;
 #pragma unroll
         for (int jb = 0; jb < 4; ++jb)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            // masked scores (-inf) give 0
-            const float p = __builtin_amdgcn_exp2f(fmaf(s[c][jb][i], scale_log2e, -m_use));
-            s[c][jb][i] = p;
-            psum += p;
-          }
-        psum = quad_sum(psum);
-        l[c] = l[c] * alpha + psum;
+          for (int i = 0; i < 4; ++i)   // masked scores (-inf) give 0
+            s[c][jb][i] = __builtin_amdgcn_exp2f(fmaf(s[c][jb][i], scale_log2e, -m_use));
         m[c] = m_new;
         if (__any(alpha != 1.0f)) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) lsum[c][i] *= alpha;
 #pragma unroll
           for (int db = 0; db < DBLK; ++db)
 #pragma unroll
             for (int i = 0; i < 4; ++i) o[c][db][i] *= alpha;
         }
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk)
+        for (int kk = 0; kk < 2; ++kk) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             pf[c][kk][i] = (bf16_t)s[c][2 * kk][i];
             pf[c][kk][4 + i] = (bf16_t)s[c][2 * kk + 1][i];
           }
+          // the row's sum of the ROUNDED probabilities, by the matrix core (a first operand
+          // of ones): every one of the accumulator's four values is the sum over the 32
+          // keys of the step for the lane's query row, all four lane groups' keys included
+          lsum[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones8, pf[c][kk], lsum[c], 0, 0, 0);
+        }
       }
 #pragma unroll
       for (int db = 0; db < DBLK; ++db)
@@ -574,11 +590,11 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
           *reinterpret_cast<f32x4_t*>(pa + db * 16 + grp * 4) = o[c][db];
         if (grp == 0) {
           part_ml[(orow * nsplit + z) * 2] = m[c];
-          part_ml[(orow * nsplit + z) * 2 + 1] = l[c];
+          part_ml[(orow * nsplit + z) * 2 + 1] = lsum[c][0];
         }
         continue;
       }
-      const float inv = l[c] > 0.f ? 1.0f / l[c] : 0.f;
+      const float inv = lsum[c][0] > 0.f ? 1.0f / lsum[c][0] : 0.f;
       bf16_t* dst = out + orow * D;
 #pragma unroll
       for (int db = 0; db < DBLK; ++db) {
@@ -783,30 +799,29 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
     const float m_new = fmaxf(m, ceilf(tmax));
     const float m_use = m_new > -INFINITY ? m_new : 0.f;
     const float alpha = m > -INFINITY ? ldexpf(1.0f, (int)(m - m_use)) : 1.0f;
-    float psum = 0.f;
 #pragma unroll
     for (int jb = 0; jb < 4; ++jb)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float p = __builtin_amdgcn_exp2f(s[jb][i] - m_use);
-        s[jb][i] = p;
-        psum += p;
-      }
-    psum = quad_sum(psum);
-    l = l * alpha + psum;
+      for (int i = 0; i < 4; ++i) s[jb][i] = __builtin_amdgcn_exp2f(s[jb][i] - m_use);
     m = m_new;
 #pragma unroll
     for (int db = 0; db < DBLK; ++db)
 #pragma unroll
       for (int i = 0; i < 4; ++i) o[db][i] *= alpha;
+    // the probabilities rounded for the second product; the sum that normalises the result
+    // is the sum of the rounded values, as in paged_attention_mfma_kernel
     bf16x8_t pf[2];
+    float psum = 0.f;
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         pf[kk][i] = (bf16_t)s[2 * kk][i];
         pf[kk][4 + i] = (bf16_t)s[2 * kk + 1][i];
+        psum += (float)pf[kk][i] + (float)pf[kk][4 + i];
       }
+    psum = quad_sum(psum);
+    l = l * alpha + psum;
 #pragma unroll
     for (int db = 0; db < DBLK; ++db)
 #pragma unroll

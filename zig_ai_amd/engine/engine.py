@@ -27,6 +27,7 @@ class Engine:
                  num_pages: Optional[int] = None, max_num_seqs: int = 64,
                  max_num_batched_tokens: int = 2048, chunk_size: int = 512,
                  max_model_len: Optional[int] = None, use_graphs: bool = True,
+                 portion_graphs: bool = False,
                  on_step=None, memory_fraction: float = 0.85, multi_step: int = 8,
                  reproducible: bool = False):
         """``num_pages``: pages per cache group; by default enough for
@@ -35,6 +36,8 @@ class Engine:
         fit into ``memory_fraction`` of the device memory that is free once the
         weights are loaded.
         ``use_graphs=False`` launches every decode step kernel by kernel.
+        ``portion_graphs=True`` also records steps with prompt portions, from the second
+        time a shape is seen (see ``DecodeGraphs.run_portions``).
         ``multi_step``: while every running request decodes and none waits, up to this
         many decode steps are issued without the host waiting for the tokens in
         between (each step's tokens reach the next on the device); a request that
@@ -74,7 +77,7 @@ class Engine:
                         " GiB); lower max_model_len")
                 num_pages = min(num_pages, fit)
         self.runner = ModelRunner(self.model, page_size, num_pages, max_num_seqs,
-                                  use_graphs=use_graphs)
+                                  use_graphs=use_graphs, portion_graphs=portion_graphs)
         self.on_step = on_step
         self.multi_step = 1 if on_step is not None else max(1, int(multi_step))
         self.scheduler = Scheduler(self.runner.cache, max_num_seqs, max_num_batched_tokens,

@@ -32,6 +32,7 @@ from .batch import PreparedEntries, StepEntry, StepError, build_step
 PAGE_BUCKET = 64        # block-table width is rounded up to a multiple of this
 KEYS_BUCKET = 1024      # and the longest context to a multiple of this
 MAX_GRAPHS = 96         # recorded shapes kept; the one replayed longest ago goes first
+MAX_PORTION_GRAPHS = 24 # the same for steps with prompt portions (their tensors are larger)
 
 
 def _round_up(n: int, m: int) -> int:
@@ -53,6 +54,10 @@ class DecodeGraphs:
         self._lib = hostlib.lib()
         self.captures = 0
         self.replays = 0
+        # steps of any other shape (prompt portions, alone or beside single tokens)
+        self.portion_entries: Dict[tuple, dict] = {}          # in order of last use
+        self.portion_captures = 0
+        self.portion_replays = 0
 
     def _scratch(self, S: int) -> dict:
         sc = self._arrays.get(S)
@@ -208,4 +213,76 @@ class DecodeGraphs:
             return logits
         graph.replay()                                     # the shape's second step
         self.replays += 1
+        return slot["logits"]
+
+    # ------------------------------------------------- steps with prompt portions
+    def run_portions(self, runner, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """A step of any shape (pages already reserved): prompt portions, alone or beside
+        single tokens.  A serving loop that cuts prompts into portions of one size issues
+        the same shapes again and again (the reference's ``-ub 512``,
+        /root/reference/src/main.zig:796-799), and a step of a few hundred tokens is some
+        150 launches that the host issues more slowly than the GPU runs them; replayed
+        from a graph the step is bound by the GPU again.
+
+        The shape: tokens and wanted rows of every entry, in order, the width of the
+        block tables and the longest context, both rounded up.  A shape's first step
+        runs as it is; its second is recorded and replayed (so shapes that never come
+        back cost nothing), every later one is a replay."""
+        cache, model = runner.cache, runner.model
+        prepared = PreparedEntries(entries, cache, self._vocab)
+        grans = np.asarray(sorted(set(int(g) for g in self._granularities)), dtype=np.int32)
+        sections = np.zeros((2 * (7 + 2 * len(cache.groups) + 3 * len(grans)),), dtype=np.int64)
+        prepared.build(cache, grans, self._max_position, 0, sections, None, 0)     # sizes only
+        widest, longest = int(prepared.meta[3]), int(prepared.meta[4])
+        key = (tuple(prepared.counts.tolist()), tuple(prepared.want_counts.tolist()),
+               _round_up(max(widest, 1), PAGE_BUCKET), _round_up(max(longest, 1), KEYS_BUCKET))
+        slot = self.portion_entries.get(key)
+        if slot is None:
+            if len(self.portion_entries) >= 4 * MAX_PORTION_GRAPHS:    # sightings are cheap, not free
+                for old in [k for k, v in self.portion_entries.items() if v["graph"] is None][:MAX_PORTION_GRAPHS]:
+                    self.portion_entries.pop(old)
+            self.portion_entries[key] = {"graph": None, "seen": 1}
+            ctx = build_step(entries, cache, runner.device, self._vocab, self._granularities,
+                             self._max_position, prepared=prepared)
+            return model.forward(ctx, runner.views)
+        self.portion_entries[key] = self.portion_entries.pop(key)      # now the most recently used
+        if slot["graph"] is None:
+            probe = build_step(entries, cache, torch.device("cpu"), self._vocab, self._granularities,
+                               self._max_position, min_pages=key[2], max_keys=key[3], prepared=prepared)
+            words = probe.host.size
+            recorded = [k for k, v in self.portion_entries.items() if v["graph"] is not None]
+            if len(recorded) >= MAX_PORTION_GRAPHS:
+                torch.cuda.current_stream().synchronize()    # its last replay may still run
+                self.portion_entries.pop(recorded[0])
+            slot.update(buffer=torch.full((words,), -1, dtype=torch.int32, device=runner.device),
+                        pinned=torch.empty((words,), dtype=torch.int32, pin_memory=True),
+                        copied=None, words=words)
+            ctx = build_step(entries, cache, runner.device, self._vocab, self._granularities,
+                             self._max_position, min_pages=key[2], max_keys=key[3],
+                             into=slot["buffer"], prepared=prepared)
+            graph = torch.cuda.CUDAGraph()
+            was_enabled = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(graph):                  # recorded, not executed
+                    slot["logits"] = model.forward(ctx, runner.views)
+            finally:
+                if was_enabled:
+                    gc.enable()
+            slot["graph"] = graph
+            self.portion_captures += 1
+        else:
+            if slot["copied"] is not None:
+                slot["copied"].synchronize()        # the last transfer out of the staging buffer
+            ctx = build_step(entries, cache, runner.device, self._vocab, self._granularities,
+                             self._max_position, min_pages=key[2], max_keys=key[3],
+                             into=slot["buffer"], staging=slot["pinned"], prepared=prepared)
+            if ctx.host.size != slot["words"]:
+                raise StepError(f"the step's layout has {ctx.host.size} entries, the recorded one "
+                                f"{slot['words']}")
+            if slot["copied"] is None:
+                slot["copied"] = torch.cuda.Event()
+            slot["copied"].record()
+        slot["graph"].replay()
+        self.portion_replays += 1
         return slot["logits"]

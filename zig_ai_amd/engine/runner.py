@@ -26,14 +26,16 @@ from .model import DecoderModel
 
 class ModelRunner:
     def __init__(self, model: DecoderModel, page_size: int = 16, num_pages: int = 1024,
-                 num_slots: int = 64, use_graphs: bool = True):
+                 num_slots: int = 64, use_graphs: bool = True, portion_graphs: bool = False):
         """``use_graphs``: replay steps of single tokens as HIP graphs when every part
-        of the model declares itself safe to record (``graph_safe``)."""
+        of the model declares itself safe to record (``graph_safe``).  ``portion_graphs``:
+        also steps with prompt portions, from the second time a shape is seen."""
         self.model = model
         self.device = model.runtime.device
         self.cache = model.make_cache(page_size, num_pages, num_slots)
         self.views = model.cache_views(self.cache)
         self.steps_run = 0
+        self.portion_graphs = bool(portion_graphs)
         self.graphs = (DecodeGraphs(model.spec.vocab_size, model.item_granularities, model.spec.max_position)
                        if (use_graphs and model.graph_safe) else None)
 
@@ -69,6 +71,9 @@ class ModelRunner:
         if taps is None and self.graphs is not None and entries \
                 and all(len(e.tokens) == 1 for e in entries):
             logits = self._graph_step(entries)
+        elif taps is None and self.graphs is not None and entries and self.portion_graphs:
+            self.reserve(entries)
+            logits = self.graphs.run_portions(self, entries)
         else:
             ctx = self.prepare(entries)
             logits = self.model.forward(ctx, self.views, taps)
