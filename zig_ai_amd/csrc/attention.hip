@@ -646,7 +646,6 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
   const bool row_valid = r16 < rows;
   const int tok = row0 + (row_valid ? r16 / G : 0);
   const int head = gkv * G + (row_valid ? r16 % G : 0);
-  const int pos_row = row_valid ? positions[tok] : -1;
   const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 
   bf16x8_t qf[KSTEPS];
@@ -655,17 +654,6 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
     qf[ks] = row_valid ? *reinterpret_cast<const bf16x8_t*>(
                              q + ((size_t)tok * nh + head) * D + ks * 32 + grp * 8)
                        : zero8;
-
-  const int pos_first = positions[row0];
-  const int pos_last = positions[row0 + count - 1];
-  const int lo = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
-  const int hi = pos_last;
-  int range_lo = z * keys_per_split;
-  int range_hi = range_lo + keys_per_split - 1;
-  if (nsplit == 1) { range_lo = 0; range_hi = hi; }
-  if (range_hi > hi) range_hi = hi;
-  int tile_first = (lo / AM_KT) * AM_KT;
-  if (tile_first < range_lo) tile_first = range_lo;
 
   f32x4_t o[DBLK];
 #pragma unroll
@@ -685,11 +673,8 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
   // (two of 8 bytes when the page size is no multiple of 8).
   bf16x8_t kf[4][KSTEPS];
   bf16x8_t vf[DBLK][2];
-  // The block-table entries are read whether or not the key turns out to be in
-  // range (unused entries hold -1 and read page 0 instead), so that these loads do
-  // not wait for the positions the range is computed from.  A key that must not
-  // count is masked in the scores, whatever its row holds; its values are cleared,
-  // since 0 * (not a number) would not be 0.
+  // Block-table entries are read whether or not their keys turn out to be in range
+  // (an entry beyond the table reads the last one, an unused entry, -1, page 0).
   const int last_entry = bt_stride - 1;
   const int ps_shift = page_shift_of(page_size);
   const bool wide = page_size % 8 == 0;
@@ -698,19 +683,25 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
     const int e = page_entry(key, page_size, ps_shift);
     return table[e < last_entry ? e : last_entry];
   };
-  auto fetch = [&](int tile0, bf16x8_t (&kfr)[4][KSTEPS], bf16x8_t (&vfr)[DBLK][2]) {
+  // With pages of 16, 32, 64 ... keys a block of 16 keys lies in one page (tiles start at
+  // multiples of 16 keys): four entries a tile, the same for the whole wave.  The entries
+  // of the wave's next sixteen tiles are read by ONE vector load, lane i * 4 + b taking
+  // block b of the i-th tile, and handed out lane by lane: a tile's loads of keys and
+  // values then wait for no table lookup of their own.
+  int tbl = 0;
+  auto load_entries = [&](int first_tile0) {
+    const int key = first_tile0 + (lane >> 2) * (NWV * AM_KT) + (lane & 3) * 16;
+    const int e = key >> (ps_shift >= 4 ? ps_shift : 4);
+    tbl = table[e < last_entry ? e : last_entry];
+  };
+  // `nth`: which of the wave's tiles since the entries were read (0 .. 15)
+  auto fetch = [&](int tile0, int nth, bf16x8_t (&kfr)[4][KSTEPS], bf16x8_t (&vfr)[DBLK][2]) {
     int kpage[4], vpage[4];      // vpage: per run of 4 keys, kk * 2 + half
     if (ps_shift >= 4) {
-      // Tiles start at multiples of 16 keys, so with pages of 16, 32, 64 ... keys a
-      // block of 16 keys lies in one page: one entry for the whole wave, which the
-      // scalar unit reads without waiting for the vector loads in flight.
-      const int t0 = __builtin_amdgcn_readfirstlane(tile0);
+      const int first = __builtin_amdgcn_readfirstlane(nth) * 4;
       int pg[4];
 #pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const int e = (t0 + b * 16) >> ps_shift;
-        pg[b] = table[e < last_entry ? e : last_entry];
-      }
+      for (int b = 0; b < 4; ++b) pg[b] = __builtin_amdgcn_readlane(tbl, first + b);
 #pragma unroll
       for (int jb = 0; jb < 4; ++jb) {
         kpage[jb] = (r16 & 8) ? pg[(jb >> 1) * 2 + 1] : pg[(jb >> 1) * 2];
@@ -733,7 +724,6 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
       for (int ks = 0; ks < KSTEPS; ++ks)
         kfr[jb][ks] = *reinterpret_cast<const bf16x8_t*>(krow + ks * 32 + grp * 8);
     }
-    const bool inner = tile0 >= lo && tile0 + AM_KT - 1 <= range_hi;
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
       const int kp = tile0 + kk * 32 + grp * 8;          // this lane's eight keys
@@ -754,24 +744,66 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
           const bf16x4_t xb = *reinterpret_cast<const bf16x4_t*>(vb + row);
           x = __builtin_shufflevector(xa, xb, 0, 1, 2, 3, 4, 5, 6, 7);
         }
-        if (!inner) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (vpage[2 * kk + (e >> 2)] < 0 || kp + e < lo || kp + e > range_hi)
-              x[e] = (bf16_t)0.f;
-        }
         vfr[db][kk] = x;
       }
     }
   };
 
+  // Without a window the wave's first tile is known before the positions have arrived
+  // (a range starts where the launch says): its entries, keys and values are requested
+  // at once, so that the kernel's start is two trips to memory (entries and positions
+  // side by side, then keys and values) and not three.  A wave whose tile turns out to
+  // lie beyond the context has loaded in vain (from inside the pool, as every load here).
+  const bool early = window == 0;
+  if (early) {
+    const int first_tile0 = (nsplit == 1 ? 0 : z * keys_per_split) + wave * AM_KT;
+    if (ps_shift >= 4) load_entries(first_tile0);
+    fetch(first_tile0, 0, kf, vf);
+  }
+
+  const int pos_first = positions[row0];
+  const int pos_last = positions[row0 + count - 1];
+  const int pos_row = row_valid ? positions[tok] : -1;
+  const int lo = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
+  const int hi = pos_last;
+  int range_lo = z * keys_per_split;
+  int range_hi = range_lo + keys_per_split - 1;
+  if (nsplit == 1) { range_lo = 0; range_hi = hi; }
+  if (range_hi > hi) range_hi = hi;
+  int tile_first = (lo / AM_KT) * AM_KT;
+  if (tile_first < range_lo) tile_first = range_lo;
+
   int tile0 = tile_first + wave * AM_KT;
-  if (tile0 <= range_hi) fetch(tile0, kf, vf);
+  if (!early && tile0 <= range_hi) {
+    if (ps_shift >= 4) load_entries(tile0);
+    fetch(tile0, 0, kf, vf);
+  }
+  int nth = 0;
   for (; tile0 <= range_hi; tile0 += NWV * AM_KT) {
     bf16x8_t kfn[4][KSTEPS];
     bf16x8_t vfn[DBLK][2];
     const int next = tile0 + NWV * AM_KT;
-    if (next <= range_hi) fetch(next, kfn, vfn);
+    if (next <= range_hi) {
+      if (++nth == 16) {
+        nth = 0;
+        if (ps_shift >= 4) load_entries(next);
+      }
+      fetch(next, nth, kfn, vfn);
+    }
+    // A key that must not count is masked in the scores, whatever its row holds; its
+    // values are cleared, since 0 * (not a number) would not be 0.  (Keys whose page is
+    // not there, entry -1, lie outside [lo, range_hi] too.)
+    if (tile0 < lo || tile0 + AM_KT - 1 > range_hi) {
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        const int kp = tile0 + kk * 32 + grp * 8;
+#pragma unroll
+        for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (kp + e < lo || kp + e > range_hi) vf[db][kk][e] = (bf16_t)0.f;
+      }
+    }
 
     f32x4_t s[4];
 #pragma unroll
