@@ -76,6 +76,54 @@ def test_groups_and_views():
     assert m.bytes_per_slot == 2 * 8 * 3 * 4
 
 
+def test_planes_and_typed_state_in_memory():
+    """What mixers declare decides the memory: planes of different sizes in one page, a
+    storage type per need, state of any type; on the CPU here, the layout is the same."""
+    import torch
+    latent = PagedNeed(((1, 24),), dtype=torch.float32)              # one vector per token
+    uneven = PagedNeed(((2, 16), (2, 8), (1, 4)))                    # three planes, different sizes
+    needs = {"kv": PagedNeed.kv(2, 16), ("a", "mixer"): latent, ("b", "mixer"): latent, "u": uneven,
+             "count": StateNeed((1,), dtype=torch.int32), "conv": StateNeed((8, 3)),
+             "flag": StateNeed((5,), dtype=torch.uint8)}
+    m = CacheManager(needs, 4, {PagedNeed.kv(2, 16): 6, latent: 5, uneven: 3}, 3,
+                     device=torch.device("cpu"), dtype=torch.bfloat16)
+    assert [len(g.cache_ids) for g in m.groups] == [1, 2, 1]
+    kv, lat, une = m.groups
+    assert kv.memory.shape == (1, 6, 4 * 2 * 2 * 16) and kv.memory.dtype == torch.bfloat16
+    assert lat.memory.shape == (2, 5, 4 * 24) and lat.memory.dtype == torch.float32
+    assert une.memory.shape == (1, 3, 4 * (32 + 16 + 4))
+    assert kv.kv.shape == (1, 6, 2, 2, 4, 16) and lat.kv is None and une.kv is None
+    v = m.view("kv")
+    assert v.kv.shape == (6, 2, 2, 4, 16) and [tuple(p.shape) for p in v.planes] == [(6, 2, 4, 16)] * 2
+    v.planes[1][3, 1, 2, 5] = 7.0                  # the second plane IS the values' half of kv
+    assert float(v.kv[3, 1, 1, 2, 5]) == 7.0
+    second = m.view(("b", "mixer"))
+    assert second.kv is None and tuple(second.planes[0].shape) == (5, 1, 4, 24)
+    second.planes[0][2, 0, 1, 3] = 1.5
+    assert float(lat.memory[1, 2, 1 * 24 + 3]) == 1.5 and float(lat.memory[0].abs().sum()) == 0.0
+    shapes = [tuple(p.shape) for p in m.view("u").planes]
+    assert shapes == [(3, 2, 4, 16), (3, 2, 4, 8), (3, 1, 4, 4)]
+    m.view("u").planes[2][1, 0, 3, 2] = 2.0         # the last element but one row of page 1
+    assert float(une.memory[0, 1, 4 * 48 + 3 * 4 + 2]) == 2.0
+    # a page more in every group costs the bytes of one page of every entry
+    assert CacheManager.bytes_per_page_index(needs, 4, torch.bfloat16) == \
+        4 * (64 * 2 + 24 * 4 * 2 + 52 * 2)
+    # state: typed windows of one row of bytes per slot, each 16-byte aligned
+    count, conv, flag = m.view("count").state, m.view("conv").state, m.view("flag").state
+    assert (count.dtype, conv.dtype, flag.dtype) == (torch.int32, torch.float32, torch.uint8)
+    assert tuple(count.shape) == (3, 1) and tuple(conv.shape) == (3, 8, 3) and tuple(flag.shape) == (3, 5)
+    assert m.bytes_per_slot == 16 + 96 + 16
+    slot = m.admit("r")
+    count[slot, 0] = 41
+    conv[slot] = 2.5
+    flag[slot] = 9
+    m.release("r")
+    assert m.admit("again") == slot                 # the slot comes back cleared
+    assert int(count[slot, 0]) == 0 and float(conv[slot].abs().sum()) == 0.0 and int(flag[slot].sum()) == 0
+    with pytest.raises(ValueError):
+        CacheManager({0: PagedNeed(())}, 4, 4, 1, allocate=False)
+
+
 def test_reserve_is_all_or_nothing():
     m = manager(num_pages=4, window=6)
     m.admit("a")

@@ -108,6 +108,23 @@ def test_tokens_do_not_depend_on_scheduling():
     assert all(g["pages_free"] == g["pages"] for g in stats["groups"])
 
 
+def test_a_length_limit_beyond_the_models_own_is_refused():
+    """``max_model_len`` above the model's ``max_position_embeddings`` would stop a step in
+    the middle of a call and every request of the call with it: refused when the engine is
+    made."""
+    from zig_ai_amd.engine import Engine
+    short = dict(TINY_A, max_position_embeddings=64)
+    folder = eu.model_folder(short, 0, torch.float32, **eu.sharp_kwargs())
+    with pytest.raises(ValueError, match="max_position_embeddings"):
+        Engine(folder, dtype="float32", page_size=4, num_pages=64, max_model_len=100)
+    engine = Engine(folder, dtype="float32", page_size=4, num_pages=64)
+    assert engine.max_model_len == 64
+    with pytest.raises(ValueError):
+        engine.generate([eu.random_tokens(60, 256, 1)], max_new_tokens=10, temperature=0.0)
+    assert len(engine.generate([eu.random_tokens(50, 256, 1)], max_new_tokens=10,
+                               temperature=0.0, eos_token_id=-1)[0]) == 10
+
+
 def test_eos_and_length_stop():
     from zig_ai_amd.engine import Engine
     folder = folder_for(TINY_A, 0)
