@@ -642,7 +642,7 @@ def items_for(seq_lens, rows_per_item):
 
 
 def run_attention(dtype, nh, nkv, d, page_size, ctx, new, window=0, keys_per_split=0, nsplit=1,
-                  seed=30, sharpen=False, mfma=False, mfma_decode=False):
+                  seed=30, sharpen=False, mfma=False, mfma_decode=False, tile_keys=64):
     """ctx[s] cached tokens and new[s] query tokens per request."""
     G = nh // nkv
     ks, vs, qs, pos = [], [], [], []
@@ -668,7 +668,7 @@ def run_attention(dtype, nh, nkv, d, page_size, ctx, new, window=0, keys_per_spl
     elif mfma:
         out = ops().paged_attention_mfma(q_all, cache.to(dev()), table.to(dev()), positions,
                                          *items_for(new, max(1, 128 // G)), 1.0 / math.sqrt(d),
-                                         window, keys_per_split, nsplit)
+                                         window, keys_per_split, nsplit, tile_keys=tile_keys)
     else:
         out = ops().paged_attention(q_all, cache.to(dev()), table.to(dev()), positions,
                                     *items_for(new, max(1, 32 // G)), 1.0 / math.sqrt(d), window,
@@ -710,30 +710,33 @@ def test_paged_attention_reference_shapes(dtype):
     (32, 8, 64, 16), (4, 4, 64, 4), (8, 4, 128, 16), (16, 2, 64, 8), (16, 1, 128, 32), (2, 1, 64, 16),
     (6, 2, 64, 12), (5, 1, 128, 20), (7, 7, 64, 64)])
 @pytest.mark.parametrize("window", [0, 70])
-def test_paged_attention_matrix_cores(nh, nkv, d, page_size, window):
+@pytest.mark.parametrize("tile_keys", [64, 128])
+def test_paged_attention_matrix_cores(nh, nkv, d, page_size, window, tile_keys):
     """The matrix-core kernel on mixed steps: long portions, portions that do not fill
-    a work item, single tokens with long contexts."""
+    a work item, single tokens with long contexts; with tiles of 64 and of 128 keys."""
     ctx = [0, 37, 129, 5, 300]
     new = [150, 1, 17, 70, 2]
     out, expect = run_attention(torch.bfloat16, nh, nkv, d, page_size, ctx, new, window=window,
-                                mfma=True)
+                                mfma=True, tile_keys=tile_keys)
     assert rel_err(out, expect) < BF16_TOL
     out, expect = run_attention(torch.bfloat16, nh, nkv, d, page_size, [700, 300], [1, 40],
-                                sharpen=True, mfma=True)
+                                sharpen=True, mfma=True, tile_keys=tile_keys)
     assert rel_err(out, expect) < BF16_TOL
     assert float(expect.abs().max()) > 0.5
 
 
 @pytest.mark.parametrize("keys,nsplit", [(64, 12), (256, 3), (1024, 1)])
 @pytest.mark.parametrize("window", [0, 70])
-def test_paged_attention_matrix_cores_cut_contexts(keys, nsplit, window):
+@pytest.mark.parametrize("tile_keys", [64, 128])
+def test_paged_attention_matrix_cores_cut_contexts(keys, nsplit, window, tile_keys):
     """Prompt portions with their contexts cut into ranges: ranges that a row cannot
     see at all, ranges that end inside a tile's worth of rows, empty ranges."""
     ctx = [700, 0, 255, 64, 300]
     new = [40, 150, 3, 70, 1]
     for nh, nkv, d, ps in [(32, 8, 64, 16), (6, 2, 128, 8)]:
         out, expect = run_attention(torch.bfloat16, nh, nkv, d, ps, ctx, new, window=window,
-                                    keys_per_split=keys, nsplit=nsplit, sharpen=True, mfma=True)
+                                    keys_per_split=keys, nsplit=nsplit, sharpen=True, mfma=True,
+                                    tile_keys=tile_keys)
         assert rel_err(out, expect) < BF16_TOL
 
 

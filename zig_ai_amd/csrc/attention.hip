@@ -265,7 +265,7 @@ attention_combine_kernel(const float* __restrict__ part_acc, const float* __rest
 // Operand layout of v_mfma_f32_16x16x32_bf16: lane l supplies row (l % 16), k-slots
 // (l / 16) * 8 .. + 7 of either operand and receives rows (l / 16) * 4 .. + 3, column
 // (l % 16) of the product.
-#define AM_KT 64
+#define AM_KT 64       // keys of a tile in the decode kernel (the prefill kernel: 64 or 128)
 #define AM_ROWS 128
 #define ZA_DECODE_WIDE_BELOW 384   // workgroups: up to here the decode kernel runs eight waves
 
@@ -305,7 +305,7 @@ __device__ __forceinline__ int page_offset(int kp, int page_size, int shift) {
   return shift >= 0 ? kp & (page_size - 1) : kp % page_size;
 }
 
-template <int D, int NW, int NS>
+template <int D, int NW, int NS, int KT>
 __global__ void __launch_bounds__(NW * 64)
 paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                             const bf16_t* __restrict__ kv, const int* __restrict__ block_table,
@@ -316,18 +316,22 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
                             int nkv, int page_size, float scale_log2e, int window,
                             int keys_per_split, int nsplit) {
   constexpr int LDK = D + 8;        // padded rows, in elements
-  constexpr int LDV = AM_KT + 8;
+  constexpr int LDV = KT + 8;
   constexpr int KSTEPS = D / 32;    // matrix-core steps over the head dimension
   constexpr int DBLK = D / 16;      // 16-wide blocks of the head dimension
   constexpr int VEC_PER_ROW = D / 8;
   constexpr int NT = NW * 64;                      // threads
-  constexpr int KVEC = AM_KT * VEC_PER_ROW / NT;   // 16-byte pieces of a key tile per thread
-  constexpr int VVEC = D * (AM_KT / 4) / NT;       // 8-byte pieces of a value tile per thread
+  constexpr int KVEC = KT * VEC_PER_ROW / NT;   // 16-byte pieces of a key tile per thread
+  constexpr int VVEC = D * (KT / 4) / NT;       // 8-byte pieces of a value tile per thread
   constexpr int KROWS = NT / VEC_PER_ROW;          // keys between a thread's pieces
-  static_assert(NW * NS * 16 == AM_ROWS && KVEC >= 1 && VVEC >= 1, "tile shape");
+  constexpr int JB = KT / 16;                      // blocks of 16 keys in a tile
+  constexpr int KK = KT / 32;                      // matrix-core steps over a tile's keys
+  constexpr int VRUNS = KT / 4;                    // runs of 4 keys in a tile
+  static_assert(NW * NS * 16 == AM_ROWS && KVEC >= 1 && VVEC >= 1 && (KT == 64 || KT == 128),
+                "tile shape");
   extern __shared__ __attribute__((aligned(16))) unsigned char am_smem[];
   bf16_t* Ks = reinterpret_cast<bf16_t*>(am_smem);   // [2][key][dim]
-  bf16_t* Vt = Ks + 2 * AM_KT * LDK;                 // [2][dim][key slot]
+  bf16_t* Vt = Ks + 2 * KT * LDK;                 // [2][dim][key slot]
 
   const int gkv = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -404,13 +408,13 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
   // krow0 + v * KROWS, and VVEC 8-byte runs of 4 consecutive keys (run vkr of the
   // tile) for head-dimension elements vdd0 + v * (NT / 16).  What does not change from
   // tile to tile is folded into two base pointers.
-  const int krow0 = tid / VEC_PER_ROW, vkr = tid & 15, vdd0 = tid >> 4;
+  const int krow0 = tid / VEC_PER_ROW, vkr = tid & (VRUNS - 1), vdd0 = tid / VRUNS;
   // (elements of one page, keys and values of all heads: below 2^32, the host checks;
   // page * stride is then ONE 32 x 32 -> 64-bit multiply-add per load)
   const unsigned page_stride = 2u * (unsigned)nkv * (unsigned)page_size * (unsigned)D;
   const bf16_t* kbase = kv + (size_t)gkv * page_size * D + (tid % VEC_PER_ROW) * 8;
   const bf16_t* vbase = kv + ((size_t)nkv + gkv) * page_size * D + (size_t)vdd0 * page_size;
-  const int vstep = (NT / 16) * page_size;   // elements between a thread's value pieces
+  const int vstep = (NT / VRUNS) * page_size;   // elements between a thread's value pieces
 
   int kpg[KVEC], vpg;
   bf16x8_t kreg[KVEC];
@@ -444,16 +448,16 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
   };
   // keys jb * 16 + g4 * 4 .. + 3 of the tile sit in slots: 32-key step, then lane group,
   // then block
-  const int vslot = ((vkr >> 3) & 1) * 32 + (vkr & 3) * 8 + ((vkr >> 2) & 1) * 4;
+  const int vslot = (vkr >> 3) * 32 + (vkr & 3) * 8 + ((vkr >> 2) & 1) * 4;
   auto store_tile = [&](int buf, int tile0) {
-    bf16_t* ks = Ks + buf * AM_KT * LDK;
+    bf16_t* ks = Ks + buf * KT * LDK;
     bf16_t* vt = Vt + buf * D * LDV;
 #pragma unroll
     for (int v = 0; v < KVEC; ++v)
       *reinterpret_cast<bf16x8_t*>(ks + (krow0 + v * KROWS) * LDK + (tid % VEC_PER_ROW) * 8) =
           kreg[v];
     const int kp = tile0 + vkr * 4;
-    const bool edge_tile = tile0 < lo || tile0 + AM_KT - 1 > hi;   // the same for all threads
+    const bool edge_tile = tile0 < lo || tile0 + KT - 1 > hi;   // the same for all threads
 #pragma unroll
     for (int v = 0; v < VVEC; ++v) {
       bf16x4_t x = vreg[v];
@@ -463,33 +467,33 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
         for (int e = 0; e < 4; ++e)
           if (kp + e < lo || kp + e > hi) x[e] = (bf16_t)0.f;
       }
-      *reinterpret_cast<bf16x4_t*>(vt + (vdd0 + v * (NT / 16)) * LDV + vslot) = x;
+      *reinterpret_cast<bf16x4_t*>(vt + (vdd0 + v * (NT / VRUNS)) * LDV + vslot) = x;
     }
   };
 
-  int tile_first = (lo / AM_KT) * AM_KT;
+  int tile_first = (lo / KT) * KT;
   if (nsplit > 1 && z * keys_per_split > tile_first) tile_first = z * keys_per_split;
-  const int n_tiles = hi >= tile_first ? (hi - tile_first) / AM_KT + 1 : 0;   // 0: an empty range
+  const int n_tiles = hi >= tile_first ? (hi - tile_first) / KT + 1 : 0;   // 0: an empty range
   load_pages(tile_first);
   load_data(tile_first);
-  load_pages(tile_first + AM_KT);
+  load_pages(tile_first + KT);
   store_tile(0, tile_first);
   __syncthreads();
 
   for (int t = 0; t < n_tiles; ++t) {
-    const int tile0 = tile_first + t * AM_KT;
+    const int tile0 = tile_first + t * KT;
     const int buf = t & 1;
-    load_data(tile0 + AM_KT);
-    load_pages(tile0 + 2 * AM_KT);
+    load_data(tile0 + KT);
+    load_pages(tile0 + 2 * KT);
 
     bool wave_sees = wave_active && tile0 <= wave_hi;
-    if (window > 0 && tile0 + AM_KT - 1 <= wave_lo - window) wave_sees = false;
+    if (window > 0 && tile0 + KT - 1 <= wave_lo - window) wave_sees = false;
     if (wave_sees) {
-      const bf16_t* ks = Ks + buf * AM_KT * LDK;
+      const bf16_t* ks = Ks + buf * KT * LDK;
       const bf16_t* vt = Vt + buf * D * LDV;
-      f32x4_t s[NS][4];
+      f32x4_t s[NS][JB];
 #pragma unroll
-      for (int jb = 0; jb < 4; ++jb) {
+      for (int jb = 0; jb < JB; ++jb) {
 #pragma unroll
         for (int c = 0; c < NS; ++c) s[c][jb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -502,9 +506,9 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
         }
       }
       // a tile every key of which counts for every row of the wave needs no mask
-      const bool needs_mask = !wave_full || tile0 + AM_KT - 1 > wave_lo || tile0 < lo ||
-                              tile0 + AM_KT - 1 > hi || (window > 0 && tile0 <= wave_hi - window);
-      bf16x8_t pf[NS][2];
+      const bool needs_mask = !wave_full || tile0 + KT - 1 > wave_lo || tile0 < lo ||
+                              tile0 + KT - 1 > hi || (window > 0 && tile0 <= wave_hi - window);
+      bf16x8_t pf[NS][KK];
 #pragma unroll
       for (int c = 0; c < NS; ++c) {
         if (needs_mask) {
@@ -518,7 +522,7 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
           first -= tile0 + grp * 4;
           const bool below = __any(first > 0);   // does any lane have keys before its first?
 #pragma unroll
-          for (int jb = 0; jb < 4; ++jb)
+          for (int jb = 0; jb < JB; ++jb)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               bool valid = jb * 16 + i <= last;
@@ -528,7 +532,7 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
         }
         float tmax = -INFINITY;
 #pragma unroll
-        for (int jb = 0; jb < 4; ++jb)
+        for (int jb = 0; jb < JB; ++jb)
 #pragma unroll
           for (int i = 0; i < 4; ++i) tmax = fmaxf(tmax, s[c][jb][i]);
         tmax = quad_max(tmax);
@@ -537,7 +541,7 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
         // (nothing is accumulated yet while m is -inf: any finite factor does)
         const float alpha = m[c] > -INFINITY ? ldexpf(1.0f, (int)(m[c] - m_use)) : 1.0f;
 #pragma unroll
-        for (int jb = 0; jb < 4; ++jb)
+        for (int jb = 0; jb < JB; ++jb)
 #pragma unroll
           for (int i = 0; i < 4; ++i)   // masked scores (-inf) give 0
             s[c][jb][i] = __builtin_amdgcn_exp2f(fmaf(s[c][jb][i], scale_log2e, -m_use));
@@ -551,7 +555,7 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
             for (int i = 0; i < 4; ++i) o[c][db][i] *= alpha;
         }
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
+        for (int kk = 0; kk < KK; ++kk) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             pf[c][kk][i] = (bf16_t)s[c][2 * kk][i];
@@ -566,7 +570,7 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
 #pragma unroll
       for (int db = 0; db < DBLK; ++db)
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
+        for (int kk = 0; kk < KK; ++kk) {
           const bf16x8_t vf = *reinterpret_cast<const bf16x8_t*>(
               vt + (db * 16 + r16) * LDV + kk * 32 + grp * 8);
 #pragma unroll
@@ -574,7 +578,7 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
             o[c][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[c][kk], o[c][db], 0, 0, 0);
         }
     }
-    if (t + 1 < n_tiles) store_tile(buf ^ 1, tile0 + AM_KT);
+    if (t + 1 < n_tiles) store_tile(buf ^ 1, tile0 + KT);
     __syncthreads();
   }
 
@@ -975,7 +979,7 @@ extern "C" int za_paged_attention(const void* q, void* out, const void* kv, cons
   return za_launch_status();
 }
 
-template <int D>
+template <int D, int KT>
 static int launch_attention_mfma(const void* q, void* out, const void* kv, const int* block_table,
                                  int bt_stride, const int* positions, const int* wi_seq,
                                  const int* wi_row0, const int* wi_count, int n_items,
@@ -983,8 +987,8 @@ static int launch_attention_mfma(const void* q, void* out, const void* kv, const
                                  int page_size, float scale, int window, int keys_per_split,
                                  int nsplit, hipStream_t stream) {
   constexpr int NW = 8, NS = AM_ROWS / (NW * 16);
-  const size_t shmem = ((size_t)2 * AM_KT * (D + 8) + (size_t)2 * D * (AM_KT + 8)) * sizeof(bf16_t);
-  auto kernel = paged_attention_mfma_kernel<D, NW, NS>;
+  const size_t shmem = ((size_t)2 * KT * (D + 8) + (size_t)2 * D * (KT + 8)) * sizeof(bf16_t);
+  auto kernel = paged_attention_mfma_kernel<D, NW, NS, KT>;
   static bool allowed = false;
   if (!allowed) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel,
@@ -1018,25 +1022,31 @@ extern "C" int za_paged_attention_mfma(const void* q, void* out, const void* kv,
                                        const int* wi_row0, const int* wi_count, int n_items,
                                        int n_tokens, float* part_acc, float* part_ml, int nh,
                                        int nkv, int d, int page_size, float scale, int window,
-                                       int keys_per_split, int nsplit, hipStream_t stream) {
+                                       int keys_per_split, int nsplit, int tile_keys,
+                                       hipStream_t stream) {
   if (n_items == 0 || n_tokens == 0) return 0;
   if (nsplit < 1 || nsplit > 65535 ||
       (nsplit > 1 && (!part_acc || !part_ml || keys_per_split <= 0 || keys_per_split % 64 != 0)))
     return ZA_ERR_ARG;
   if (n_items < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || page_size <= 0 || bt_stride <= 0 ||
-      !q || !out || !kv || !block_table || !positions || !wi_seq || !wi_row0 || !wi_count)
+      !q || !out || !kv || !block_table || !positions || !wi_seq || !wi_row0 || !wi_count ||
+      (tile_keys != 64 && tile_keys != 128))
     return ZA_ERR_ARG;
   const int G = nh / nkv;
+  // (a page's elements, keys and values of all heads, must fit 32 bits: the kernel
+  // multiplies page numbers by that stride in one instruction)
   if ((d != 64 && d != 128) || G > AM_ROWS || page_size % 4 != 0 || !(scale > 0.f) ||
-      nkv > 65535)
+      nkv > 65535 || 2ull * nkv * page_size * d > 0xffffffffull)
     return ZA_ERR_UNSUPPORTED;
-  if (d == 64)
-    return launch_attention_mfma<64>(q, out, kv, block_table, bt_stride, positions, wi_seq,
-                                     wi_row0, wi_count, n_items, n_tokens, part_acc, part_ml, nh,
-                                     nkv, page_size, scale, window, keys_per_split, nsplit, stream);
-  return launch_attention_mfma<128>(q, out, kv, block_table, bt_stride, positions, wi_seq,
-                                    wi_row0, wi_count, n_items, n_tokens, part_acc, part_ml, nh,
-                                    nkv, page_size, scale, window, keys_per_split, nsplit, stream);
+#define ZA_AM_ARGS                                                                             \
+  q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0, wi_count, n_items, n_tokens, \
+      part_acc, part_ml, nh, nkv, page_size, scale, window, keys_per_split, nsplit, stream
+  // tiles of 128 keys spread a tile's fixed work (running maximum, addresses) over twice
+  // the scores: for long contexts; head size 128 keeps tiles of 64 (LDS)
+  if (d == 64) return tile_keys == 128 ? launch_attention_mfma<64, 128>(ZA_AM_ARGS)
+                                       : launch_attention_mfma<64, 64>(ZA_AM_ARGS);
+  return launch_attention_mfma<128, 64>(ZA_AM_ARGS);
+#undef ZA_AM_ARGS
 }
 
 // Matrix-core decode variant: bfloat16, head_dim 64 or 128, page sizes that are

@@ -40,7 +40,7 @@ _SIGNATURES = {
     ("attention", "za_paged_attention_mfma"): [c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                                c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                                c_int, c_void_p, c_void_p, c_int, c_int, c_int,
-                                               c_int, c_float, c_int, c_int, c_int, c_void_p],
+                                               c_int, c_float, c_int, c_int, c_int, c_int, c_void_p],
     ("attention", "za_paged_attention_decode_mfma"): [c_void_p, c_void_p, c_void_p, c_void_p,
                                                       c_int, c_void_p, c_void_p, c_void_p,
                                                       c_void_p, c_int, c_int, c_void_p, c_void_p,
@@ -654,13 +654,16 @@ def paged_attention_mfma(q: torch.Tensor, kv_cache: torch.Tensor, block_table: t
                          positions: torch.Tensor, item_seq: torch.Tensor,
                          item_row0: torch.Tensor, item_count: torch.Tensor, n_items: int,
                          scale: float, window: int = 0, keys_per_split: int = 0,
-                         nsplit: int = 1) -> torch.Tensor:
+                         nsplit: int = 1, tile_keys: int = 64) -> torch.Tensor:
     """The same attention on the matrix cores (bfloat16, head_dim 64 or 128, at most
     16 query heads per key/value head, a page size that is a multiple of 4, a
     positive scale).  Work items hold at most
     ``ATTENTION_MFMA_ROWS // (heads // kv_heads)`` query tokens; long contexts may be
     cut into ``nsplit`` ranges of ``keys_per_split`` keys (a portion of a prompt far
-    into its request yields few work items)."""
+    into its request yields few work items).  ``tile_keys``: 64, or 128 for long contexts
+    (head_dim 64 only; head_dim 128 always takes 64)."""
+    if tile_keys not in (64, 128):
+        raise KernelError(f"tile_keys must be 64 or 128, got {tile_keys}")
     if q.dim() != 3:
         raise KernelError(f"q must be [T, heads, head_dim], got {tuple(q.shape)}")
     T, nh, d = q.shape
@@ -692,7 +695,7 @@ def paged_attention_mfma(q: torch.Tensor, kv_cache: torch.Tensor, block_table: t
         _ptr(q), _ptr(out), _ptr(kv_cache), _ptr(block_table), block_table.shape[1],
         _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
         _ptr(part_acc), _ptr(part_ml), nh, nkv, d, page_size, float(scale), int(window),
-        int(keys_per_split), int(nsplit), _stream())
+        int(keys_per_split), int(nsplit), int(tile_keys), _stream())
     _check(rc, "paged_attention_mfma")
     _note("attention", kernel="mfma", rows=T, dtype=q.dtype, nsplit=int(nsplit))
     return out

@@ -160,9 +160,11 @@ class GroupedQueryAttention(Mixer):
             items = step.attention_items(self.mfma_rows_per_item)
             # a portion far into a long request yields few work items: cut its context
             keys, nsplit = plan_split(items[3], nkv, step.max_keys, target=BUSY_WORKGROUPS)
+            # tiles of 128 keys spread a tile's fixed work over twice the scores (measured
+            # faster from 512 tokens to 32,768); head size 128 keeps tiles of 64 (LDS)
             o = ops.paged_attention_mfma(q, cache.kv, step.block_tables[cache.group],
                                          step.positions, *items, self.scale, self.window,
-                                         keys, nsplit)
+                                         keys, nsplit, tile_keys=128 if d == 64 else 64)
         elif mfma:
             # single tokens only: the matrix-core kernel whose waves split the keys
             # (every request brings one token: row i is request i, no work-item arrays)
