@@ -16,7 +16,9 @@
 // differ from each other in rounding only).
 #include "common.h"
 
+#include <mutex>
 #include <type_traits>
+#include <vector>
 
 // ---------------------------------------------------------------- 32-bit FMA
 #define F32_BM 64
@@ -373,7 +375,135 @@ __device__ __forceinline__ float normed_row_scale(const float (&ssw)[NW][16], in
   return 1.0f / sqrtf(total / (float)K + eps);
 }
 
-template <int NW, int KSTEPS, typename TC, bool NORM>
+// Up to eight rows reach the waves through LDS instead (STAGED): a wave reads its slice
+// of K of every row with one or two instructions a row, whole cache lines side by side,
+// and takes the fragments out of LDS.  The fragment loads above ask for every line of
+// the rows twice (each instruction takes 64 bytes of 16 rows), and with hundreds of
+// workgroups asking for the same few lines at a kernel's start that is what a step of
+// few rows waits for: measured at 8 rows, gate|up of 8192 x 2048, 15.1 us with fragment
+// loads, 14.3 staged, 13.4 with no rows at all.  A staged row of a wave's slice takes
+// ROWS16_STAGE_STRIDE elements (eight more than the slice: the sixteen lanes that read
+// one step of sixteen rows then fall into different banks).
+#define ROWS16_STAGE_STRIDE (16 * 32 + 8)
+#define ROWS16_STAGE_ROWS 8
+extern __shared__ __attribute__((aligned(16))) unsigned char rows16_staged[];
+
+__host__ __device__ inline size_t rows16_stage_bytes(int nw, int M) {
+  return (size_t)nw * M * ROWS16_STAGE_STRIDE * sizeof(bf16_t);
+}
+
+// The fragments of the wave's slice, out of the rows it staged itself (LDS operations of
+// one wave run in order: no barrier).  A lane without a row reads row 0.
+template <int KSTEPS>
+__device__ __forceinline__ void staged_fragments(bf16x8_t (&xa)[KSTEPS], const bf16_t* mine, int M,
+                                                 int lane) {
+  const int frag_row = lane & 15, frag_k = (lane >> 4) * 8;
+  const bf16_t* fr = mine + (frag_row < M ? frag_row : 0) * ROWS16_STAGE_STRIDE + frag_k;
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s) xa[s] = *reinterpret_cast<const bf16x8_t*>(fr + s * 32);
+}
+
+// bfloat16 rows A [M, K], M <= ROWS16_STAGE_ROWS; `kslice` is the first k of the wave's
+// slice.  K is a multiple of 8, so a lane's eight elements are inside K or outside
+// together; outside, zeros are staged (the address read is moved inside the operand).
+template <int KSTEPS>
+__device__ __forceinline__ void stage_rows(bf16x8_t (&xa)[KSTEPS], const bf16_t* __restrict__ A,
+                                           int M, int K, int kslice, bf16_t* mine, int lane) {
+  static_assert(KSTEPS == 16, "one instruction of a wave covers a row's slice of 512 elements");
+  const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int k = kslice + lane * 8;
+  const bool kin = k < K;
+  const bf16_t* src = A + (kin ? k : 0);
+  bf16x8_t v[ROWS16_STAGE_ROWS];
+#pragma unroll
+  for (int r = 0; r < ROWS16_STAGE_ROWS; ++r)
+    if (r < M) v[r] = *reinterpret_cast<const bf16x8_t*>(src + (size_t)r * K);
+#pragma unroll
+  for (int r = 0; r < ROWS16_STAGE_ROWS; ++r)
+    if (r < M)
+      *reinterpret_cast<bf16x8_t*>(mine + r * ROWS16_STAGE_STRIDE + lane * 8) = kin ? v[r] : zero8;
+  staged_fragments<KSTEPS>(xa, mine, M, lane);
+}
+
+// load_normed_rows for M <= ROWS16_STAGE_ROWS through LDS: a lane reads four elements of
+// each half of the slice of every row, adds up their squares, and stages
+// bf16(x * weight).  The lanes' sums of squares of the eight rows meet in a butterfly
+// that halves the rows a lane carries at each of its first three steps: ten exchanges
+// instead of six a row, and the same tree of additions for every row wherever it stands.
+template <int NW, int KSTEPS, typename Prefetch>
+__device__ __forceinline__ void stage_normed_rows(bf16x8_t (&xa)[KSTEPS],
+                                                  const float* __restrict__ x,
+                                                  const int* __restrict__ rows,
+                                                  const float* __restrict__ weight, int M, int K,
+                                                  int tid, float (&ssw)[NW][16], bf16_t* staged,
+                                                  Prefetch&& prefetch) {
+  static_assert(KSTEPS == 16, "two instructions of a wave cover a row's slice of 512 elements");
+  const int lane = tid & 63, wave = tid >> 6;
+  const bool inside = (wave + 1) * (KSTEPS * 32) <= K;      // the same for a whole wave
+  bf16_t* mine = staged + (size_t)wave * M * ROWS16_STAGE_STRIDE;
+  if (inside) {
+    const int kw = wave * (KSTEPS * 32) + lane * 4;
+    f32x4_t v[ROWS16_STAGE_ROWS][2];
+#pragma unroll
+    for (int r = 0; r < ROWS16_STAGE_ROWS; ++r)
+      if (r < M) {
+        const float* src = x + (rows ? (size_t)rows[r] : (size_t)r) * K + kw;
+        v[r][0] = *reinterpret_cast<const f32x4_t*>(src);
+        v[r][1] = *reinterpret_cast<const f32x4_t*>(src + 256);
+      }
+    const f32x4_t n0 = *reinterpret_cast<const f32x4_t*>(weight + kw);
+    const f32x4_t n1 = *reinterpret_cast<const f32x4_t*>(weight + kw + 256);
+    // the first weights are requested behind the rows and arrive while the rows are
+    // worked on (loads return in the order in which they were issued)
+    __builtin_amdgcn_sched_barrier(0);
+    prefetch();
+    __builtin_amdgcn_sched_barrier(0);
+    float p[ROWS16_STAGE_ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS16_STAGE_ROWS; ++r) {
+      p[r] = 0.f;
+      if (r < M) {
+        bf16x4_t lo, hi;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float a = v[r][0][e], b = v[r][1][e];
+          p[r] += a * a;
+          p[r] += b * b;
+          lo[e] = (bf16_t)(a * n0[e]);
+          hi[e] = (bf16_t)(b * n1[e]);
+        }
+        bf16_t* dst = mine + r * ROWS16_STAGE_STRIDE + lane * 4;
+        *reinterpret_cast<bf16x4_t*>(dst) = lo;
+        *reinterpret_cast<bf16x4_t*>(dst + 256) = hi;
+      }
+    }
+    // rows 4-7 go to the upper half of the lanes, then rows 2-3 and 6-7 to the lanes with
+    // bit 4, then the odd rows to the lanes with bit 3; three plain steps finish the sums
+    float q[4], t[2];
+    const bool b5 = lane & 32, b4 = lane & 16, b3 = lane & 8;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      q[i] = (b5 ? p[i + 4] : p[i]) + __shfl_xor(b5 ? p[i] : p[i + 4], 32, ZA_WAVE);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      t[i] = (b4 ? q[i + 2] : q[i]) + __shfl_xor(b4 ? q[i] : q[i + 2], 16, ZA_WAVE);
+    float u = (b3 ? t[1] : t[0]) + __shfl_xor(b3 ? t[0] : t[1], 8, ZA_WAVE);
+    u += __shfl_xor(u, 4, ZA_WAVE);
+    u += __shfl_xor(u, 2, ZA_WAVE);
+    u += __shfl_xor(u, 1, ZA_WAVE);
+    const int row = (b5 ? 4 : 0) + (b4 ? 2 : 0) + (b3 ? 1 : 0);
+    if ((lane & 7) == 0) ssw[wave][row] = u;
+    staged_fragments<KSTEPS>(xa, mine, M, lane);
+  } else {
+    const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) xa[s] = zero8;
+    if (lane < ROWS16_STAGE_ROWS) ssw[wave][lane] = 0.f;
+  }
+  __syncthreads();
+}
+
+template <int NW, int KSTEPS, typename TC, bool NORM, bool STAGED, bool ROLL>
 __global__ void __launch_bounds__(NW * 64, 2)
 gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
                         const bf16_t* __restrict__ W, const float* __restrict__ bias,
@@ -381,7 +511,7 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
                         int accumulate) {
   __shared__ float red[2][NW][64][4];
   __shared__ float ssw[NW][16];
-  __shared__ float nws[NORM ? NW * KSTEPS * 32 : 1];
+  __shared__ float nws[NORM && !STAGED ? NW * KSTEPS * 32 : 1];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int frag_row = lane & 15, frag_k = (lane >> 4) * 8;
@@ -395,15 +525,36 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
   // group's while the rows are on their way
   [[maybe_unused]] bf16x8_t fn[NORM ? KSTEPS : 1];
   [[maybe_unused]] const bool inside = (wave + 1) * (KSTEPS * 32) <= K;
-  [[maybe_unused]] auto load_group = [&](int g) {
-    const int wrow = min((int)(blockIdx.x * groups_per_block + g) * 16 + frag_row, N - 1);
+  [[maybe_unused]] auto load_first = [&](auto first, auto last) {
+    const int wrow = min((int)(blockIdx.x * groups_per_block) * 16 + frag_row, N - 1);
     const bf16_t* wp = W + (size_t)wrow * K + kbase;
 #pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) fn[s] = *reinterpret_cast<const bf16x8_t*>(wp + s * 32);
+    for (int s = first; s < last; ++s) fn[s] = *reinterpret_cast<const bf16x8_t*>(wp + s * 32);
   };
-  if constexpr (NORM) {
+  constexpr std::integral_constant<int, 0> S0{};
+  constexpr std::integral_constant<int, KSTEPS / 2> S1{};
+  constexpr std::integral_constant<int, KSTEPS> S2{};
+  [[maybe_unused]] bf16_t* staged = reinterpret_cast<bf16_t*>(rows16_staged);
+  if constexpr (NORM && STAGED) {
+    // the rows take a quarter of the registers while they are on their way: the whole
+    // first group is requested with them
+    stage_normed_rows<NW, KSTEPS>(xa, normed.x, normed.rows, normed.weight, M, K, tid, ssw,
+                                  staged, [&]() { load_first(S0, S2); });
+  } else if constexpr (NORM && ROLL) {
+    // the first half of the first group with the rows (whose 32-bit values fill half of
+    // the registers meanwhile), the second half once they are converted
     load_normed_rows<NW, KSTEPS>(xa, normed.x, normed.rows, normed.weight, M, K, tid, kbase,
-                                 ssw, nws, [&]() { load_group(0); });
+                                 ssw, nws, [&]() { load_first(S0, S1); });
+    if (inside) {
+      load_first(S1, S2);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  } else if constexpr (NORM) {
+    load_normed_rows<NW, KSTEPS>(xa, normed.x, normed.rows, normed.weight, M, K, tid, kbase,
+                                 ssw, nws, [&]() { load_first(S0, S2); });
+  } else if constexpr (STAGED) {
+    stage_rows<KSTEPS>(xa, A, M, K, (blockIdx.y * NW + wave) * KSTEPS * 32,
+                       staged + (size_t)wave * M * ROWS16_STAGE_STRIDE, lane);
   } else {
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) {
@@ -414,19 +565,32 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
   }
 
   const bool partial = gridDim.y > 1 && !accumulate;
-  for (int g = 0; g < groups_per_block; ++g) {
+  // One row group; `more` (a compile-time flag): another group of this workgroup follows.
+  auto row_group = [&](int g, auto more, auto burst) {
     const int n0 = (blockIdx.x * groups_per_block + g) * 16;
-    if (n0 >= N) break;
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
     if constexpr (NORM) {
       if (inside) {
-        if (g > 0) {
-          load_group(g);
-          __builtin_amdgcn_sched_barrier(0);   // every load is requested before the first product
-        }
+        if constexpr (decltype(burst)::value) {
+          if (g > 0) {
+            const bf16_t* wp = W + (size_t)min(n0 + frag_row, N - 1) * K + kbase;
 #pragma unroll
-        for (int s = 0; s < KSTEPS; ++s)
+            for (int s = 0; s < KSTEPS; ++s) fn[s] = *reinterpret_cast<const bf16x8_t*>(wp + s * 32);
+            __builtin_amdgcn_sched_barrier(0);   // every load is requested before the first product
+          }
+        }
+        // `more`: the next row group's fragments are requested one by one into the registers
+        // that the products free, so the wave's requests to memory never run dry between groups
+        [[maybe_unused]] const bf16_t* nxt =
+            W + (size_t)min(n0 + 16 + frag_row, N - 1) * K + kbase;
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
           acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fn[s], xa[s], acc, 0, 0, 0);
+          if constexpr (decltype(more)::value) {
+            fn[s] = *reinterpret_cast<const bf16x8_t*>(nxt + s * 32);
+            __builtin_amdgcn_sched_barrier(0);   // in this order: the compiler would bunch the loads
+          }
+        }
       }
     } else {
       const int wrow = n0 + frag_row;
@@ -479,6 +643,19 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
         }
       }
     }
+  };
+  // the row groups of this workgroup that lie inside N (at least one: the grid is made so)
+  const int first = blockIdx.x * groups_per_block;
+  const int count = min(groups_per_block, (N + 15) / 16 - first);
+  // ROLL (two groups a workgroup): the second is requested while the first is multiplied.
+  // With more (the output head: two workgroups a compute unit take turns) a group requested
+  // whole before its products measured faster (8 rows, 65536 x 2048: 52.5 against 53.8 us).
+  if constexpr (ROLL) {
+    int g = 0;
+    for (; g + 1 < count; ++g) row_group(g, std::true_type{}, std::false_type{});
+    row_group(g, std::false_type{}, std::false_type{});
+  } else {
+    for (int g = 0; g < count; ++g) row_group(g, std::false_type{}, std::true_type{});
   }
 }
 
@@ -488,14 +665,14 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
 //   C[m, n] = silu(gate[m, n]) * up[m, n],   silu(g) = g / (1 + exp(-g)),
 // from the 32-bit accumulators (/root/reference/src/transformer/ffn.zig:24-30), so
 // the [M, 2I] intermediate never goes to memory.  K is not split over workgroups.
-template <int NW, int KSTEPS, bool NORM>
+template <int NW, int KSTEPS, bool NORM, bool STAGED>
 __global__ void __launch_bounds__(NW * 64, 2)
 gemm_bf16_rows16_swiglu_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
                                const bf16_t* __restrict__ W, bf16_t* __restrict__ C, int M, int I,
                                int K, int groups_per_block) {
   __shared__ float red[2][2][NW][64][4];
   __shared__ float ssw[NW][16];
-  __shared__ float nws[NORM ? NW * KSTEPS * 32 : 1];
+  __shared__ float nws[NORM && !STAGED ? NW * KSTEPS * 32 : 1];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int frag_row = lane & 15, frag_k = (lane >> 4) * 8;
@@ -505,8 +682,8 @@ gemm_bf16_rows16_swiglu_kernel(const bf16_t* __restrict__ A, NormedRowsArg norme
 
   bf16x8_t xa[KSTEPS];
   // NORM: as in gemm_bf16_rows16_kernel, with all of a row group's gate and up rows in
-  // registers; the first group's first half is requested with the rows, its second half
-  // once the rows' registers are free
+  // registers; the first group's first quarter is requested with the rows (whose 32-bit
+  // values fill half of the registers meanwhile), the rest once they are converted
   [[maybe_unused]] bf16x8_t ng[NORM ? KSTEPS : 1], nu[NORM ? KSTEPS : 1];
   [[maybe_unused]] const bool inside = (wave + 1) * (KSTEPS * 32) <= K;
   [[maybe_unused]] auto load_steps = [&](int g, auto first, auto last) {
@@ -520,11 +697,20 @@ gemm_bf16_rows16_swiglu_kernel(const bf16_t* __restrict__ A, NormedRowsArg norme
     }
   };
   constexpr std::integral_constant<int, 0> S0{};
-  constexpr std::integral_constant<int, KSTEPS / 2> S1{};
+  constexpr std::integral_constant<int, KSTEPS / (STAGED ? 2 : 4)> S1{};
   constexpr std::integral_constant<int, KSTEPS> S2{};
-  if constexpr (NORM) {
+  [[maybe_unused]] bf16_t* staged = reinterpret_cast<bf16_t*>(rows16_staged);
+  if constexpr (NORM && STAGED) {
+    // (the rows take a quarter of the registers on their way: half of the first group
+    // is requested with them)
+    stage_normed_rows<NW, KSTEPS>(xa, normed.x, normed.rows, normed.weight, M, K, tid, ssw,
+                                  staged, [&]() { load_steps(0, S0, S1); });
+  } else if constexpr (NORM) {
     load_normed_rows<NW, KSTEPS>(xa, normed.x, normed.rows, normed.weight, M, K, tid, kbase,
                                  ssw, nws, [&]() { load_steps(0, S0, S1); });
+  } else if constexpr (STAGED) {
+    stage_rows<KSTEPS>(xa, A, M, K, wave * KSTEPS * 32,
+                       staged + (size_t)wave * M * ROWS16_STAGE_STRIDE, lane);
   } else {
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) {
@@ -534,19 +720,38 @@ gemm_bf16_rows16_swiglu_kernel(const bf16_t* __restrict__ A, NormedRowsArg norme
     }
   }
 
-  for (int g = 0; g < groups_per_block; ++g) {
+  if constexpr (NORM) {
+    if (inside) {
+      load_steps(0, S1, S2);
+      __builtin_amdgcn_sched_barrier(0);   // every load is requested before the first product
+    }
+  }
+  // One row group; `more` (a compile-time flag): another group of this workgroup follows.
+  auto row_group = [&](int g, auto more, auto burst) {
     const int n0 = (blockIdx.x * groups_per_block + g) * 16;
-    if (n0 >= I) break;
     f32x4_t ag = {0.f, 0.f, 0.f, 0.f}, au = {0.f, 0.f, 0.f, 0.f};
     if constexpr (NORM) {
       if (inside) {
-        if (g > 0) load_steps(g, S0, S1);
-        load_steps(g, S1, S2);
-        __builtin_amdgcn_sched_barrier(0);   // every load is requested before the first product
+        if constexpr (decltype(burst)::value) {
+          if (g > 0) {
+            load_steps(g, S0, S2);
+            __builtin_amdgcn_sched_barrier(0);   // every load is requested before the first product
+          }
+        }
+        // `more`: the next row group's fragments are requested one by one into the registers
+        // that the products free, so the wave's requests to memory never run dry between groups
+        [[maybe_unused]] const bf16_t* ngp =
+            W + (size_t)min(n0 + 16 + frag_row, I - 1) * K + kbase;
+        [[maybe_unused]] const bf16_t* nup = ngp + (size_t)I * K;
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
           ag = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ng[s], xa[s], ag, 0, 0, 0);
           au = __builtin_amdgcn_mfma_f32_16x16x32_bf16(nu[s], xa[s], au, 0, 0, 0);
+          if constexpr (decltype(more)::value) {
+            ng[s] = *reinterpret_cast<const bf16x8_t*>(ngp + s * 32);
+            nu[s] = *reinterpret_cast<const bf16x8_t*>(nup + s * 32);
+            __builtin_amdgcn_sched_barrier(0);   // in this order: the compiler would bunch the loads
+          }
         }
       }
     } else {
@@ -605,12 +810,37 @@ gemm_bf16_rows16_swiglu_kernel(const bf16_t* __restrict__ A, NormedRowsArg norme
         }
       }
     }
-  }
+  };
+  // the row groups of this workgroup that lie inside I (at least one: the grid is made so)
+  const int first = blockIdx.x * groups_per_block;
+  const int count = min(groups_per_block, (I + 15) / 16 - first);
+  int g = 0;
+  for (; g + 1 < count; ++g) row_group(g, std::true_type{}, std::false_type{});
+  row_group(g, std::false_type{}, std::false_type{});
 }
 
 // `normed` (with normed->x set) replaces the bfloat16 activations `a` by rows of the
 // 32-bit stream that the kernel normalises itself; it needs one workgroup to cover K
 // with 16 steps a wave (K <= 4096, a multiple of 512) and K not split over workgroups.
+// A workgroup may ask for 64 KB of LDS at launch; a kernel that wants more (eight waves
+// staging eight rows) is told so once.  The kernels are few: a short list remembers them.
+static int rows16_allow_lds(const void* kernel, size_t bytes) {
+  if (bytes <= 48 * 1024) return 0;
+  static std::mutex guard;
+  static std::vector<const void*> allowed;
+  std::lock_guard<std::mutex> lock(guard);
+  for (const void* k : allowed)
+    if (k == kernel) return 0;
+  const hipError_t rc =
+      hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+  if (rc != hipSuccess) {
+    (void)hipGetLastError();
+    return (int)rc;
+  }
+  allowed.push_back(kernel);
+  return 0;
+}
+
 static bool rows16_takes_norm(int K, int ksplit) {
   return ksplit == 1 && K <= 4096 && K % 512 == 0;
 }
@@ -638,22 +868,38 @@ static int launch_rows16(const bf16_t* a, const NormedRowsArg* normed, const bf1
   if (groups_per_block > 0) per_block = groups_per_block;
   dim3 grid((groups + per_block - 1) / per_block, ksplit);
   const NormedRowsArg none = {nullptr, nullptr, nullptr, 0.f};
-#define ZA_R16_LAUNCH(NW, KS, TC, NORM)                                                       \
-  hipLaunchKernelGGL((gemm_bf16_rows16_kernel<NW, KS, TC, NORM>), grid, dim3(NW * 64), 0,     \
-                     stream, a, NORM ? *normed : none, w, bias, (TC*)C, M, N, K, per_block,   \
-                     accumulate)
+  // up to ROWS16_STAGE_ROWS rows go through LDS (16 steps a wave only)
+  const bool stage = M <= ROWS16_STAGE_ROWS;
+#define ZA_R16_LAUNCH(NW, KS, TC, NORM, STAGED, ROLL)                                         \
+  {                                                                                           \
+    const size_t lds = STAGED ? rows16_stage_bytes(NW, M) : 0;                                \
+    auto kernel = gemm_bf16_rows16_kernel<NW, KS, TC, NORM, STAGED, ROLL>;                    \
+    if (const int rc = rows16_allow_lds((const void*)kernel, lds)) return rc;                         \
+    hipLaunchKernelGGL(kernel, grid, dim3(NW * 64), lds, stream, a, NORM ? *normed : none, w, \
+                       bias, (TC*)C, M, N, K, per_block, accumulate);                         \
+  }
+#define ZA_R16_TYPES(NW, KS, NORM, STAGED, ROLL)                                              \
+  {                                                                                           \
+    if (c_dtype == 0) ZA_R16_LAUNCH(NW, KS, float, NORM, STAGED, ROLL)                        \
+    else ZA_R16_LAUNCH(NW, KS, bf16_t, NORM, STAGED, ROLL)                                    \
+  }
+#define ZA_R16_NORM(NW, KS, STAGED)                                                           \
+  {                                                                                           \
+    if (per_block <= 2) ZA_R16_TYPES(NW, KS, true, STAGED, true)                              \
+    else ZA_R16_TYPES(NW, KS, true, STAGED, false)                                            \
+  }
 #define ZA_R16_CASE(NW, KS)                                                                   \
   {                                                                                           \
-    if (norm) {                                                                               \
-      if constexpr (KS == 16) {                                                               \
-        if (c_dtype == 0) ZA_R16_LAUNCH(NW, KS, float, true);                                 \
-        else ZA_R16_LAUNCH(NW, KS, bf16_t, true);                                             \
+    if constexpr (KS == 16) {                                                                 \
+      if (norm) {                                                                             \
+        if (stage) ZA_R16_NORM(NW, KS, true) else ZA_R16_NORM(NW, KS, false)                  \
       } else {                                                                                \
-        return ZA_ERR_UNSUPPORTED;                                                            \
+        if (stage) ZA_R16_TYPES(NW, KS, false, true, false)                                   \
+        else ZA_R16_TYPES(NW, KS, false, false, false)                                        \
       }                                                                                       \
     } else {                                                                                  \
-      if (c_dtype == 0) ZA_R16_LAUNCH(NW, KS, float, false);                                  \
-      else ZA_R16_LAUNCH(NW, KS, bf16_t, false);                                              \
+      if (norm) return ZA_ERR_UNSUPPORTED;                                                    \
+      ZA_R16_TYPES(NW, KS, false, false, false)                                               \
     }                                                                                         \
     return za_launch_status();                                                                \
   }
@@ -663,6 +909,8 @@ static int launch_rows16(const bf16_t* a, const NormedRowsArg* normed, const bf1
   if (kper <= 4096) ZA_R16_CASE(8, 16)
   ZA_R16_CASE(8, 32)
 #undef ZA_R16_CASE
+#undef ZA_R16_NORM
+#undef ZA_R16_TYPES
 #undef ZA_R16_LAUNCH
 }
 
@@ -780,17 +1028,26 @@ extern "C" int za_gemm_bf16_rows16_swiglu(const void* A, const float* x, const i
   // 8 rows, I = 8192: 18.1 -> 16.9 us)
   const int per_block = groups >= 2048 ? 4 : (norm && groups >= 384 ? 2 : 1);
   dim3 grid((groups + per_block - 1) / per_block);
-#define ZA_SG_LAUNCH(NW, KS, NORM)                                                            \
-  hipLaunchKernelGGL((gemm_bf16_rows16_swiglu_kernel<NW, KS, NORM>), grid, dim3(NW * 64), 0,  \
-                     stream, (const bf16_t*)A, normed, (const bf16_t*)W, (bf16_t*)C, M, I, K, \
-                     per_block)
+  const bool stage = M <= ROWS16_STAGE_ROWS;
+#define ZA_SG_LAUNCH(NW, KS, NORM, STAGED)                                                    \
+  {                                                                                           \
+    const size_t lds = STAGED ? rows16_stage_bytes(NW, M) : 0;                                \
+    auto kernel = gemm_bf16_rows16_swiglu_kernel<NW, KS, NORM, STAGED>;                       \
+    if (const int rc = rows16_allow_lds((const void*)kernel, lds)) return rc;                         \
+    hipLaunchKernelGGL(kernel, grid, dim3(NW * 64), lds, stream, (const bf16_t*)A, normed,    \
+                       (const bf16_t*)W, (bf16_t*)C, M, I, K, per_block);                     \
+  }
 #define ZA_SG_CASE(NW, KS)                                                                    \
   {                                                                                           \
-    if (norm) {                                                                               \
-      if constexpr (KS == 16) ZA_SG_LAUNCH(NW, KS, true);                                     \
-      else return ZA_ERR_UNSUPPORTED;                                                         \
+    if constexpr (KS == 16) {                                                                 \
+      if (norm) {                                                                             \
+        if (stage) ZA_SG_LAUNCH(NW, KS, true, true) else ZA_SG_LAUNCH(NW, KS, true, false)    \
+      } else {                                                                                \
+        if (stage) ZA_SG_LAUNCH(NW, KS, false, true) else ZA_SG_LAUNCH(NW, KS, false, false)  \
+      }                                                                                       \
     } else {                                                                                  \
-      ZA_SG_LAUNCH(NW, KS, false);                                                            \
+      if (norm) return ZA_ERR_UNSUPPORTED;                                                    \
+      ZA_SG_LAUNCH(NW, KS, false, false)                                                      \
     }                                                                                         \
     return za_launch_status();                                                                \
   }
