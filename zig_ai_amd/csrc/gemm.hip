@@ -406,9 +406,10 @@ __device__ __forceinline__ void staged_fragments(bf16x8_t (&xa)[KSTEPS], const b
 // bfloat16 rows A [M, K], M <= ROWS16_STAGE_ROWS; `kslice` is the first k of the wave's
 // slice.  K is a multiple of 8, so a lane's eight elements are inside K or outside
 // together; outside, zeros are staged (the address read is moved inside the operand).
-template <int KSTEPS>
+template <int KSTEPS, typename Prefetch>
 __device__ __forceinline__ void stage_rows(bf16x8_t (&xa)[KSTEPS], const bf16_t* __restrict__ A,
-                                           int M, int K, int kslice, bf16_t* mine, int lane) {
+                                           int M, int K, int kslice, bf16_t* mine, int lane,
+                                           Prefetch&& prefetch) {
   static_assert(KSTEPS == 16, "one instruction of a wave covers a row's slice of 512 elements");
   const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   const int k = kslice + lane * 8;
@@ -418,6 +419,10 @@ __device__ __forceinline__ void stage_rows(bf16x8_t (&xa)[KSTEPS], const bf16_t*
 #pragma unroll
   for (int r = 0; r < ROWS16_STAGE_ROWS; ++r)
     if (r < M) v[r] = *reinterpret_cast<const bf16x8_t*>(src + (size_t)r * K);
+  // (weights requested behind the rows arrive while the rows pass through LDS)
+  __builtin_amdgcn_sched_barrier(0);
+  prefetch();
+  __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int r = 0; r < ROWS16_STAGE_ROWS; ++r)
     if (r < M)
@@ -520,11 +525,13 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
   constexpr int HALF = KSTEPS > 16 ? 16 : KSTEPS;   // weight fragments in flight at once
 
   bf16x8_t xa[KSTEPS];
-  // NORM: a wave is all inside K or idle, and a row group's weights are loaded without
-  // conditions (a lane beyond N reads row N - 1; its sums are never stored), the first
-  // group's while the rows are on their way
-  [[maybe_unused]] bf16x8_t fn[NORM ? KSTEPS : 1];
-  [[maybe_unused]] const bool inside = (wave + 1) * (KSTEPS * 32) <= K;
+  // FAST (the norm in the kernel, or staged rows: K is then a multiple of a wave's slice):
+  // a wave is all inside K or idle, and a row group's weights are loaded without conditions
+  // (a lane beyond N reads row N - 1; its sums are never stored), the first group's while
+  // the rows are on their way
+  constexpr bool FAST = NORM || STAGED;
+  [[maybe_unused]] bf16x8_t fn[FAST ? KSTEPS : 1];
+  [[maybe_unused]] const bool inside = (int)(blockIdx.y * NW + wave + 1) * (KSTEPS * 32) <= K;
   [[maybe_unused]] auto load_first = [&](auto first, auto last) {
     const int wrow = min((int)(blockIdx.x * groups_per_block) * 16 + frag_row, N - 1);
     const bf16_t* wp = W + (size_t)wrow * K + kbase;
@@ -553,8 +560,14 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
     load_normed_rows<NW, KSTEPS>(xa, normed.x, normed.rows, normed.weight, M, K, tid, kbase,
                                  ssw, nws, [&]() { load_first(S0, S2); });
   } else if constexpr (STAGED) {
-    stage_rows<KSTEPS>(xa, A, M, K, (blockIdx.y * NW + wave) * KSTEPS * 32,
-                       staged + (size_t)wave * M * ROWS16_STAGE_STRIDE, lane);
+    if (inside) {
+      stage_rows<KSTEPS>(xa, A, M, K, (blockIdx.y * NW + wave) * KSTEPS * 32,
+                         staged + (size_t)wave * M * ROWS16_STAGE_STRIDE, lane,
+                         [&]() { load_first(S0, S2); });
+    } else {
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) xa[s] = zero8;
+    }
   } else {
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) {
@@ -569,7 +582,7 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
   auto row_group = [&](int g, auto more, auto burst) {
     const int n0 = (blockIdx.x * groups_per_block + g) * 16;
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-    if constexpr (NORM) {
+    if constexpr (FAST) {
       if (inside) {
         if constexpr (decltype(burst)::value) {
           if (g > 0) {
@@ -710,7 +723,7 @@ gemm_bf16_rows16_swiglu_kernel(const bf16_t* __restrict__ A, NormedRowsArg norme
                                  ssw, nws, [&]() { load_steps(0, S0, S1); });
   } else if constexpr (STAGED) {
     stage_rows<KSTEPS>(xa, A, M, K, wave * KSTEPS * 32,
-                       staged + (size_t)wave * M * ROWS16_STAGE_STRIDE, lane);
+                       staged + (size_t)wave * M * ROWS16_STAGE_STRIDE, lane, []() {});
   } else {
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) {
@@ -841,6 +854,11 @@ static int rows16_allow_lds(const void* kernel, size_t bytes) {
   return 0;
 }
 
+// For tuning runs: row groups per workgroup of the decode products that take no such
+// argument (0: the launchers choose).
+static int rows16_groups_override = 0;
+extern "C" void za_gemm_rows16_set_groups_per_block(int groups) { rows16_groups_override = groups; }
+
 static bool rows16_takes_norm(int K, int ksplit) {
   return ksplit == 1 && K <= 4096 && K % 512 == 0;
 }
@@ -865,11 +883,14 @@ static int launch_rows16(const bf16_t* a, const NormedRowsArg* normed, const bf1
   // with the norm in the kernel every workgroup prepares the step's rows first: two row
   // groups share that from 384 groups on (8 rows: in_proj 10.7 -> 9.1 us)
   if (norm && per_block == 1 && groups >= 384) per_block = 2;
+  if (rows16_groups_override > 0) per_block = rows16_groups_override;
   if (groups_per_block > 0) per_block = groups_per_block;
   dim3 grid((groups + per_block - 1) / per_block, ksplit);
   const NormedRowsArg none = {nullptr, nullptr, nullptr, 0.f};
   // up to ROWS16_STAGE_ROWS rows go through LDS (16 steps a wave only)
-  const bool stage = M <= ROWS16_STAGE_ROWS;
+  // (without the norm: only where K is a multiple of a wave's slice, the condition of the
+  // kernel's loads without conditions)
+  const bool stage = M <= ROWS16_STAGE_ROWS && (norm || K % 512 == 0);
 #define ZA_R16_LAUNCH(NW, KS, TC, NORM, STAGED, ROLL)                                         \
   {                                                                                           \
     const size_t lds = STAGED ? rows16_stage_bytes(NW, M) : 0;                                \
@@ -894,7 +915,8 @@ static int launch_rows16(const bf16_t* a, const NormedRowsArg* normed, const bf1
       if (norm) {                                                                             \
         if (stage) ZA_R16_NORM(NW, KS, true) else ZA_R16_NORM(NW, KS, false)                  \
       } else {                                                                                \
-        if (stage) ZA_R16_TYPES(NW, KS, false, true, false)                                   \
+        if (stage && per_block <= 2) ZA_R16_TYPES(NW, KS, false, true, true)                  \
+        else if (stage) ZA_R16_TYPES(NW, KS, false, true, false)                              \
         else ZA_R16_TYPES(NW, KS, false, false, false)                                        \
       }                                                                                       \
     } else {                                                                                  \
@@ -1026,7 +1048,8 @@ extern "C" int za_gemm_bf16_rows16_swiglu(const void* A, const float* x, const i
   const int groups = (I + 15) / 16;
   // (with the norm in the kernel two row groups share the preparation of the step's rows:
   // 8 rows, I = 8192: 18.1 -> 16.9 us)
-  const int per_block = groups >= 2048 ? 4 : (norm && groups >= 384 ? 2 : 1);
+  int per_block = groups >= 2048 ? 4 : (norm && groups >= 384 ? 2 : 1);
+  if (rows16_groups_override > 0) per_block = rows16_groups_override;
   dim3 grid((groups + per_block - 1) / per_block);
   const bool stage = M <= ROWS16_STAGE_ROWS;
 #define ZA_SG_LAUNCH(NW, KS, NORM, STAGED)                                                    \
