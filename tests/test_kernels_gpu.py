@@ -188,6 +188,29 @@ def test_gemm_bf16_library_keeps_32_bits(M, N, K):
     assert rel_err(low, x.double() @ w.double().T) < BF16_TOL
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 2048, 2048), (700, 1000, 4096), (512, 264, 1024)])
+def test_gemm_bf16_library_candidates_timed_at_first_use(M, N, K, monkeypatch):
+    """From 256 rows on the library's candidates for a shape are timed at its first call
+    and the fastest is kept: the result is a product like any other, a second call runs
+    the same kernel (the same bits), a neighbouring row count takes the same choice, and
+    with the timing switched off the first candidate gives the same product to rounding."""
+    x, w = rand((M, K), torch.bfloat16, 140), rand((N, K), torch.bfloat16, 141)
+    exact = x.double() @ w.double().T
+    xd, wd = x.to(dev()), w.to(dev())
+    monkeypatch.setattr(ops(), "library_tuning", True)
+    first = ops().linear(xd, wd, out_dtype=torch.float32)
+    assert rel_err(first, exact) < F32_TOL
+    assert torch.equal(ops().linear(xd, wd, out_dtype=torch.float32), first)
+    near = ops().linear(xd[:M - 3].contiguous(), wd, out_dtype=torch.float32)
+    assert rel_err(near, exact[:M - 3]) < F32_TOL
+    low = ops().linear(xd, wd)
+    assert low.dtype == torch.bfloat16 and rel_err(low, exact) < BF16_TOL
+    monkeypatch.setattr(ops(), "library_tuning", False)
+    plain = ops().linear(xd, wd, out_dtype=torch.float32)
+    assert rel_err(plain, exact) < F32_TOL
+    assert torch.equal(ops().linear(xd, wd, out_dtype=torch.float32), plain)
+
+
 def test_gemm_rows_do_not_depend_on_batch():
     """A token's projection is the same whatever else is in the step: bitwise
     within one of this package's kernels (each sums over k in an order fixed by K

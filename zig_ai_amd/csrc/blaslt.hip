@@ -13,6 +13,16 @@
 // M, N, K, output type, P) and kept, so a later call is one hipblasLtMatmul, or, for
 // operands seen before, one launch of a prepared instance (see InstanceKey).
 // The same shape therefore always runs the same kernel, recorded in a graph or not.
+//
+// Which algorithm: for products of many rows (TUNE_MIN_ROWS and more) the heuristic's first
+// answer is not always the fastest on this GPU (measured at 2,048 rows, bfloat16 out:
+// [2048, 8192] weights 88 us with the first answer, 76 with the eighteenth; [2048, 2048]
+// 29 against 25; at 512 rows [16384, 2048] 39 against 34), so with `tune` the first call
+// of a shape times the first TUNE_CANDIDATES answers on the call's own operands and keeps
+// the fastest.  Shapes whose row counts fall into the same block of TUNE_BUCKET rows share
+// the choice, so a server that sees every portion length times a few dozen shapes, not
+// thousands.  Which answer wins can differ from run to run when two are close: callers
+// that want the same bits run after run pass tune = 0 and get the first answer.
 #include <hip/hip_runtime.h>
 #include <hipblaslt/hipblaslt-ext.hpp>
 #include <hipblaslt/hipblaslt.h>
@@ -23,6 +33,7 @@
 #include <mutex>
 #include <string>
 #include <tuple>
+#include <vector>
 
 #include "common.h"
 
@@ -36,9 +47,17 @@ struct Plan {
   hipblasLtMatmulAlgo_t algo;
   size_t workspace = 0;
   bool usable = false;
+  bool settled = true;   // false: the candidates are still to be timed
+  std::vector<hipblasLtMatmulHeuristicResult_t> candidates;
 };
 
-using Key = std::tuple<int, int, int, int, int, int>;   // device, M, N, K, output type, P
+constexpr int TUNE_MIN_ROWS = 256;
+constexpr int TUNE_BUCKET = 256;
+constexpr int TUNE_CANDIDATES = 24;
+
+using Key = std::tuple<int, int, int, int, int, int, int>;   // device, M, N, K, output type, P, tune
+// device, block of rows, N, K, output type, P -> the library's index of the algorithm that won
+using TunedKey = std::tuple<int, int, int, int, int, int>;
 
 // A product on given operands, with its kernel arguments made: issuing it again is one
 // launch (some 6 us less on the host than hipblasLtMatmul, which derives the arguments
@@ -62,6 +81,7 @@ size_t max_instances() {
 std::mutex g_lock;
 std::map<int, hipblasLtHandle_t> g_handles;
 std::map<Key, Plan> g_plans;
+std::map<TunedKey, int> g_tuned;
 std::map<InstanceKey, std::unique_ptr<hipblaslt_ext::Gemm>> g_instances;
 const float kOne = 1.0f, kZero = 0.0f;
 thread_local std::string g_error;
@@ -81,7 +101,7 @@ bool ok(hipblasStatus_t s, const char* what, std::string* why) {
 // times x^T (stored K x M).  A range p of K starts p * K/P elements into a row of
 // either operand; its result is the p-th [M, N] block of y.
 bool make_plan(hipblasLtHandle_t handle, int M, int N, int K, int out_f32, int P,
-               size_t workspace_bytes, Plan* plan, std::string* why) {
+               size_t workspace_bytes, bool tune, Plan* plan, std::string* why) {
   const int kp = K / P;
   const hipDataType out_type = out_f32 ? HIP_R_32F : HIP_R_16BF;
   if (!ok(hipblasLtMatmulDescCreate(&plan->op, HIPBLAS_COMPUTE_32F, HIP_R_32F), "MatmulDescCreate", why))
@@ -112,12 +132,13 @@ bool make_plan(hipblasLtHandle_t handle, int M, int N, int K, int out_f32, int P
   hipblasLtMatmulPreference_t pref = nullptr;
   if (!ok(hipblasLtMatmulPreferenceCreate(&pref), "PreferenceCreate", why)) return false;
   const uint64_t limit = workspace_bytes;
-  hipblasLtMatmulHeuristicResult_t found[1];
+  const int wanted = tune ? TUNE_CANDIDATES : 1;
+  std::vector<hipblasLtMatmulHeuristicResult_t> found(wanted);
   int n_found = 0;
   bool good = ok(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES,
                                                        &limit, sizeof(limit)), "set workspace limit", why) &&
               ok(hipblasLtMatmulAlgoGetHeuristic(handle, plan->op, plan->a, plan->b, plan->c, plan->c, pref,
-                                                 1, found, &n_found), "AlgoGetHeuristic", why);
+                                                 wanted, found.data(), &n_found), "AlgoGetHeuristic", why);
   hipblasLtMatmulPreferenceDestroy(pref);
   if (!good) return false;
   if (n_found < 1 || found[0].state != HIPBLAS_STATUS_SUCCESS || found[0].workspaceSize > workspace_bytes) {
@@ -127,7 +148,60 @@ bool make_plan(hipblasLtHandle_t handle, int M, int N, int K, int out_f32, int P
   plan->algo = found[0].algo;
   plan->workspace = found[0].workspaceSize;
   plan->usable = true;
+  if (tune) {
+    for (int i = 0; i < n_found; ++i)
+      if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize <= workspace_bytes)
+        plan->candidates.push_back(found[i]);
+    plan->settled = plan->candidates.size() < 2;
+  }
   return true;
+}
+
+// Times the plan's candidates on the call's operands (y is overwritten by every one of
+// them, and by the product proper afterwards) and returns the fastest: one run to warm
+// up, then TUNE_RUNS timed together.  The stream is waited for; this happens once per
+// block of row counts.  A candidate that fails, or takes three times the best so far in
+// its first run, is out.
+constexpr int TUNE_RUNS = 3;
+int fastest_candidate(hipblasLtHandle_t handle, const Plan& plan, const void* x, const void* w,
+                      void* y, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  hipEvent_t t0 = nullptr, t1 = nullptr;
+  if (hipEventCreate(&t0) != hipSuccess || hipEventCreate(&t1) != hipSuccess) {
+    if (t0) (void)hipEventDestroy(t0);
+    (void)hipGetLastError();
+    return 0;
+  }
+  int best = 0;
+  float best_ms = -1.f;
+  for (size_t i = 0; i < plan.candidates.size(); ++i) {
+    hipblasLtMatmulAlgo_t algo = plan.candidates[i].algo;
+    auto run = [&]() {
+      return hipblasLtMatmul(handle, plan.op, &kOne, w, plan.a, x, plan.b, &kZero, y, plan.c, y,
+                             plan.c, &algo, workspace, workspace_bytes, stream) == HIPBLAS_STATUS_SUCCESS;
+    };
+    float ms = 0.f;
+    if (hipEventRecord(t0, stream) != hipSuccess || !run() || hipEventRecord(t1, stream) != hipSuccess ||
+        hipEventSynchronize(t1) != hipSuccess || hipEventElapsedTime(&ms, t0, t1) != hipSuccess) {
+      (void)hipGetLastError();
+      continue;
+    }
+    if (best_ms > 0.f && ms > 3.f * best_ms) continue;
+    bool fine = hipEventRecord(t0, stream) == hipSuccess;
+    for (int r = 0; r < TUNE_RUNS && fine; ++r) fine = run();
+    if (!fine || hipEventRecord(t1, stream) != hipSuccess || hipEventSynchronize(t1) != hipSuccess ||
+        hipEventElapsedTime(&ms, t0, t1) != hipSuccess) {
+      (void)hipGetLastError();
+      continue;
+    }
+    ms /= TUNE_RUNS;
+    if (best_ms < 0.f || ms < best_ms) {
+      best_ms = ms;
+      best = (int)i;
+    }
+  }
+  (void)hipEventDestroy(t0);
+  (void)hipEventDestroy(t1);
+  return best;
 }
 
 }  // namespace
@@ -136,8 +210,10 @@ ZA_API const char* za_lt_last_error() { return g_error.c_str(); }
 
 // Returns 0, ZA_ERR_ARG, ZA_ERR_UNSUPPORTED (the library has no algorithm for the
 // shape: nothing was launched) or a positive hipBLAS status.
+// `tune`: see the head of this file.
 ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int K, int out_f32,
-                        int P, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+                        int P, int tune, void* workspace, size_t workspace_bytes,
+                        hipStream_t stream) {
   if (!x || !w || !y || M < 1 || N < 1 || K < 1 || P < 1 || K % P || (P > 1 && !out_f32))
     return fail(ZA_ERR_ARG, "za_lt_matmul: bad argument");
   int device = 0;
@@ -154,23 +230,54 @@ ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int
       h = g_handles.emplace(device, made).first;
     }
     handle = h->second;
-    const Key key(device, M, N, K, out_f32, P);
+    const bool tuning = tune && M >= TUNE_MIN_ROWS;
+    const Key key(device, M, N, K, out_f32, P, tuning ? 1 : 0);
     auto it = g_plans.find(key);
     if (it == g_plans.end()) {
       Plan made;
       std::string why;
-      if (!make_plan(handle, M, N, K, out_f32, P, workspace_bytes, &made, &why))
+      if (!make_plan(handle, M, N, K, out_f32, P, workspace_bytes, tuning, &made, &why))
         return fail(ZA_ERR_ARG, "za_lt_matmul: " + why);
       it = g_plans.emplace(key, made).first;
     }
-    plan = it->second;
+    Plan& kept = it->second;
+    if (kept.usable && !kept.settled) {
+      const TunedKey block(device, (M + TUNE_BUCKET - 1) / TUNE_BUCKET, N, K, out_f32, P);
+      auto choose = [&](size_t i) {
+        kept.algo = kept.candidates[i].algo;
+        kept.workspace = kept.candidates[i].workspaceSize;
+      };
+      hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+      const bool recording = hipStreamIsCapturing(stream, &capturing) != hipSuccess ||
+                             capturing != hipStreamCaptureStatusNone;
+      auto won = g_tuned.find(block);
+      if (won != g_tuned.end()) {
+        // a neighbouring row count has been timed: its winner, if it is among this
+        // shape's answers (else the first answer stays)
+        for (size_t i = 0; i < kept.candidates.size(); ++i)
+          if (hipblaslt_ext::getIndexFromAlgo(kept.candidates[i].algo) == won->second) {
+            choose(i);
+            break;
+          }
+      } else if (!recording) {
+        const int best = fastest_candidate(handle, kept, x, w, y, workspace, workspace_bytes, stream);
+        choose((size_t)best);
+        g_tuned.emplace(block, hipblaslt_ext::getIndexFromAlgo(kept.algo));
+      }
+      // (a shape first met while a stream is recorded keeps the first answer for good:
+      // the same shape always runs the same kernel)
+      kept.settled = true;
+      kept.candidates.clear();
+      kept.candidates.shrink_to_fit();
+    }
+    plan = kept;
   }
   if (!plan.usable || plan.workspace > workspace_bytes)
     return fail(ZA_ERR_UNSUPPORTED, "za_lt_matmul: the library names no algorithm for this shape");
   hipblaslt_ext::Gemm* instance = nullptr;
   {
     std::lock_guard<std::mutex> guard(g_lock);
-    const InstanceKey ikey(Key(device, M, N, K, out_f32, P), x, w, y, workspace);
+    const InstanceKey ikey(Key(device, M, N, K, out_f32, P, tune && M >= TUNE_MIN_ROWS ? 1 : 0), x, w, y, workspace);
     auto it = g_instances.find(ikey);
     if (it == g_instances.end()) {
       if (g_instances.size() >= max_instances()) {

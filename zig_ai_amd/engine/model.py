@@ -13,6 +13,7 @@ from ..cache.manager import CacheManager, CacheView
 from ..config import load_config
 from ..config.spec import LayerCall, ModelSpec, PartSpec
 from ..kernels import build as kernel_build
+from ..kernels import ops
 from ..parts import base as parts
 from ..weights.loader import load_tensors
 from .batch import StepContext
@@ -206,6 +207,16 @@ class DecoderModel:
         entry's parts left under ``step.taps`` (the attention mixer: its queries, the
         keys and values it stored, its output); all copies that later kernels do not
         touch."""
+        # a model that keeps every sum in a fixed order also keeps the GEMM library's first
+        # answer for every shape: which of its candidates is fastest is decided by a clock
+        wanted, ops.library_tuning = ops.library_tuning, self.runtime.stream_additions
+        try:
+            return self._forward(step, views, taps)
+        finally:
+            ops.library_tuning = wanted
+
+    def _forward(self, step: StepContext, views: Sequence[CacheView],
+                 taps: Optional[List[Dict[str, torch.Tensor]]]) -> torch.Tensor:
         residual = self.embedding.forward(step.token_ids)
         pending = None
         if taps is not None:

@@ -10,6 +10,7 @@ operands other than the ones its indexing assumes.
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Optional, Tuple
 
 import torch
@@ -67,7 +68,7 @@ _SIGNATURES = {
     ("calibrate", "za_read_stream"): [c_void_p, c_size_t, c_int, c_void_p, c_void_p],
     ("calibrate", "za_mfma_loop"): [c_int, c_int, c_void_p, c_void_p],
     ("blaslt", "za_lt_matmul"): [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                                 c_void_p, c_size_t, c_void_p],
+                                 c_int, c_void_p, c_size_t, c_void_p],
 }
 _functions = {}
 
@@ -314,6 +315,11 @@ def _k_splits(M: int, N: int, K: int) -> int:
 
 LIBRARY_WORKSPACE_BYTES = 64 << 20
 _library_workspace = {}
+# Whether the GEMM library's candidates for a shape of many rows are timed at the shape's
+# first call (csrc/blaslt.hip).  Which candidate wins can differ from run to run; a model
+# that promises the same bits run after run switches this off around its steps, and
+# ZIG_AI_GEMM_TUNE=0 switches it off for a whole process.
+library_tuning = os.environ.get("ZIG_AI_GEMM_TUNE", "1") != "0"
 
 
 def _library_matmul(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype,
@@ -332,7 +338,8 @@ def _library_matmul(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtyp
     shape = (splits, M, N) if splits > 1 else (M, N)
     out = torch.empty(shape, dtype=torch.float32 if f32 else torch.bfloat16, device=x.device)
     rc = _fn("blaslt", "za_lt_matmul")(_ptr(x), _ptr(weight), _ptr(out), M, N, K, 1 if f32 else 0,
-                                       splits, _ptr(work), LIBRARY_WORKSPACE_BYTES, _stream())
+                                       splits, 1 if library_tuning else 0, _ptr(work),
+                                       LIBRARY_WORKSPACE_BYTES, _stream())
     if rc == -2:
         return None
     if rc != 0:
