@@ -89,10 +89,9 @@ def serve(cfg, name, n_requests, new_tokens, portion_graphs=False) -> int:
         # so that no library loads its kernels inside the timed run
         engine.generate([p[:64] for p in prompts[:20]], max_new_tokens=4, temperature=0.7, seed=3,
                         eos_token_id=-1)
-        # and the prompts themselves once, two tokens each: the GEMM library's candidates
-        # for steps of many rows are timed at a shape's first call (a server does that
-        # once in its life)
-        engine.generate(prompts, max_new_tokens=2, temperature=0.7, seed=3, eos_token_id=-1)
+        # and the run itself once: the GEMM library's candidates for a shape are timed at
+        # the shape's first call (some 10 ms each; a server does that once in its life)
+        engine.generate(prompts, max_new_tokens=new_tokens, temperature=0.7, seed=3, eos_token_id=-1)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         out = engine.generate(prompts, max_new_tokens=new_tokens, temperature=0.7, seed=3,

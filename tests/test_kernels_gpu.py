@@ -188,10 +188,11 @@ def test_gemm_bf16_library_keeps_32_bits(M, N, K):
     assert rel_err(low, x.double() @ w.double().T) < BF16_TOL
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 2048, 2048), (700, 1000, 4096), (512, 264, 1024)])
+@pytest.mark.parametrize("M,N,K", [(256, 2048, 2048), (700, 1000, 4096), (512, 264, 1024),
+                                   (64, 3072, 2048), (20, 1000, 4096)])
 def test_gemm_bf16_library_candidates_timed_at_first_use(M, N, K, monkeypatch):
-    """From 256 rows on the library's candidates for a shape are timed at its first call
-    and the fastest is kept: the result is a product like any other, a second call runs
+    """The library's candidates for a shape are timed at its first call (below 256 rows
+    with the weights out of the caches) and the fastest is kept: the result is a product like any other, a second call runs
     the same kernel (the same bits), a neighbouring row count takes the same choice, and
     with the timing switched off the first candidate gives the same product to rounding."""
     x, w = rand((M, K), torch.bfloat16, 140), rand((N, K), torch.bfloat16, 141)

@@ -14,19 +14,29 @@
 // operands seen before, one launch of a prepared instance (see InstanceKey).
 // The same shape therefore always runs the same kernel, recorded in a graph or not.
 //
-// Which algorithm: for products of many rows (TUNE_MIN_ROWS and more) the heuristic's first
-// answer is not always the fastest on this GPU (measured at 2,048 rows, bfloat16 out:
-// [2048, 8192] weights 88 us with the first answer, 76 with the eighteenth; [2048, 2048]
-// 29 against 25; at 512 rows [16384, 2048] 39 against 34), so with `tune` the first call
-// of a shape times the first TUNE_CANDIDATES answers on the call's own operands and keeps
-// the fastest.  Shapes whose row counts fall into the same block of TUNE_BUCKET rows share
-// the choice, so a server that sees every portion length times a few dozen shapes, not
-// thousands.  Which answer wins can differ from run to run when two are close: callers
-// that want the same bits run after run pass tune = 0 and get the first answer.
+// Which algorithm: the heuristic's first answer is not always the fastest on this GPU
+// (measured, bfloat16 out, weights from memory: 2,048 rows on [2048, 8192] weights 88 us with
+// the first answer, 76 with the eighteenth; on [2048, 2048] 29 against 25; 64 rows on
+// [3072, 2048] 15.4 against 9.0, on [6144, 2048] 13.5 against 11.0), so with `tune` the first
+// call of a shape times the first TUNE_CANDIDATES answers on the call's own operands and
+// keeps the fastest.  Products of fewer than TUNE_COLD_ROWS rows wait for their weights,
+// not for the matrix cores, and in a model every weight comes from memory: between their
+// timed runs TUNE_EVICT_BYTES of a buffer allocated for the occasion are cleared, so that
+// the weights do not lie in a cache (timed warm, the ranking is another one and a decode
+// step of 64 rows got slower).  Shapes whose row counts fall into the same block (of
+// TUNE_BUCKET rows from TUNE_COLD_ROWS on, between two powers of two below) share the
+// choice, so a server that sees every batch size and portion length times a few dozen
+// shapes, some 10 ms each, not thousands.  (Naming the winner to the library by its index
+// for a new row count of a block, instead of looking for it among the heuristic's answers
+// for that row count, cost 300 ms at its first use.)  Which answer wins can differ from run
+// to run when two are close: callers that want the same bits run after run pass tune = 0
+// and get the first answer.  ZIG_AI_GEMM_TUNE_LOG=1 prints a line for every shape timed.
 #include <hip/hip_runtime.h>
 #include <hipblaslt/hipblaslt-ext.hpp>
 #include <hipblaslt/hipblaslt.h>
 
+#include <chrono>
+#include <cstdio>
 #include <cstdlib>
 #include <map>
 #include <memory>
@@ -51,9 +61,26 @@ struct Plan {
   std::vector<hipblasLtMatmulHeuristicResult_t> candidates;
 };
 
-constexpr int TUNE_MIN_ROWS = 256;
+constexpr int TUNE_MIN_ROWS = 17;      // (up to 16 rows this package's own kernels run)
+constexpr int TUNE_COLD_ROWS = 256;
 constexpr int TUNE_BUCKET = 256;
 constexpr int TUNE_CANDIDATES = 24;
+constexpr size_t TUNE_EVICT_BYTES = (size_t)320 << 20;   // more than the caches hold
+
+bool tune_log() {
+  static const bool on = [] {
+    const char* v = std::getenv("ZIG_AI_GEMM_TUNE_LOG");
+    return v && v[0] == '1';
+  }();
+  return on;
+}
+
+int tune_block(int M) {
+  if (M >= TUNE_COLD_ROWS) return 16 + (M + TUNE_BUCKET - 1) / TUNE_BUCKET;
+  int block = 0;
+  while ((1 << block) < M) ++block;
+  return block;
+}
 
 using Key = std::tuple<int, int, int, int, int, int, int>;   // device, M, N, K, output type, P, tune
 // device, block of rows, N, K, output type, P -> the library's index of the algorithm that won
@@ -159,12 +186,23 @@ bool make_plan(hipblasLtHandle_t handle, int M, int N, int K, int out_f32, int P
 
 // Times the plan's candidates on the call's operands (y is overwritten by every one of
 // them, and by the product proper afterwards) and returns the fastest: one run to warm
-// up, then TUNE_RUNS timed together.  The stream is waited for; this happens once per
-// block of row counts.  A candidate that fails, or takes three times the best so far in
-// its first run, is out.
+// up, then TUNE_RUNS timed together, or with `cold` each alone behind a pass over a
+// buffer larger than the caches.  The stream is waited for; this happens once per block
+// of row counts.  A candidate that fails, or takes three times the best so far in its
+// first run, is out.
 constexpr int TUNE_RUNS = 3;
 int fastest_candidate(hipblasLtHandle_t handle, const Plan& plan, const void* x, const void* w,
-                      void* y, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+                      void* y, void* workspace, size_t workspace_bytes, bool cold,
+                      hipStream_t stream) {
+  void* evict = nullptr;
+  if (cold && hipMalloc(&evict, TUNE_EVICT_BYTES) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;                     // no room to time it properly: the first answer
+  }
+  struct Release {
+    void* p;
+    ~Release() { if (p) (void)hipFree(p); }
+  } release{evict};
   hipEvent_t t0 = nullptr, t1 = nullptr;
   if (hipEventCreate(&t0) != hipSuccess || hipEventCreate(&t1) != hipSuccess) {
     if (t0) (void)hipEventDestroy(t0);
@@ -187,20 +225,39 @@ int fastest_candidate(hipblasLtHandle_t handle, const Plan& plan, const void* x,
                              plan.c, &algo, workspace, workspace_bytes, stream) == HIPBLAS_STATUS_SUCCESS;
     };
     float ms = 0.f;
-    if (hipEventRecord(t0, stream) != hipSuccess || !run() || hipEventRecord(t1, stream) != hipSuccess ||
-        hipEventSynchronize(t1) != hipSuccess || hipEventElapsedTime(&ms, t0, t1) != hipSuccess) {
-      (void)hipGetLastError();
-      continue;
+    if (cold) {
+      // one run to load the kernel, then every timed run alone, its weights out of the caches
+      float total = 0.f;
+      bool fine = run();
+      for (int r = 0; r < TUNE_RUNS && fine; ++r) {
+        fine = hipMemsetAsync(evict, 0, TUNE_EVICT_BYTES, stream) == hipSuccess &&
+               hipEventRecord(t0, stream) == hipSuccess && run() &&
+               hipEventRecord(t1, stream) == hipSuccess && hipEventSynchronize(t1) == hipSuccess &&
+               hipEventElapsedTime(&ms, t0, t1) == hipSuccess;
+        total += ms;
+        if (fine && r == 0 && best_ms > 0.f && ms > 3.f * best_ms) fine = false;
+      }
+      if (!fine) {
+        (void)hipGetLastError();
+        continue;
+      }
+      ms = total / TUNE_RUNS;
+    } else {
+      if (hipEventRecord(t0, stream) != hipSuccess || !run() || hipEventRecord(t1, stream) != hipSuccess ||
+          hipEventSynchronize(t1) != hipSuccess || hipEventElapsedTime(&ms, t0, t1) != hipSuccess) {
+        (void)hipGetLastError();
+        continue;
+      }
+      if (best_ms > 0.f && ms > 3.f * best_ms) continue;
+      bool fine = hipEventRecord(t0, stream) == hipSuccess;
+      for (int r = 0; r < TUNE_RUNS && fine; ++r) fine = run();
+      if (!fine || hipEventRecord(t1, stream) != hipSuccess || hipEventSynchronize(t1) != hipSuccess ||
+          hipEventElapsedTime(&ms, t0, t1) != hipSuccess) {
+        (void)hipGetLastError();
+        continue;
+      }
+      ms /= TUNE_RUNS;
     }
-    if (best_ms > 0.f && ms > 3.f * best_ms) continue;
-    bool fine = hipEventRecord(t0, stream) == hipSuccess;
-    for (int r = 0; r < TUNE_RUNS && fine; ++r) fine = run();
-    if (!fine || hipEventRecord(t1, stream) != hipSuccess || hipEventSynchronize(t1) != hipSuccess ||
-        hipEventElapsedTime(&ms, t0, t1) != hipSuccess) {
-      (void)hipGetLastError();
-      continue;
-    }
-    ms /= TUNE_RUNS;
     if (best_ms < 0.f || ms < best_ms) {
       best_ms = ms;
       best = (int)i;
@@ -249,7 +306,7 @@ ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int
     }
     Plan& kept = it->second;
     if (kept.usable && !kept.settled) {
-      const TunedKey block(device, (M + TUNE_BUCKET - 1) / TUNE_BUCKET, N, K, out_f32, P);
+      const TunedKey block(device, tune_block(M), N, K, out_f32, P);
       auto choose = [&](size_t i) {
         kept.algo = kept.candidates[i].algo;
         kept.workspace = kept.candidates[i].workspaceSize;
@@ -267,8 +324,14 @@ ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int
             break;
           }
       } else if (!recording) {
-        const int best = fastest_candidate(handle, kept, x, w, y, workspace, workspace_bytes, stream);
+        const auto began = std::chrono::steady_clock::now();
+        const int best = fastest_candidate(handle, kept, x, w, y, workspace, workspace_bytes,
+                                           M < TUNE_COLD_ROWS, stream);
         choose((size_t)best);
+        if (tune_log())
+          fprintf(stderr, "[zig_ai_amd] timed %zu candidates for M=%d N=%d K=%d P=%d %s: answer %d in %.1f ms\n",
+                  kept.candidates.size(), M, N, K, P, out_f32 ? "f32" : "bf16", best,
+                  std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - began).count());
         g_tuned.emplace(block, hipblaslt_ext::getIndexFromAlgo(kept.algo));
       }
       // (a shape first met while a stream is recorded keeps the first answer for good:

@@ -209,7 +209,8 @@ class DecoderModel:
         touch."""
         # a model that keeps every sum in a fixed order also keeps the GEMM library's first
         # answer for every shape: which of its candidates is fastest is decided by a clock
-        wanted, ops.library_tuning = ops.library_tuning, self.runtime.stream_additions
+        wanted = ops.library_tuning
+        ops.library_tuning = wanted and self.runtime.stream_additions
         try:
             return self._forward(step, views, taps)
         finally:
