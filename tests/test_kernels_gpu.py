@@ -188,7 +188,7 @@ def test_gemm_bf16_library_keeps_32_bits(M, N, K):
     assert rel_err(low, x.double() @ w.double().T) < BF16_TOL
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 2048, 2048), (700, 1000, 4096), (512, 264, 1024),
+@pytest.mark.parametrize("M,N,K", [(256, 2048, 2048), (700, 1000, 4096), (512, 520, 1024),
                                    (64, 3072, 2048), (20, 1000, 4096)])
 def test_gemm_bf16_library_candidates_timed_at_first_use(M, N, K, monkeypatch):
     """The library's candidates for a shape are timed at its first call (below 256 rows
@@ -965,6 +965,77 @@ def test_short_conv_whole_and_in_portions(dtype, H, L, bias):
             row += p.shape[0]
     for i in range(3):
         assert rel_err(torch.cat(got[i]), expect[i]) < tol_of(dtype)
+
+
+@pytest.mark.parametrize("M,H,L,bias", [(1, 512, 3, False), (8, 2048, 3, False), (5, 1024, 4, True),
+                                        (8, 2560, 3, True), (3, 1536, 1, False), (7, 4096, 8, True),
+                                        (2, 3584, 2, False)])
+def test_in_proj_gated_conv_is_the_three_kernels_in_one(M, H, L, bias):
+    """A decode batch of the ShortConv mixer, one token a request: norm + in_proj +
+    convolution in one kernel give the bits (outputs AND new state) that the norm inside
+    in_proj followed by the convolution's own kernel give, over three steps of the same
+    requests (so the carried state matters), at widths other than the engine's, with
+    slots out of order in a wider row; and both agree with the plain formulas."""
+    K = H
+    w_in = rand((3 * H, K), torch.bfloat16, 300, 0.03).to(dev())
+    taps = rand((H, L), torch.float32, 301)
+    b = rand((H,), torch.float32, 302) if bias else None
+    norm_w = (1.0 + 0.3 * rand((K,), torch.float32, 303)).to(dev())
+    slots = [5, 0, 7, 2, 6, 1, 3, 4][:M]
+    slot_id = torch.tensor(slots, dtype=torch.int32, device=dev())
+    token_seq = torch.arange(M, dtype=torch.int32, device=dev())
+    seq_start = torch.arange(M + 1, dtype=torch.int32, device=dev())
+    taps_t, bd = taps.t().contiguous().to(dev()), b.to(dev()) if bias else None
+
+    def memory():
+        mem = torch.zeros((8, H * L + 5), dtype=torch.float32, device=dev())
+        return mem, mem[:, 2:2 + H * L].unflatten(1, (H, L))
+
+    (mem_a, state_a), (mem_b, state_b) = memory(), memory()
+    hist = torch.zeros((M, L, H), dtype=torch.float64)
+    for step in range(3):
+        stream = rand((M, K), torch.float32, 310 + step, 2.0).to(dev())
+        x = ops().NormedRows(stream, norm_w, 1e-5, torch.bfloat16)
+        assert ops().gated_conv_fusable(x, w_in, taps_t)
+        mem_before = mem_a.clone()
+        fused = ops().in_proj_gated_conv(x, w_in, taps_t, bd, state_a, slot_id)
+        z = ops().linear(x, w_in)
+        apart = ops().short_conv(z, taps_t, bd, state_b, token_seq, seq_start, slot_id)
+        assert torch.equal(fused, apart), (step, rel_err(fused, apart))
+        assert torch.equal(mem_a, mem_b)
+        for channels in (4, 8, 16):             # however many channels a workgroup takes
+            mem_c = mem_before.clone()
+            state_c = mem_c[:, 2:2 + H * L].unflatten(1, (H, L))
+            again = ops().in_proj_gated_conv(x, w_in, taps_t, bd, state_c, slot_id, channels=channels)
+            assert torch.equal(again, apart) and torch.equal(mem_c, mem_b), channels
+        # the plain formulas, on the projection's own (rounded) output
+        zd = z.double().cpu()
+        u = zd[:, :H] * zd[:, 2 * H:]
+        hist = torch.cat([hist[:, 1:], u[:, None, :]], dim=1)
+        c = (hist * taps.double().T[None]).sum(dim=1) + (b.double() if bias else 0.0)
+        assert rel_err(fused, zd[:, H:2 * H] * c) < BF16_TOL
+    for m, slot in enumerate(slots):
+        assert rel_err(state_a[slot].cpu().T, hist[m]) < F32_TOL
+    untouched = [s for s in range(8) if s not in slots]
+    assert (mem_a[untouched] == 0).all() and (mem_a[:, :2] == 0).all() and (mem_a[:, 2 + H * L:] == 0).all()
+
+
+def test_in_proj_gated_conv_refuses_what_it_cannot_take():
+    w = rand((3 * 96, 512), torch.bfloat16, 320).to(dev())          # width 96: fine; K 512
+    taps = rand((3, 96), torch.float32, 321).to(dev())
+    nw = torch.ones(512, device=dev())
+    many = ops().NormedRows(torch.zeros((9, 512), device=dev()), nw, 1e-5, torch.bfloat16)
+    assert not ops().gated_conv_fusable(many, w, taps)                 # nine rows
+    odd = ops().NormedRows(torch.zeros((2, 520), device=dev()), torch.ones(520, device=dev()), 1e-5,
+                           torch.bfloat16)
+    assert not ops().gated_conv_fusable(odd, rand((3 * 96, 520), torch.bfloat16, 322).to(dev()), taps)
+    assert not ops().gated_conv_fusable(torch.zeros((2, 512), dtype=torch.bfloat16, device=dev()), w, taps)
+    narrow = rand((3, 104), torch.float32, 323).to(dev())             # width no multiple of 16
+    few = ops().NormedRows(torch.zeros((2, 512), device=dev()), nw, 1e-5, torch.bfloat16)
+    assert not ops().gated_conv_fusable(few, rand((312, 512), torch.bfloat16, 324).to(dev()), narrow)
+    with pytest.raises(ops().KernelError):
+        ops().in_proj_gated_conv(many, w, taps, None, torch.zeros((1, 96, 3), device=dev()),
+                                 torch.zeros(9, dtype=torch.int32, device=dev()))
 
 
 def test_short_conv_identity_filter():

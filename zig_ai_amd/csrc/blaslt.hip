@@ -62,6 +62,7 @@ struct Plan {
 };
 
 constexpr int TUNE_MIN_ROWS = 17;      // (up to 16 rows this package's own kernels run)
+constexpr size_t TUNE_MIN_WEIGHT = (size_t)1 << 19;   // elements: a megabyte of bfloat16; below, nothing to gain
 constexpr int TUNE_COLD_ROWS = 256;
 constexpr int TUNE_BUCKET = 256;
 constexpr int TUNE_CANDIDATES = 24;
@@ -294,7 +295,7 @@ ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int
       h = g_handles.emplace(device, made).first;
     }
     handle = h->second;
-    const bool tuning = tune && M >= TUNE_MIN_ROWS;
+    const bool tuning = tune && M >= TUNE_MIN_ROWS && (size_t)N * K >= TUNE_MIN_WEIGHT;
     const Key key(device, M, N, K, out_f32, P, tuning ? 1 : 0);
     auto it = g_plans.find(key);
     if (it == g_plans.end()) {
@@ -347,7 +348,9 @@ ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int
   hipblaslt_ext::Gemm* instance = nullptr;
   {
     std::lock_guard<std::mutex> guard(g_lock);
-    const InstanceKey ikey(Key(device, M, N, K, out_f32, P, tune && M >= TUNE_MIN_ROWS ? 1 : 0), x, w, y, workspace);
+    const InstanceKey ikey(Key(device, M, N, K, out_f32, P,
+                               tune && M >= TUNE_MIN_ROWS && (size_t)N * K >= TUNE_MIN_WEIGHT ? 1 : 0),
+                           x, w, y, workspace);
     auto it = g_instances.find(ikey);
     if (it == g_instances.end()) {
       if (g_instances.size() >= max_instances()) {

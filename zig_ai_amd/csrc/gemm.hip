@@ -672,6 +672,142 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
   }
 }
 
+// The ShortConv mixer's in_proj for a decode batch in which every request brings one
+// token, with the mixer's gated convolution in the epilogue
+// (/root/reference/src/cuda/layer_kernels.cu:192-222 folds convolution, activation and
+// state into one kernel too).  W = [B rows (H); C rows (H); x rows (H)], rows of K.  A
+// workgroup takes CH channels (4, 8 or 16: the launcher chooses so that about 256
+// workgroups run) and with them 3 * CH weight rows, B then C then x of its channels, in
+// TILES = ceil(3 * CH / 16) tiles of 16 (a lane reads whatever row its fragment names,
+// so nothing is laid out anew; rows beyond 3 * CH repeat addresses that other lanes ask
+// for).  The tiles' sums, scaled and rounded as the projection would store them, meet in
+// LDS, and wave 0 does what short_conv_kernel's head threads do, with the same operations
+// in the same order, lane (m, q) for token m and the channels q * CH / 4 ... of the CH:
+//   u = B * x;  the state's L values move up by one and take u;  c = bias + sum_j w[j] * state[j];
+//   y = C * c
+// Slot, state and filter are requested at the kernel's start, so they have arrived when
+// the products are done.  Rows come as NormedRows, staged through LDS: M <= 8.
+template <int NW, int TILES>
+__global__ void __launch_bounds__(NW * 64, 2)
+gemm_bf16_rows16_gated_conv_kernel(NormedRowsArg normed, const bf16_t* __restrict__ W,
+                                   const float* __restrict__ taps,
+                                   const float* __restrict__ conv_bias, float* __restrict__ state,
+                                   long long slot_stride, const int* __restrict__ slot_id,
+                                   bf16_t* __restrict__ y, int M, int H, int K, int L) {
+  constexpr int KSTEPS = 16, MAXL = 8;
+  constexpr int CH = TILES == 1 ? 4 : (TILES == 2 ? 8 : 16);
+  constexpr int PER = CH / 4;                       // channels of a lane in the epilogue
+  __shared__ float red[2][NW][64][4];
+  __shared__ float ssw[NW][16];
+  __shared__ float zs[TILES * 16][ROWS16_STAGE_ROWS + 1];   // [weight row of the workgroup][token]
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int frag_row = lane & 15, frag_k = (lane >> 4) * 8;
+  const int kbase = wave * KSTEPS * 32 + frag_k;
+  const bool inside = (wave + 1) * (KSTEPS * 32) <= K;
+  const int c0 = blockIdx.x * CH;
+  // the weight row of this lane's fragment in tile t: row v = t * 16 + frag_row of the
+  // workgroup's 3 * CH (a row beyond them takes the place of one CH earlier)
+  auto weight_row = [&](int t) {
+    int v = t * 16 + frag_row;
+    if (v >= 3 * CH) v -= CH;
+    return W + (size_t)((v / CH) * H + c0 + v % CH) * K + kbase;
+  };
+
+  // wave 0: token m, channels ch .. ch + PER - 1
+  const int m = lane & 15, ch = c0 + (lane >> 4) * PER;
+  const bool mine = wave == 0 && m < M;
+  float hist[MAXL][PER], wt[MAXL][PER], cb[PER];
+  float* st = nullptr;
+  if (mine) {
+    st = state + (size_t)slot_id[m] * (size_t)slot_stride + (size_t)ch * L;
+#pragma unroll
+    for (int j = 0; j < MAXL; ++j)
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        hist[j][i] = j < L ? st[i * L + j] : 0.f;
+        wt[j][i] = j < L ? taps[(size_t)j * H + ch + i] : 0.f;
+      }
+#pragma unroll
+    for (int i = 0; i < PER; ++i) cb[i] = conv_bias ? conv_bias[ch + i] : 0.f;
+  }
+
+  bf16x8_t xa[KSTEPS], fn[KSTEPS];
+  stage_normed_rows<NW, KSTEPS>(xa, normed.x, normed.rows, normed.weight, M, K, tid, ssw,
+                                reinterpret_cast<bf16_t*>(rows16_staged), [&]() {
+                                  const bf16_t* wp = weight_row(0);
+#pragma unroll
+                                  for (int s = 0; s < KSTEPS; ++s)
+                                    fn[s] = *reinterpret_cast<const bf16x8_t*>(wp + s * 32);
+                                });
+  // One tile; `more` (a compile-time flag): the next tile's fragments are requested into
+  // the registers that the products free.
+  auto tile = [&](int t, auto more) {
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    if (inside) {
+      if constexpr (decltype(more)::value) {
+        const bf16_t* nxt = weight_row(t + 1);
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fn[s], xa[s], acc, 0, 0, 0);
+          fn[s] = *reinterpret_cast<const bf16x8_t*>(nxt + s * 32);
+          __builtin_amdgcn_sched_barrier(0);   // in this order: the compiler would bunch the loads
+        }
+      } else {
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fn[s], xa[s], acc, 0, 0, 0);
+      }
+    }
+    if (NW > 1) {
+      float* mine_red = red[t & 1][wave][lane];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mine_red[r] = acc[r];
+      __syncthreads();
+    }
+    if (wave == 0 && m < M) {
+      const float scale = normed_row_scale<NW>(ssw, m, K, normed.eps);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float v = acc[r];
+        if (NW > 1) {
+          v = red[t & 1][0][lane][r];
+#pragma unroll
+          for (int w = 1; w < NW; ++w) v += red[t & 1][w][lane][r];
+        }
+        zs[t * 16 + (lane >> 4) * 4 + r][m] = (float)(bf16_t)(v * scale);
+      }
+    }
+  };
+  if constexpr (TILES >= 2) tile(0, std::true_type{});
+  if constexpr (TILES >= 3) tile(1, std::true_type{});
+  tile(TILES - 1, std::false_type{});
+  if (!mine) return;
+  // (wave 0 reads what its own lanes wrote: LDS operations of one wave run in order)
+  bf16_t out[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int c = (lane >> 4) * PER + i;
+    const float u = zs[c][m] * zs[2 * CH + c][m];
+#pragma unroll
+    for (int j = 0; j < MAXL - 1; ++j)
+      if (j < L - 1) hist[j][i] = hist[j + 1][i];
+#pragma unroll
+    for (int j = 0; j < MAXL; ++j)
+      if (j == L - 1) hist[j][i] = u;
+    float acc = cb[i];
+#pragma unroll
+    for (int j = 0; j < MAXL; ++j)
+      if (j < L) acc = fmaf(wt[j][i], hist[j][i], acc);
+    out[i] = (bf16_t)(zs[CH + c][m] * acc);
+#pragma unroll
+    for (int j = 0; j < MAXL; ++j)
+      if (j < L) st[i * L + j] = hist[j][i];
+  }
+#pragma unroll
+  for (int i = 0; i < PER; ++i) y[(size_t)m * H + ch + i] = out[i];
+}
+
 // The same kernel for the fused gate|up projection of a SwiGLU feed-forward,
 // W = [gate rows (I); up rows (I)]: a workgroup computes a row group of the gate
 // and the matching row group of the up projection and writes
@@ -1081,4 +1217,54 @@ extern "C" int za_gemm_bf16_rows16_swiglu(const void* A, const float* x, const i
   ZA_SG_CASE(8, 32)
 #undef ZA_SG_CASE
 #undef ZA_SG_LAUNCH
+}
+
+// The ShortConv mixer from the 32-bit stream to the convolution's output in one kernel
+// (gemm_bf16_rows16_gated_conv_kernel), for a decode batch of M <= 8 requests with one
+// token each: row m of the product is token m and belongs to the request whose state
+// slot is slot_id[m].  W [3H, K] bfloat16 (B, C, x rows), taps [L, H] and conv_bias [H]
+// (or null) 32-bit, state as za_short_conv takes it, y [M, H] bfloat16.  K a multiple of
+// 512 up to 4096, H a multiple of 16, L <= 8.  `channels` (0: the launcher chooses) is
+// the number of channels a workgroup takes: 4, 8 or 16.
+extern "C" int za_gemm_bf16_rows16_gated_conv(const float* x, const int* rows,
+                                              const float* norm_weight, float eps, const void* W,
+                                              const float* taps, const float* conv_bias,
+                                              float* state, long long slot_stride,
+                                              const int* slot_id, void* y, int M, int H, int K,
+                                              int L, int channels, hipStream_t stream) {
+  if (M == 0 || H == 0) return 0;
+  if (M < 0 || H < 0 || K <= 0 || L <= 0 || !x || !norm_weight || !W || !taps || !state || !slot_id ||
+      !y || slot_stride < (long long)H * L)
+    return ZA_ERR_ARG;
+  if (M > ROWS16_STAGE_ROWS || H % 16 != 0 || L > 8 || !rows16_takes_norm(K, 1))
+    return ZA_ERR_UNSUPPORTED;
+  if (channels != 0 && channels != 4 && channels != 8 && channels != 16) return ZA_ERR_ARG;
+  // measured at 8 rows and at 1 (us; widths 1024, 1536, 2048, 2560, 4096):
+  //   4 channels   5.1 / 4.4    7.8 / 6.7    9.8 / 8.1   17.5 / 14.8   34.8 / 26.2
+  //   8            6.5 / 5.8    8.0 / 7.3    9.5 / 9.0   18.2 / 16.2   28.5 / 24.6
+  //   16           7.7 / 6.9    9.6 / 8.8   11.0 / 10.9  14.5 / 13.4   22.7 / 20.7
+  if (channels == 0) channels = H <= 1536 ? 4 : (H <= 2048 ? (M <= 2 ? 4 : 8) : 16);
+  const NormedRowsArg normed = {x, rows, norm_weight, eps};
+  dim3 grid(H / channels);
+#define ZA_GC_LAUNCH(NW, TILES)                                                               \
+  {                                                                                           \
+    const size_t lds = rows16_stage_bytes(NW, M);                                             \
+    auto kernel = gemm_bf16_rows16_gated_conv_kernel<NW, TILES>;                              \
+    if (const int rc = rows16_allow_lds((const void*)kernel, lds)) return rc;                 \
+    hipLaunchKernelGGL(kernel, grid, dim3(NW * 64), lds, stream, normed, (const bf16_t*)W,    \
+                       taps, conv_bias, state, slot_stride, slot_id, (bf16_t*)y, M, H, K, L); \
+    return za_launch_status();                                                                \
+  }
+#define ZA_GC_CASE(NW)                                                                        \
+  {                                                                                           \
+    if (channels == 4) ZA_GC_LAUNCH(NW, 1)                                                    \
+    if (channels == 8) ZA_GC_LAUNCH(NW, 2)                                                    \
+    ZA_GC_LAUNCH(NW, 3)                                                                       \
+  }
+  if (K <= 512) ZA_GC_CASE(1)
+  if (K <= 1024) ZA_GC_CASE(2)
+  if (K <= 2048) ZA_GC_CASE(4)
+  ZA_GC_CASE(8)
+#undef ZA_GC_CASE
+#undef ZA_GC_LAUNCH
 }

@@ -61,6 +61,10 @@ _SIGNATURES = {
                                              c_int, c_int, c_int, c_void_p],
     ("gemm", "za_gemm_bf16_rows16_swiglu"): [c_void_p, c_void_p, c_void_p, c_void_p, c_float,
                                              c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    ("gemm", "za_gemm_bf16_rows16_gated_conv"): [c_void_p, c_void_p, c_void_p, c_float, c_void_p,
+                                                 c_void_p, c_void_p, c_void_p, c_longlong,
+                                                 c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                                 c_int, c_void_p],
     ("sampling", "za_sample"): [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                 c_void_p, c_int, c_void_p],
     ("sampling", "za_repetition_penalty"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
@@ -765,6 +769,58 @@ def paged_attention_decode_mfma(q: torch.Tensor, kv_cache: torch.Tensor,
 
 
 # ---------------------------------------------------------------- short conv
+GATED_CONV_MAX_ROWS = 8
+
+
+def gated_conv_fusable(x, w_in: torch.Tensor, taps: torch.Tensor) -> bool:
+    """Whether ``in_proj_gated_conv`` takes these operands: rows that still await their
+    norm, at most eight of them, bfloat16 weights whose K the fused norm covers, and a
+    width that is a multiple of 16."""
+    if not isinstance(x, NormedRows) or x.dtype != torch.bfloat16 or w_in.dtype != torch.bfloat16:
+        return False
+    M, K = x.shape
+    L, width = taps.shape
+    return (0 < M <= GATED_CONV_MAX_ROWS and normed_rows_fusable(M, K) and width % 16 == 0
+            and L <= 8 and tuple(w_in.shape) == (3 * width, K))
+
+
+def in_proj_gated_conv(x: "NormedRows", w_in: torch.Tensor, taps: torch.Tensor,
+                       bias: Optional[torch.Tensor], state: torch.Tensor,
+                       slot_id: torch.Tensor, channels: int = 0) -> torch.Tensor:
+    """The ShortConv mixer from the residual stream to the convolution's output for a
+    decode batch in which every request brings ONE token (row m belongs to the request
+    with state slot ``slot_id[m]``): the norm, ``in_proj`` (no bias) and ``short_conv``
+    in one kernel, with the bits that the three kernels give one after the other.
+    Operands as ``linear`` and ``short_conv`` take them; see ``gated_conv_fusable``.
+    ``channels`` (4, 8 or 16; 0 leaves it to the launcher): channels per workgroup."""
+    if not gated_conv_fusable(x, w_in, taps):
+        raise KernelError("in_proj_gated_conv: operands outside what the fused kernel takes")
+    M, K = x.shape
+    L, width = taps.shape
+    _need(w_in, "w_in", torch.bfloat16, (3 * width, K))
+    _need(taps, "taps", torch.float32)
+    if bias is not None:
+        _need(bias, "bias", torch.float32, (width,))
+    if not (isinstance(state, torch.Tensor) and state.is_cuda and state.dtype == torch.float32):
+        raise KernelError("state must be a float32 tensor on the GPU")
+    if state.dim() != 3 or tuple(state.shape[1:]) != (width, L):
+        raise KernelError(f"state has shape {tuple(state.shape)}, expected [slots, {width}, {L}]")
+    if state.stride(2) != 1 or state.stride(1) != L or state.stride(0) < width * L:
+        raise KernelError(f"state has strides {state.stride()}; a slot must be laid out "
+                          f"[{width}, {L}] contiguously")
+    _need(slot_id, "slot_id", torch.int32)
+    if slot_id.numel() < M:
+        raise KernelError(f"{M} rows but {slot_id.numel()} state slots")
+    y = torch.empty((M, width), dtype=torch.bfloat16, device=w_in.device)
+    rc = _fn("gemm", "za_gemm_bf16_rows16_gated_conv")(
+        _ptr(x.residual), _ptr(x.rows), _ptr(x.weight), x.eps, _ptr(w_in), _ptr(taps), _ptr(bias),
+        _ptr(state), state.stride(0), _ptr(slot_id), _ptr(y), M, width, K, L, channels, _stream())
+    _check(rc, "gemm_bf16_rows16_gated_conv", f"M={M} width={width} K={K} L={L}")
+    _note("linear", M=M, N=3 * width, K=K, norm_in_product=True, added_to_stream=False,
+          partial_sums=1, out=torch.bfloat16)
+    return y
+
+
 def short_conv(z: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tensor],
                state: torch.Tensor, token_seq: torch.Tensor, seq_start: torch.Tensor,
                slot_id: torch.Tensor) -> torch.Tensor:

@@ -62,9 +62,15 @@ class ShortConv(Mixer):
         ops.check_projection_weight(self.w_out, "short_conv w_out")
 
     def forward(self, x, step, cache, stream: Optional[torch.Tensor] = None):
-        z = ops.linear(x, self.w_in, self.b_in)
-        y = ops.short_conv(z, self.w_conv, self.b_conv, cache.state, step.token_seq,
-                           step.seq_start, step.slot_id)
+        if step.n_tokens == step.n_seqs and self.b_in is None \
+                and ops.gated_conv_fusable(x, self.w_in, self.w_conv):
+            # a decode batch, one token a request: norm, in_proj and convolution in one kernel
+            y = ops.in_proj_gated_conv(x, self.w_in, self.w_conv, self.b_conv, cache.state,
+                                       step.slot_id)
+        else:
+            z = ops.linear(x, self.w_in, self.b_in)
+            y = ops.short_conv(z, self.w_conv, self.b_conv, cache.state, step.token_seq,
+                               step.seq_start, step.slot_id)
         return ops.linear(y, self.w_out, self.b_out, partial_ok=True, accumulate=stream)
 
 
