@@ -19,12 +19,11 @@
 // the first answer, 76 with the eighteenth; on [2048, 2048] 29 against 25; 64 rows on
 // [3072, 2048] 15.4 against 9.0, on [6144, 2048] 13.5 against 11.0), so with `tune` the first
 // call of a shape times the first TUNE_CANDIDATES answers on the call's own operands and
-// keeps the fastest.  Products of fewer than TUNE_COLD_ROWS rows wait for their weights,
-// not for the matrix cores, and in a model every weight comes from memory: between their
-// timed runs TUNE_EVICT_BYTES of a buffer allocated for the occasion are cleared, so that
-// the weights do not lie in a cache (timed warm, the ranking is another one and a decode
-// step of 64 rows got slower).  Shapes whose row counts fall into the same block (of
-// TUNE_BUCKET rows from TUNE_COLD_ROWS on, between two powers of two below) share the
+// keeps the fastest.  In a model every weight comes from memory: between the timed runs
+// TUNE_EVICT_BYTES of a buffer allocated for the occasion are cleared, so that the weights
+// do not lie in a cache (timed warm, the ranking is another one: a decode step of 64 rows
+// got slower).  Shapes whose row counts fall into the same block (of
+// TUNE_BUCKET rows from TUNE_BUCKET rows on, between two powers of two below) share the
 // choice, so a server that sees every batch size and portion length times a few dozen
 // shapes, some 10 ms each, not thousands.  (Naming the winner to the library by its index
 // for a new row count of a block, instead of looking for it among the heuristic's answers
@@ -63,7 +62,6 @@ struct Plan {
 
 constexpr int TUNE_MIN_ROWS = 17;      // (up to 16 rows this package's own kernels run)
 constexpr size_t TUNE_MIN_WEIGHT = (size_t)1 << 19;   // elements: a megabyte of bfloat16; below, nothing to gain
-constexpr int TUNE_COLD_ROWS = 256;
 constexpr int TUNE_BUCKET = 256;
 constexpr int TUNE_CANDIDATES = 24;
 constexpr size_t TUNE_EVICT_BYTES = (size_t)320 << 20;   // more than the caches hold
@@ -77,7 +75,7 @@ bool tune_log() {
 }
 
 int tune_block(int M) {
-  if (M >= TUNE_COLD_ROWS) return 16 + (M + TUNE_BUCKET - 1) / TUNE_BUCKET;
+  if (M >= TUNE_BUCKET) return 16 + (M + TUNE_BUCKET - 1) / TUNE_BUCKET;
   int block = 0;
   while ((1 << block) < M) ++block;
   return block;
@@ -186,17 +184,16 @@ bool make_plan(hipblasLtHandle_t handle, int M, int N, int K, int out_f32, int P
 }
 
 // Times the plan's candidates on the call's operands (y is overwritten by every one of
-// them, and by the product proper afterwards) and returns the fastest: one run to warm
-// up, then TUNE_RUNS timed together, or with `cold` each alone behind a pass over a
-// buffer larger than the caches.  The stream is waited for; this happens once per block
-// of row counts.  A candidate that fails, or takes three times the best so far in its
-// first run, is out.
+// them, and by the product proper afterwards) and returns the fastest: one run to load
+// the kernel, then TUNE_RUNS timed ones, each alone behind a pass over a buffer larger
+// than the caches.  The stream is waited for; this happens once per block of row counts.
+// A candidate that fails, or takes three times the best so far in its first timed run,
+// is out.
 constexpr int TUNE_RUNS = 3;
 int fastest_candidate(hipblasLtHandle_t handle, const Plan& plan, const void* x, const void* w,
-                      void* y, void* workspace, size_t workspace_bytes, bool cold,
-                      hipStream_t stream) {
+                      void* y, void* workspace, size_t workspace_bytes, hipStream_t stream) {
   void* evict = nullptr;
-  if (cold && hipMalloc(&evict, TUNE_EVICT_BYTES) != hipSuccess) {
+  if (hipMalloc(&evict, TUNE_EVICT_BYTES) != hipSuccess) {
     (void)hipGetLastError();
     return 0;                     // no room to time it properly: the first answer
   }
@@ -225,40 +222,22 @@ int fastest_candidate(hipblasLtHandle_t handle, const Plan& plan, const void* x,
       return hipblasLtMatmul(handle, plan.op, &kOne, w, plan.a, x, plan.b, &kZero, y, plan.c, y,
                              plan.c, &algo, workspace, workspace_bytes, stream) == HIPBLAS_STATUS_SUCCESS;
     };
-    float ms = 0.f;
-    if (cold) {
-      // one run to load the kernel, then every timed run alone, its weights out of the caches
-      float total = 0.f;
-      bool fine = run();
-      for (int r = 0; r < TUNE_RUNS && fine; ++r) {
-        fine = hipMemsetAsync(evict, 0, TUNE_EVICT_BYTES, stream) == hipSuccess &&
-               hipEventRecord(t0, stream) == hipSuccess && run() &&
-               hipEventRecord(t1, stream) == hipSuccess && hipEventSynchronize(t1) == hipSuccess &&
-               hipEventElapsedTime(&ms, t0, t1) == hipSuccess;
-        total += ms;
-        if (fine && r == 0 && best_ms > 0.f && ms > 3.f * best_ms) fine = false;
-      }
-      if (!fine) {
-        (void)hipGetLastError();
-        continue;
-      }
-      ms = total / TUNE_RUNS;
-    } else {
-      if (hipEventRecord(t0, stream) != hipSuccess || !run() || hipEventRecord(t1, stream) != hipSuccess ||
-          hipEventSynchronize(t1) != hipSuccess || hipEventElapsedTime(&ms, t0, t1) != hipSuccess) {
-        (void)hipGetLastError();
-        continue;
-      }
-      if (best_ms > 0.f && ms > 3.f * best_ms) continue;
-      bool fine = hipEventRecord(t0, stream) == hipSuccess;
-      for (int r = 0; r < TUNE_RUNS && fine; ++r) fine = run();
-      if (!fine || hipEventRecord(t1, stream) != hipSuccess || hipEventSynchronize(t1) != hipSuccess ||
-          hipEventElapsedTime(&ms, t0, t1) != hipSuccess) {
-        (void)hipGetLastError();
-        continue;
-      }
-      ms /= TUNE_RUNS;
+    // one run to load the kernel, then every timed run alone, its weights out of the caches
+    float ms = 0.f, total = 0.f;
+    bool fine = run();
+    for (int r = 0; r < TUNE_RUNS && fine; ++r) {
+      fine = hipMemsetAsync(evict, 0, TUNE_EVICT_BYTES, stream) == hipSuccess &&
+             hipEventRecord(t0, stream) == hipSuccess && run() &&
+             hipEventRecord(t1, stream) == hipSuccess && hipEventSynchronize(t1) == hipSuccess &&
+             hipEventElapsedTime(&ms, t0, t1) == hipSuccess;
+      total += ms;
+      if (fine && r == 0 && best_ms > 0.f && ms > 3.f * best_ms) fine = false;
     }
+    if (!fine) {
+      (void)hipGetLastError();
+      continue;
+    }
+    ms = total / TUNE_RUNS;
     if (best_ms < 0.f || ms < best_ms) {
       best_ms = ms;
       best = (int)i;
@@ -326,8 +305,7 @@ ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int
           }
       } else if (!recording) {
         const auto began = std::chrono::steady_clock::now();
-        const int best = fastest_candidate(handle, kept, x, w, y, workspace, workspace_bytes,
-                                           M < TUNE_COLD_ROWS, stream);
+        const int best = fastest_candidate(handle, kept, x, w, y, workspace, workspace_bytes, stream);
         choose((size_t)best);
         if (tune_log())
           fprintf(stderr, "[zig_ai_amd] timed %zu candidates for M=%d N=%d K=%d P=%d %s: answer %d in %.1f ms\n",
