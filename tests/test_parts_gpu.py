@@ -185,6 +185,56 @@ def test_short_conv_part(dtype, bias):
         assert rel_err(torch.cat(got[r]), expect[r]) < TOL[dtype]
 
 
+@pytest.mark.parametrize("bias", [False, True])
+def test_short_conv_part_decoding_from_the_stream(bias, monkeypatch):
+    """The mixer given rows that still await their norm, as a block gives them: two
+    prompts in one step (the three kernels), then single tokens of both requests (norm,
+    in_proj and convolution in one kernel when in_proj has no bias), against the plain
+    norm and mixer on the whole sequences; the fused kernel is seen to run."""
+    from zig_ai_amd.cache import CacheManager
+    from zig_ai_amd.kernels import ops
+    from zig_ai_amd.parts import lookup
+    cls = lookup("mixer", "short_conv")
+    H, L, eps = 512, 3, 1e-5
+    params = {"hidden_size": H, "kernel_size": L, "bias": bias}
+    w = {"in_proj.weight": rnd((3 * H, H), 111, 0.05), "conv.weight": rnd((H, L), 112, 0.5),
+         "out_proj.weight": rnd((H, H), 113, 0.05)}
+    if bias:
+        w.update({"in_proj.bias": rnd((3 * H,), 114, 0.1), "conv.bias": rnd((H,), 115, 0.1)})
+    nw = (rnd((H,), 116, 0.2) + 1).to(dev())
+    part = cls(params, place(w, cls.tensor_rules(params), torch.bfloat16), runtime(torch.bfloat16))
+    cache = CacheManager({0: cls.cache_need(params)}, 4, 16, 3, device=dev(), dtype=torch.bfloat16)
+    view = cache.view(0)
+    streams = {"a": rnd((11, H), 117, 2.0), "b": rnd((6, H), 118, 2.0)}
+    bf = lambda t: t.to(torch.bfloat16).double()
+    wd = {"in_proj": bf(w["in_proj.weight"]), "conv": w["conv.weight"].double(), "out_proj": bf(w["out_proj.weight"])}
+    if bias:
+        wd.update({"in_proj_bias": w["in_proj.bias"].double(), "conv_bias": w["conv.bias"].double()})
+    expect = {r: plain.short_conv_mixer(plain.rms_norm(x.double(), nw.double().cpu(), eps), wd)
+              for r, x in streams.items()}
+    calls = []
+    fused = ops.in_proj_gated_conv
+    monkeypatch.setattr(ops, "in_proj_gated_conv", lambda *a, **k: (calls.append(a[0].shape[0]), fused(*a, **k))[1])
+    cuts = {"a": [7, 1, 1, 1, 1], "b": [2, 1, 1, 1, 1]}
+    done, got = {"a": 0, "b": 0}, {"a": [], "b": []}
+    for r in streams:
+        cache.admit(r)
+    for stepi in range(5):
+        entries = [(r, cuts[r][stepi]) for r in ("a", "b")]
+        step = step_for(cache, entries)
+        rows = torch.cat([streams[r][done[r]:done[r] + n] for r, n in entries]).to(dev())
+        y = total(part.forward(ops.NormedRows(rows, nw, eps, torch.bfloat16), step, view)).float().cpu()
+        row = 0
+        for r, n in entries:
+            got[r].append(y[row:row + n])
+            row += n
+            done[r] += n
+            cache.commit(r, n)
+    assert calls == ([] if bias else [2, 2, 2, 2])
+    for r in streams:
+        assert rel_err(torch.cat(got[r]), expect[r]) < TOL[torch.bfloat16]
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("nh,nkv,d,window", [(4, 2, 16, 0), (3, 1, 32, 0), (8, 2, 64, 0), (8, 2, 64, 20)])
 def test_attention_part(dtype, nh, nkv, d, window):
