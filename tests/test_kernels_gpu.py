@@ -450,18 +450,28 @@ def test_gemm_bf16_decode_rows_added_to_the_stream(M, N, K):
     assert back is not None and not kept.any()
 
 
-@pytest.mark.parametrize("M", [17, 40, 64, 200])
-@pytest.mark.parametrize("N,K,few_rows,more_rows", [
-    (2048, 8192, 8, 8), (2048, 2048, 8, 1), (300, 4096, 8, 8), (1024, 4608, 4, 4),
-    (2048, 4160, 1, 1), (6144, 2048, 1, 1), (64, 1024, 1, 1)])
-def test_gemm_bf16_library_partial_sums(M, N, K, few_rows, more_rows):
-    """Beyond a decode batch the library is given K in ranges when N is small (up
-    to 64 rows from K = 2048 on, up to LIBRARY_SPLIT_ROWS rows from 4096 on): the
+def library_ranges(M, N, K):
+    """The documented choice: with few outputs, K >= 4096 goes in 8 ranges up to 256 rows
+    and in 4 up to 512, K >= 2048 in 4 ranges up to 128 rows; a range is a multiple of
+    128 elements."""
+    choices = ()
+    if N <= 4096 and K >= 4096 and M <= 512:
+        choices = (8, 4, 2) if M <= 256 else (4, 2)
+    elif N <= 4096 and K >= 2048 and M <= 128:
+        choices = (4, 2)
+    return next((p for p in choices if K % (p * 128) == 0), 1)
+
+
+@pytest.mark.parametrize("M", [17, 40, 64, 128, 200, 300])
+@pytest.mark.parametrize("N,K", [(2048, 8192), (2048, 2048), (300, 4096), (1024, 4608), (2048, 4160),
+                                 (6144, 2048), (64, 1024)])
+def test_gemm_bf16_library_partial_sums(M, N, K):
+    """Beyond a decode batch the library is given K in ranges when N is small: the
     stack of 32-bit partial results sums to the product."""
     x, w = rand((M, K), torch.bfloat16, 42), rand((N, K), torch.bfloat16, 43)
     out = ops().linear(x.to(dev()), w.to(dev()), partial_ok=True)
     expect = x.double() @ w.double().T
-    split = few_rows if M <= 64 else more_rows
+    split = library_ranges(M, N, K)
     if split > 1:
         assert out.dim() == 3 and out.dtype == torch.float32 and out.shape == (split, M, N)
         assert out.is_contiguous()

@@ -293,10 +293,12 @@ def _k_splits(M: int, N: int, K: int) -> int:
 
     * up to 16 rows (the decode kernel): 4 ranges from K = 4096 on (8192: 15 us
       instead of 19.5), 2 ranges from 2048 on (8.3 instead of 8.9);
-    * more rows (the library, as one batched product over the ranges): 8 ranges
-      from K = 4096 on up to ``LIBRARY_SPLIT_ROWS`` rows (64 rows: 18 us instead
-      of 26; 512 rows: 33 instead of 41), and from K = 2048 on up to 64 rows
-      (12 instead of 13; no gain with more rows)."""
+    * more rows (the library, as one batched product over the ranges, its algorithm
+      timed at first use): from K = 4096 on 8 ranges up to 256 rows and 4 up to
+      ``LIBRARY_SPLIT_ROWS`` (K = 8192, 64 rows: 16.5 us instead of 19.9; 128 rows: 19.4
+      instead of 26.0; 512 rows: 32.2 instead of 40.7), and from K = 2048 on 4 ranges
+      up to 128 rows (64 rows: 11.4 instead of 11.7, 8 ranges 12.6; 128 rows: 13.5
+      instead of 15.8; 512 rows: one product is fastest)."""
     if N > 4096:
         return 1
     if M <= 16:
@@ -310,10 +312,14 @@ def _k_splits(M: int, N: int, K: int) -> int:
             if K % (split * 32) == 0:
                 return split
         return 1
-    if M <= LIBRARY_SPLIT_ROWS and (K >= 4096 or (K >= 2048 and M <= 64)):
-        for split in (8, 4, 2):
-            if K % (split * 128) == 0:
-                return split
+    choices = ()
+    if K >= 4096 and M <= LIBRARY_SPLIT_ROWS:
+        choices = (8, 4, 2) if M <= 256 else (4, 2)
+    elif K >= 2048 and M <= 128:
+        choices = (4, 2)
+    for split in choices:
+        if K % (split * 128) == 0:
+            return split
     return 1
 
 
