@@ -36,4 +36,4 @@ def test_every_plan_fits_the_kernel():
 def test_the_kernel_that_runs_the_norm_covers_k_alone():
     assert ops.accumulate_plan(8, 2048, 2048, True) == 1
     assert ops.normed_rows_pay(8, 2048, 2048) and not ops.normed_rows_pay(8, 2048, 4608)
-    assert not ops.normed_rows_pay(16, 2048, 2048) and ops.normed_rows_pay(16, 16384, 2048)
+    assert ops.normed_rows_pay(16, 2048, 2048) and not ops.normed_rows_pay(17, 16384, 2048)

@@ -979,7 +979,8 @@ def test_short_conv_whole_and_in_portions(dtype, H, L, bias):
 
 @pytest.mark.parametrize("M,H,L,bias", [(1, 512, 3, False), (8, 2048, 3, False), (5, 1024, 4, True),
                                         (8, 2560, 3, True), (3, 1536, 1, False), (7, 4096, 8, True),
-                                        (2, 3584, 2, False)])
+                                        (2, 3584, 2, False), (9, 1024, 3, True), (16, 2048, 3, False),
+                                        (13, 2560, 8, True)])
 def test_in_proj_gated_conv_is_the_three_kernels_in_one(M, H, L, bias):
     """A decode batch of the ShortConv mixer, one token a request: norm + in_proj +
     convolution in one kernel give the bits (outputs AND new state) that the norm inside
@@ -991,14 +992,14 @@ def test_in_proj_gated_conv_is_the_three_kernels_in_one(M, H, L, bias):
     taps = rand((H, L), torch.float32, 301)
     b = rand((H,), torch.float32, 302) if bias else None
     norm_w = (1.0 + 0.3 * rand((K,), torch.float32, 303)).to(dev())
-    slots = [5, 0, 7, 2, 6, 1, 3, 4][:M]
+    slots = [5, 0, 7, 2, 6, 1, 3, 4, 15, 9, 12, 8, 14, 10, 13, 11][:M]
     slot_id = torch.tensor(slots, dtype=torch.int32, device=dev())
     token_seq = torch.arange(M, dtype=torch.int32, device=dev())
     seq_start = torch.arange(M + 1, dtype=torch.int32, device=dev())
     taps_t, bd = taps.t().contiguous().to(dev()), b.to(dev()) if bias else None
 
     def memory():
-        mem = torch.zeros((8, H * L + 5), dtype=torch.float32, device=dev())
+        mem = torch.zeros((16, H * L + 5), dtype=torch.float32, device=dev())
         return mem, mem[:, 2:2 + H * L].unflatten(1, (H, L))
 
     (mem_a, state_a), (mem_b, state_b) = memory(), memory()
@@ -1026,7 +1027,7 @@ def test_in_proj_gated_conv_is_the_three_kernels_in_one(M, H, L, bias):
         assert rel_err(fused, zd[:, H:2 * H] * c) < BF16_TOL
     for m, slot in enumerate(slots):
         assert rel_err(state_a[slot].cpu().T, hist[m]) < F32_TOL
-    untouched = [s for s in range(8) if s not in slots]
+    untouched = [s for s in range(16) if s not in slots]
     assert (mem_a[untouched] == 0).all() and (mem_a[:, :2] == 0).all() and (mem_a[:, 2 + H * L:] == 0).all()
 
 
@@ -1034,8 +1035,8 @@ def test_in_proj_gated_conv_refuses_what_it_cannot_take():
     w = rand((3 * 96, 512), torch.bfloat16, 320).to(dev())          # width 96: fine; K 512
     taps = rand((3, 96), torch.float32, 321).to(dev())
     nw = torch.ones(512, device=dev())
-    many = ops().NormedRows(torch.zeros((9, 512), device=dev()), nw, 1e-5, torch.bfloat16)
-    assert not ops().gated_conv_fusable(many, w, taps)                 # nine rows
+    many = ops().NormedRows(torch.zeros((17, 512), device=dev()), nw, 1e-5, torch.bfloat16)
+    assert not ops().gated_conv_fusable(many, w, taps)                 # seventeen rows
     odd = ops().NormedRows(torch.zeros((2, 520), device=dev()), torch.ones(520, device=dev()), 1e-5,
                            torch.bfloat16)
     assert not ops().gated_conv_fusable(odd, rand((3 * 96, 520), torch.bfloat16, 322).to(dev()), taps)
@@ -1045,7 +1046,7 @@ def test_in_proj_gated_conv_refuses_what_it_cannot_take():
     assert not ops().gated_conv_fusable(few, rand((312, 512), torch.bfloat16, 324).to(dev()), narrow)
     with pytest.raises(ops().KernelError):
         ops().in_proj_gated_conv(many, w, taps, None, torch.zeros((1, 96, 3), device=dev()),
-                                 torch.zeros(9, dtype=torch.int32, device=dev()))
+                                 torch.zeros(17, dtype=torch.int32, device=dev()))
 
 
 def test_short_conv_identity_filter():

@@ -294,78 +294,6 @@ struct NormedRowsArg {
   float eps;
 };
 
-// Fills xa with the wave's slice of bf16(x * weight) and leaves the sum of squares of
-// the slice of row r in ssw[wave][r]; `nws` is room for the norm weight of the
-// workgroup's K range.  Ends with a barrier.  K is a multiple of a wave's slice
-// (KSTEPS * 32 elements), so a wave is either all inside K or has nothing to do.  A lane
-// without a row reads row 0 with its neighbours (row m of the product depends on row m
-// of the operand alone, and rows from M on are never stored): straight-line loads from
-// one address with the steps as constant offsets, all in flight together, and no
-// arithmetic beyond what a row needs (every workgroup repeats it).  `prefetch` is
-// called once the rows are requested, by the waves inside K only.
-template <int NW, int KSTEPS, typename Prefetch>
-__device__ __forceinline__ void load_normed_rows(bf16x8_t (&xa)[KSTEPS],
-                                                 const float* __restrict__ x,
-                                                 const int* __restrict__ rows,
-                                                 const float* __restrict__ weight, int M, int K,
-                                                 int tid, int kbase, float (&ssw)[NW][16],
-                                                 float* nws, Prefetch&& prefetch) {
-  static_assert(KSTEPS == 16, "a thread brings eight elements of the norm weight");
-  const int lane = tid & 63, wave = tid >> 6;
-  const int frag_row = lane & 15;
-  const bool rvalid = frag_row < M;
-  const bool inside = (wave + 1) * (KSTEPS * 32) <= K;      // the same for a whole wave
-  float ss = 0.f;
-  if (inside) {
-    const int row = rvalid ? frag_row : 0;
-    const size_t src = rows ? (size_t)rows[row] : (size_t)row;
-    const float* xk = x + src * K + kbase;
-    const f32x4_t n0 = *reinterpret_cast<const f32x4_t*>(weight + tid * 8);
-    const f32x4_t n1 = *reinterpret_cast<const f32x4_t*>(weight + tid * 8 + 4);
-    f32x4_t xf[KSTEPS][2];
-#pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) {
-      xf[s][0] = *reinterpret_cast<const f32x4_t*>(xk + s * 32);
-      xf[s][1] = *reinterpret_cast<const f32x4_t*>(xk + s * 32 + 4);
-    }
-    // the first weights are requested behind the rows and arrive while the rows are
-    // worked on (loads return in the order in which they were issued)
-    __builtin_amdgcn_sched_barrier(0);
-    prefetch();
-    __builtin_amdgcn_sched_barrier(0);
-    // a wave reads only the norm weights that its own lanes brought: no barrier yet
-    *reinterpret_cast<f32x4_t*>(nws + tid * 8) = n0;
-    *reinterpret_cast<f32x4_t*>(nws + tid * 8 + 4) = n1;
-#pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) {
-      // four steps' norm weights at a time: all 32 reads hoisted to the front would
-      // take as many registers again as the rows
-      if (s % 4 == 0) __builtin_amdgcn_sched_barrier(0);
-      const f32x4_t w0 = *reinterpret_cast<const f32x4_t*>(nws + kbase + s * 32);
-      const f32x4_t w1 = *reinterpret_cast<const f32x4_t*>(nws + kbase + s * 32 + 4);
-      bf16x8_t r;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float a = xf[s][0][e], b = xf[s][1][e];
-        ss += a * a;
-        ss += b * b;
-        r[e] = (bf16_t)(a * w0[e]);
-        r[4 + e] = (bf16_t)(b * w1[e]);
-      }
-      xa[s] = r;
-    }
-    // the four lanes that hold elements of a row; the waves are added up by the reader
-    ss += __shfl_xor(ss, 16, ZA_WAVE);
-    ss += __shfl_xor(ss, 32, ZA_WAVE);
-  } else {
-    const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) xa[s] = zero8;
-  }
-  if (lane < 16) ssw[wave][lane] = ss;
-  __syncthreads();
-}
-
 // The scale of row m from the waves' sums of squares, added in a fixed order.
 template <int NW>
 __device__ __forceinline__ float normed_row_scale(const float (&ssw)[NW][16], int m, int K, float eps) {
@@ -375,10 +303,10 @@ __device__ __forceinline__ float normed_row_scale(const float (&ssw)[NW][16], in
   return 1.0f / sqrtf(total / (float)K + eps);
 }
 
-// Up to eight rows reach the waves through LDS instead (STAGED): a wave reads its slice
-// of K of every row with one or two instructions a row, whole cache lines side by side,
-// and takes the fragments out of LDS.  The fragment loads above ask for every line of
-// the rows twice (each instruction takes 64 bytes of 16 rows), and with hundreds of
+// The step's rows reach the waves through LDS (STAGED): a wave reads its slice of K of
+// every row with one or two instructions a row, whole cache lines side by side, and takes
+// the matrix-core fragments out of LDS.  Fragment loads straight from memory ask for every
+// line of the rows twice (each instruction takes 64 bytes of 16 rows), and with hundreds of
 // workgroups asking for the same few lines at a kernel's start that is what a step of
 // few rows waits for: measured at 8 rows, gate|up of 8192 x 2048, 15.1 us with fragment
 // loads, 14.3 staged, 13.4 with no rows at all.  A staged row of a wave's slice takes
@@ -388,24 +316,33 @@ __device__ __forceinline__ float normed_row_scale(const float (&ssw)[NW][16], in
 #define ROWS16_STAGE_ROWS 8
 extern __shared__ __attribute__((aligned(16))) unsigned char rows16_staged[];
 
+// Nine to sixteen rows pass through the same eight places of LDS in two turns: the lanes
+// whose fragment row lies in the first eight rows take their fragments, then the other
+// eight rows are staged over them (a wave's LDS operations run in order).
+__host__ __device__ inline int rows16_stage_places(int M) {
+  return M < ROWS16_STAGE_ROWS ? M : ROWS16_STAGE_ROWS;
+}
 __host__ __device__ inline size_t rows16_stage_bytes(int nw, int M) {
-  return (size_t)nw * M * ROWS16_STAGE_STRIDE * sizeof(bf16_t);
+  return (size_t)nw * rows16_stage_places(M) * ROWS16_STAGE_STRIDE * sizeof(bf16_t);
 }
 
-// The fragments of the wave's slice, out of the rows it staged itself (LDS operations of
-// one wave run in order: no barrier).  A lane without a row reads row 0.
+// The fragments of the wave's slice for the lanes whose row is one of rows r0 .. r0 + 7,
+// out of the rows the wave staged itself (no barrier).  A lane without a row (row >= M)
+// takes place 0 in the first turn.
 template <int KSTEPS>
 __device__ __forceinline__ void staged_fragments(bf16x8_t (&xa)[KSTEPS], const bf16_t* mine, int M,
-                                                 int lane) {
+                                                 int lane, int r0) {
   const int frag_row = lane & 15, frag_k = (lane >> 4) * 8;
-  const bf16_t* fr = mine + (frag_row < M ? frag_row : 0) * ROWS16_STAGE_STRIDE + frag_k;
+  const bool valid = frag_row < M;
+  if ((valid ? frag_row & 8 : 0) != r0) return;
+  const bf16_t* fr = mine + (valid ? frag_row & 7 : 0) * ROWS16_STAGE_STRIDE + frag_k;
 #pragma unroll
   for (int s = 0; s < KSTEPS; ++s) xa[s] = *reinterpret_cast<const bf16x8_t*>(fr + s * 32);
 }
 
-// bfloat16 rows A [M, K], M <= ROWS16_STAGE_ROWS; `kslice` is the first k of the wave's
-// slice.  K is a multiple of 8, so a lane's eight elements are inside K or outside
-// together; outside, zeros are staged (the address read is moved inside the operand).
+// bfloat16 rows A [M, K], M <= 16; `kslice` is the first k of the wave's slice.  K is a
+// multiple of 8, so a lane's eight elements are inside K or outside together; outside,
+// zeros are staged (the address read is moved inside the operand).
 template <int KSTEPS, typename Prefetch>
 __device__ __forceinline__ void stage_rows(bf16x8_t (&xa)[KSTEPS], const bf16_t* __restrict__ A,
                                            int M, int K, int kslice, bf16_t* mine, int lane,
@@ -415,27 +352,33 @@ __device__ __forceinline__ void stage_rows(bf16x8_t (&xa)[KSTEPS], const bf16_t*
   const int k = kslice + lane * 8;
   const bool kin = k < K;
   const bf16_t* src = A + (kin ? k : 0);
-  bf16x8_t v[ROWS16_STAGE_ROWS];
+  bf16x8_t v[2 * ROWS16_STAGE_ROWS];
 #pragma unroll
-  for (int r = 0; r < ROWS16_STAGE_ROWS; ++r)
+  for (int r = 0; r < 2 * ROWS16_STAGE_ROWS; ++r)
     if (r < M) v[r] = *reinterpret_cast<const bf16x8_t*>(src + (size_t)r * K);
   // (weights requested behind the rows arrive while the rows pass through LDS)
   __builtin_amdgcn_sched_barrier(0);
   prefetch();
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int r = 0; r < ROWS16_STAGE_ROWS; ++r)
-    if (r < M)
-      *reinterpret_cast<bf16x8_t*>(mine + r * ROWS16_STAGE_STRIDE + lane * 8) = kin ? v[r] : zero8;
-  staged_fragments<KSTEPS>(xa, mine, M, lane);
+  for (int r0 = 0; r0 < 2 * ROWS16_STAGE_ROWS; r0 += ROWS16_STAGE_ROWS) {
+    if (r0 > 0 && M <= r0) break;
+#pragma unroll
+    for (int r = 0; r < ROWS16_STAGE_ROWS; ++r)
+      if (r0 + r < M)
+        *reinterpret_cast<bf16x8_t*>(mine + r * ROWS16_STAGE_STRIDE + lane * 8) = kin ? v[r0 + r] : zero8;
+    staged_fragments<KSTEPS>(xa, mine, M, lane, r0);
+  }
 }
 
-// load_normed_rows for M <= ROWS16_STAGE_ROWS through LDS: a lane reads four elements of
-// each half of the slice of every row, adds up their squares, and stages
-// bf16(x * weight).  The lanes' sums of squares of the eight rows meet in a butterfly
-// that halves the rows a lane carries at each of its first three steps: ten exchanges
-// instead of six a row, and the same tree of additions for every row wherever it stands.
-template <int NW, int KSTEPS, typename Prefetch>
+// Rows that await their norm (NormedRowsArg): a lane reads four elements of each half of
+// the wave's slice of every row, adds up their squares, and stages bf16(x * weight); eight
+// rows at a time, up to MAX_ROWS (8 or 16); the sums of squares of the slice of row r go
+// to ssw[wave][r].  `prefetch` is called once the first eight rows are requested, by the
+// waves inside K only.  Ends with a barrier.  The lanes' sums of squares of eight rows meet in a butterfly that halves the rows a lane
+// carries at each of its first three steps: ten exchanges instead of six a row, and the
+// same tree of additions for every row wherever it stands.
+template <int NW, int KSTEPS, int MAX_ROWS, typename Prefetch>
 __device__ __forceinline__ void stage_normed_rows(bf16x8_t (&xa)[KSTEPS],
                                                   const float* __restrict__ x,
                                                   const int* __restrict__ rows,
@@ -445,65 +388,71 @@ __device__ __forceinline__ void stage_normed_rows(bf16x8_t (&xa)[KSTEPS],
   static_assert(KSTEPS == 16, "two instructions of a wave cover a row's slice of 512 elements");
   const int lane = tid & 63, wave = tid >> 6;
   const bool inside = (wave + 1) * (KSTEPS * 32) <= K;      // the same for a whole wave
-  bf16_t* mine = staged + (size_t)wave * M * ROWS16_STAGE_STRIDE;
+  bf16_t* mine = staged + (size_t)wave * rows16_stage_places(M) * ROWS16_STAGE_STRIDE;
   if (inside) {
     const int kw = wave * (KSTEPS * 32) + lane * 4;
-    f32x4_t v[ROWS16_STAGE_ROWS][2];
-#pragma unroll
-    for (int r = 0; r < ROWS16_STAGE_ROWS; ++r)
-      if (r < M) {
-        const float* src = x + (rows ? (size_t)rows[r] : (size_t)r) * K + kw;
-        v[r][0] = *reinterpret_cast<const f32x4_t*>(src);
-        v[r][1] = *reinterpret_cast<const f32x4_t*>(src + 256);
-      }
     const f32x4_t n0 = *reinterpret_cast<const f32x4_t*>(weight + kw);
     const f32x4_t n1 = *reinterpret_cast<const f32x4_t*>(weight + kw + 256);
-    // the first weights are requested behind the rows and arrive while the rows are
-    // worked on (loads return in the order in which they were issued)
-    __builtin_amdgcn_sched_barrier(0);
-    prefetch();
-    __builtin_amdgcn_sched_barrier(0);
-    float p[ROWS16_STAGE_ROWS];
 #pragma unroll
-    for (int r = 0; r < ROWS16_STAGE_ROWS; ++r) {
-      p[r] = 0.f;
-      if (r < M) {
-        bf16x4_t lo, hi;
+    for (int r0 = 0; r0 < MAX_ROWS; r0 += ROWS16_STAGE_ROWS) {
+      if (r0 > 0 && M <= r0) break;
+      f32x4_t v[ROWS16_STAGE_ROWS][2];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float a = v[r][0][e], b = v[r][1][e];
-          p[r] += a * a;
-          p[r] += b * b;
-          lo[e] = (bf16_t)(a * n0[e]);
-          hi[e] = (bf16_t)(b * n1[e]);
+      for (int r = 0; r < ROWS16_STAGE_ROWS; ++r)
+        if (r0 + r < M) {
+          const float* src = x + (rows ? (size_t)rows[r0 + r] : (size_t)(r0 + r)) * K + kw;
+          v[r][0] = *reinterpret_cast<const f32x4_t*>(src);
+          v[r][1] = *reinterpret_cast<const f32x4_t*>(src + 256);
         }
-        bf16_t* dst = mine + r * ROWS16_STAGE_STRIDE + lane * 4;
-        *reinterpret_cast<bf16x4_t*>(dst) = lo;
-        *reinterpret_cast<bf16x4_t*>(dst + 256) = hi;
+      if (r0 == 0) {
+        // the first weights are requested behind the rows and arrive while the rows are
+        // worked on (loads return in the order in which they were issued)
+        __builtin_amdgcn_sched_barrier(0);
+        prefetch();
+        __builtin_amdgcn_sched_barrier(0);
       }
+      float p[ROWS16_STAGE_ROWS];
+#pragma unroll
+      for (int r = 0; r < ROWS16_STAGE_ROWS; ++r) {
+        p[r] = 0.f;
+        if (r0 + r < M) {
+          bf16x4_t lo, hi;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float a = v[r][0][e], b = v[r][1][e];
+            p[r] += a * a;
+            p[r] += b * b;
+            lo[e] = (bf16_t)(a * n0[e]);
+            hi[e] = (bf16_t)(b * n1[e]);
+          }
+          bf16_t* dst = mine + r * ROWS16_STAGE_STRIDE + lane * 4;
+          *reinterpret_cast<bf16x4_t*>(dst) = lo;
+          *reinterpret_cast<bf16x4_t*>(dst + 256) = hi;
+        }
+      }
+      // rows 4-7 go to the upper half of the lanes, then rows 2-3 and 6-7 to the lanes with
+      // bit 4, then the odd rows to the lanes with bit 3; three plain steps finish the sums
+      float q[4], t[2];
+      const bool b5 = lane & 32, b4 = lane & 16, b3 = lane & 8;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        q[i] = (b5 ? p[i + 4] : p[i]) + __shfl_xor(b5 ? p[i] : p[i + 4], 32, ZA_WAVE);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        t[i] = (b4 ? q[i + 2] : q[i]) + __shfl_xor(b4 ? q[i] : q[i + 2], 16, ZA_WAVE);
+      float u = (b3 ? t[1] : t[0]) + __shfl_xor(b3 ? t[0] : t[1], 8, ZA_WAVE);
+      u += __shfl_xor(u, 4, ZA_WAVE);
+      u += __shfl_xor(u, 2, ZA_WAVE);
+      u += __shfl_xor(u, 1, ZA_WAVE);
+      const int row = (b5 ? 4 : 0) + (b4 ? 2 : 0) + (b3 ? 1 : 0);
+      if ((lane & 7) == 0) ssw[wave][r0 + row] = u;
+      staged_fragments<KSTEPS>(xa, mine, M, lane, r0);
     }
-    // rows 4-7 go to the upper half of the lanes, then rows 2-3 and 6-7 to the lanes with
-    // bit 4, then the odd rows to the lanes with bit 3; three plain steps finish the sums
-    float q[4], t[2];
-    const bool b5 = lane & 32, b4 = lane & 16, b3 = lane & 8;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      q[i] = (b5 ? p[i + 4] : p[i]) + __shfl_xor(b5 ? p[i] : p[i + 4], 32, ZA_WAVE);
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-      t[i] = (b4 ? q[i + 2] : q[i]) + __shfl_xor(b4 ? q[i] : q[i + 2], 16, ZA_WAVE);
-    float u = (b3 ? t[1] : t[0]) + __shfl_xor(b3 ? t[0] : t[1], 8, ZA_WAVE);
-    u += __shfl_xor(u, 4, ZA_WAVE);
-    u += __shfl_xor(u, 2, ZA_WAVE);
-    u += __shfl_xor(u, 1, ZA_WAVE);
-    const int row = (b5 ? 4 : 0) + (b4 ? 2 : 0) + (b3 ? 1 : 0);
-    if ((lane & 7) == 0) ssw[wave][row] = u;
-    staged_fragments<KSTEPS>(xa, mine, M, lane);
   } else {
     const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) xa[s] = zero8;
-    if (lane < ROWS16_STAGE_ROWS) ssw[wave][lane] = 0.f;
+    if (lane < 16) ssw[wave][lane] = 0.f;
   }
   __syncthreads();
 }
@@ -516,7 +465,6 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
                         int accumulate) {
   __shared__ float red[2][NW][64][4];
   __shared__ float ssw[NW][16];
-  __shared__ float nws[NORM && !STAGED ? NW * KSTEPS * 32 : 1];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int frag_row = lane & 15, frag_k = (lane >> 4) * 8;
@@ -529,7 +477,8 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
   // a wave is all inside K or idle, and a row group's weights are loaded without conditions
   // (a lane beyond N reads row N - 1; its sums are never stored), the first group's while
   // the rows are on their way
-  constexpr bool FAST = NORM || STAGED;
+  static_assert(!NORM || STAGED, "rows that await their norm are staged through LDS");
+  constexpr bool FAST = STAGED;
   [[maybe_unused]] bf16x8_t fn[FAST ? KSTEPS : 1];
   [[maybe_unused]] const bool inside = (int)(blockIdx.y * NW + wave + 1) * (KSTEPS * 32) <= K;
   [[maybe_unused]] auto load_first = [&](auto first, auto last) {
@@ -545,24 +494,12 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
   if constexpr (NORM && STAGED) {
     // the rows take a quarter of the registers while they are on their way: the whole
     // first group is requested with them
-    stage_normed_rows<NW, KSTEPS>(xa, normed.x, normed.rows, normed.weight, M, K, tid, ssw,
-                                  staged, [&]() { load_first(S0, S2); });
-  } else if constexpr (NORM && ROLL) {
-    // the first half of the first group with the rows (whose 32-bit values fill half of
-    // the registers meanwhile), the second half once they are converted
-    load_normed_rows<NW, KSTEPS>(xa, normed.x, normed.rows, normed.weight, M, K, tid, kbase,
-                                 ssw, nws, [&]() { load_first(S0, S1); });
-    if (inside) {
-      load_first(S1, S2);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  } else if constexpr (NORM) {
-    load_normed_rows<NW, KSTEPS>(xa, normed.x, normed.rows, normed.weight, M, K, tid, kbase,
-                                 ssw, nws, [&]() { load_first(S0, S2); });
+    stage_normed_rows<NW, KSTEPS, 16>(xa, normed.x, normed.rows, normed.weight, M, K, tid, ssw,
+                                      staged, [&]() { load_first(S0, S2); });
   } else if constexpr (STAGED) {
     if (inside) {
       stage_rows<KSTEPS>(xa, A, M, K, (blockIdx.y * NW + wave) * KSTEPS * 32,
-                         staged + (size_t)wave * M * ROWS16_STAGE_STRIDE, lane,
+                         staged + (size_t)wave * rows16_stage_places(M) * ROWS16_STAGE_STRIDE, lane,
                          [&]() { load_first(S0, S2); });
     } else {
 #pragma unroll
@@ -686,8 +623,8 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
 //   u = B * x;  the state's L values move up by one and take u;  c = bias + sum_j w[j] * state[j];
 //   y = C * c
 // Slot, state and filter are requested at the kernel's start, so they have arrived when
-// the products are done.  Rows come as NormedRows, staged through LDS: M <= 8.
-template <int NW, int TILES>
+// the products are done.  Rows come as NormedRows, staged through LDS.
+template <int NW, int TILES, int MAX_ROWS>
 __global__ void __launch_bounds__(NW * 64, 2)
 gemm_bf16_rows16_gated_conv_kernel(NormedRowsArg normed, const bf16_t* __restrict__ W,
                                    const float* __restrict__ taps,
@@ -699,7 +636,7 @@ gemm_bf16_rows16_gated_conv_kernel(NormedRowsArg normed, const bf16_t* __restric
   constexpr int PER = CH / 4;                       // channels of a lane in the epilogue
   __shared__ float red[2][NW][64][4];
   __shared__ float ssw[NW][16];
-  __shared__ float zs[TILES * 16][ROWS16_STAGE_ROWS + 1];   // [weight row of the workgroup][token]
+  __shared__ float zs[TILES * 16][16 + 1];   // [weight row of the workgroup][token]
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int frag_row = lane & 15, frag_k = (lane >> 4) * 8;
@@ -719,27 +656,34 @@ gemm_bf16_rows16_gated_conv_kernel(NormedRowsArg normed, const bf16_t* __restric
   const bool mine = wave == 0 && m < M;
   float hist[MAXL][PER], wt[MAXL][PER], cb[PER];
   float* st = nullptr;
-  if (mine) {
-    st = state + (size_t)slot_id[m] * (size_t)slot_stride + (size_t)ch * L;
+  // (up to eight rows: before the rows are staged, so that the two trips to memory, slot
+  // then state, are over when the products are; with more rows the staging needs the
+  // registers, and the products take long enough for the loads to follow it)
+  auto request_state = [&]() {
+    if (mine) {
+      st = state + (size_t)slot_id[m] * (size_t)slot_stride + (size_t)ch * L;
 #pragma unroll
-    for (int j = 0; j < MAXL; ++j)
+      for (int j = 0; j < MAXL; ++j)
 #pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        hist[j][i] = j < L ? st[i * L + j] : 0.f;
-        wt[j][i] = j < L ? taps[(size_t)j * H + ch + i] : 0.f;
-      }
+        for (int i = 0; i < PER; ++i) {
+          hist[j][i] = j < L ? st[i * L + j] : 0.f;
+          wt[j][i] = j < L ? taps[(size_t)j * H + ch + i] : 0.f;
+        }
 #pragma unroll
-    for (int i = 0; i < PER; ++i) cb[i] = conv_bias ? conv_bias[ch + i] : 0.f;
-  }
+      for (int i = 0; i < PER; ++i) cb[i] = conv_bias ? conv_bias[ch + i] : 0.f;
+    }
+  };
+  if constexpr (MAX_ROWS <= ROWS16_STAGE_ROWS) request_state();
 
   bf16x8_t xa[KSTEPS], fn[KSTEPS];
-  stage_normed_rows<NW, KSTEPS>(xa, normed.x, normed.rows, normed.weight, M, K, tid, ssw,
-                                reinterpret_cast<bf16_t*>(rows16_staged), [&]() {
-                                  const bf16_t* wp = weight_row(0);
+  stage_normed_rows<NW, KSTEPS, MAX_ROWS>(xa, normed.x, normed.rows, normed.weight, M, K, tid,
+                                          ssw, reinterpret_cast<bf16_t*>(rows16_staged), [&]() {
+                                            const bf16_t* wp = weight_row(0);
 #pragma unroll
-                                  for (int s = 0; s < KSTEPS; ++s)
-                                    fn[s] = *reinterpret_cast<const bf16x8_t*>(wp + s * 32);
-                                });
+                                            for (int s = 0; s < KSTEPS; ++s)
+                                              fn[s] = *reinterpret_cast<const bf16x8_t*>(wp + s * 32);
+                                          });
+  if constexpr (MAX_ROWS > ROWS16_STAGE_ROWS) request_state();
   // One tile; `more` (a compile-time flag): the next tile's fragments are requested into
   // the registers that the products free.
   auto tile = [&](int t, auto more) {
@@ -821,7 +765,6 @@ gemm_bf16_rows16_swiglu_kernel(const bf16_t* __restrict__ A, NormedRowsArg norme
                                int K, int groups_per_block) {
   __shared__ float red[2][2][NW][64][4];
   __shared__ float ssw[NW][16];
-  __shared__ float nws[NORM && !STAGED ? NW * KSTEPS * 32 : 1];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int frag_row = lane & 15, frag_k = (lane >> 4) * 8;
@@ -846,20 +789,17 @@ gemm_bf16_rows16_swiglu_kernel(const bf16_t* __restrict__ A, NormedRowsArg norme
     }
   };
   constexpr std::integral_constant<int, 0> S0{};
-  constexpr std::integral_constant<int, KSTEPS / (STAGED ? 2 : 4)> S1{};
+  constexpr std::integral_constant<int, KSTEPS / 2> S1{};
   constexpr std::integral_constant<int, KSTEPS> S2{};
   [[maybe_unused]] bf16_t* staged = reinterpret_cast<bf16_t*>(rows16_staged);
   if constexpr (NORM && STAGED) {
     // (the rows take a quarter of the registers on their way: half of the first group
     // is requested with them)
-    stage_normed_rows<NW, KSTEPS>(xa, normed.x, normed.rows, normed.weight, M, K, tid, ssw,
-                                  staged, [&]() { load_steps(0, S0, S1); });
-  } else if constexpr (NORM) {
-    load_normed_rows<NW, KSTEPS>(xa, normed.x, normed.rows, normed.weight, M, K, tid, kbase,
-                                 ssw, nws, [&]() { load_steps(0, S0, S1); });
+    stage_normed_rows<NW, KSTEPS, 16>(xa, normed.x, normed.rows, normed.weight, M, K, tid, ssw,
+                                      staged, [&]() { load_steps(0, S0, S1); });
   } else if constexpr (STAGED) {
     stage_rows<KSTEPS>(xa, A, M, K, wave * KSTEPS * 32,
-                       staged + (size_t)wave * M * ROWS16_STAGE_STRIDE, lane, []() {});
+                       staged + (size_t)wave * rows16_stage_places(M) * ROWS16_STAGE_STRIDE, lane, []() {});
   } else {
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) {
@@ -1023,10 +963,9 @@ static int launch_rows16(const bf16_t* a, const NormedRowsArg* normed, const bf1
   if (groups_per_block > 0) per_block = groups_per_block;
   dim3 grid((groups + per_block - 1) / per_block, ksplit);
   const NormedRowsArg none = {nullptr, nullptr, nullptr, 0.f};
-  // up to ROWS16_STAGE_ROWS rows go through LDS (16 steps a wave only)
-  // (without the norm: only where K is a multiple of a wave's slice, the condition of the
-  // kernel's loads without conditions)
-  const bool stage = M <= ROWS16_STAGE_ROWS && (norm || K % 512 == 0);
+  // the rows go through LDS (16 steps a wave only; without the norm: only where K is a
+  // multiple of a wave's slice, the condition of the kernel's loads without conditions)
+  const bool stage = norm || K % 512 == 0;
 #define ZA_R16_LAUNCH(NW, KS, TC, NORM, STAGED, ROLL)                                         \
   {                                                                                           \
     const size_t lds = STAGED ? rows16_stage_bytes(NW, M) : 0;                                \
@@ -1040,21 +979,17 @@ static int launch_rows16(const bf16_t* a, const NormedRowsArg* normed, const bf1
     if (c_dtype == 0) ZA_R16_LAUNCH(NW, KS, float, NORM, STAGED, ROLL)                        \
     else ZA_R16_LAUNCH(NW, KS, bf16_t, NORM, STAGED, ROLL)                                    \
   }
-#define ZA_R16_NORM(NW, KS, STAGED)                                                           \
+#define ZA_R16_ROLL(NW, KS, NORM)                                                             \
   {                                                                                           \
-    if (per_block <= 2) ZA_R16_TYPES(NW, KS, true, STAGED, true)                              \
-    else ZA_R16_TYPES(NW, KS, true, STAGED, false)                                            \
+    if (per_block <= 2) ZA_R16_TYPES(NW, KS, NORM, true, true)                                \
+    else ZA_R16_TYPES(NW, KS, NORM, true, false)                                              \
   }
 #define ZA_R16_CASE(NW, KS)                                                                   \
   {                                                                                           \
     if constexpr (KS == 16) {                                                                 \
-      if (norm) {                                                                             \
-        if (stage) ZA_R16_NORM(NW, KS, true) else ZA_R16_NORM(NW, KS, false)                  \
-      } else {                                                                                \
-        if (stage && per_block <= 2) ZA_R16_TYPES(NW, KS, false, true, true)                  \
-        else if (stage) ZA_R16_TYPES(NW, KS, false, true, false)                              \
-        else ZA_R16_TYPES(NW, KS, false, false, false)                                        \
-      }                                                                                       \
+      if (norm) ZA_R16_ROLL(NW, KS, true)                                                     \
+      else if (stage) ZA_R16_ROLL(NW, KS, false)                                              \
+      else ZA_R16_TYPES(NW, KS, false, false, false)                                          \
     } else {                                                                                  \
       if (norm) return ZA_ERR_UNSUPPORTED;                                                    \
       ZA_R16_TYPES(NW, KS, false, false, false)                                               \
@@ -1067,7 +1002,7 @@ static int launch_rows16(const bf16_t* a, const NormedRowsArg* normed, const bf1
   if (kper <= 4096) ZA_R16_CASE(8, 16)
   ZA_R16_CASE(8, 32)
 #undef ZA_R16_CASE
-#undef ZA_R16_NORM
+#undef ZA_R16_ROLL
 #undef ZA_R16_TYPES
 #undef ZA_R16_LAUNCH
 }
@@ -1187,7 +1122,6 @@ extern "C" int za_gemm_bf16_rows16_swiglu(const void* A, const float* x, const i
   int per_block = groups >= 2048 ? 4 : (norm && groups >= 384 ? 2 : 1);
   if (rows16_groups_override > 0) per_block = rows16_groups_override;
   dim3 grid((groups + per_block - 1) / per_block);
-  const bool stage = M <= ROWS16_STAGE_ROWS;
 #define ZA_SG_LAUNCH(NW, KS, NORM, STAGED)                                                    \
   {                                                                                           \
     const size_t lds = STAGED ? rows16_stage_bytes(NW, M) : 0;                                \
@@ -1199,11 +1133,7 @@ extern "C" int za_gemm_bf16_rows16_swiglu(const void* A, const float* x, const i
 #define ZA_SG_CASE(NW, KS)                                                                    \
   {                                                                                           \
     if constexpr (KS == 16) {                                                                 \
-      if (norm) {                                                                             \
-        if (stage) ZA_SG_LAUNCH(NW, KS, true, true) else ZA_SG_LAUNCH(NW, KS, true, false)    \
-      } else {                                                                                \
-        if (stage) ZA_SG_LAUNCH(NW, KS, false, true) else ZA_SG_LAUNCH(NW, KS, false, false)  \
-      }                                                                                       \
+      if (norm) ZA_SG_LAUNCH(NW, KS, true, true) else ZA_SG_LAUNCH(NW, KS, false, true)       \
     } else {                                                                                  \
       if (norm) return ZA_ERR_UNSUPPORTED;                                                    \
       ZA_SG_LAUNCH(NW, KS, false, false)                                                      \
@@ -1220,7 +1150,7 @@ extern "C" int za_gemm_bf16_rows16_swiglu(const void* A, const float* x, const i
 }
 
 // The ShortConv mixer from the 32-bit stream to the convolution's output in one kernel
-// (gemm_bf16_rows16_gated_conv_kernel), for a decode batch of M <= 8 requests with one
+// (gemm_bf16_rows16_gated_conv_kernel), for a decode batch of M <= 16 requests with one
 // token each: row m of the product is token m and belongs to the request whose state
 // slot is slot_id[m].  W [3H, K] bfloat16 (B, C, x rows), taps [L, H] and conv_bias [H]
 // (or null) 32-bit, state as za_short_conv takes it, y [M, H] bfloat16.  K a multiple of
@@ -1236,7 +1166,7 @@ extern "C" int za_gemm_bf16_rows16_gated_conv(const float* x, const int* rows,
   if (M < 0 || H < 0 || K <= 0 || L <= 0 || !x || !norm_weight || !W || !taps || !state || !slot_id ||
       !y || slot_stride < (long long)H * L)
     return ZA_ERR_ARG;
-  if (M > ROWS16_STAGE_ROWS || H % 16 != 0 || L > 8 || !rows16_takes_norm(K, 1))
+  if (M > 16 || H % 16 != 0 || L > 8 || !rows16_takes_norm(K, 1))
     return ZA_ERR_UNSUPPORTED;
   if (channels != 0 && channels != 4 && channels != 8 && channels != 16) return ZA_ERR_ARG;
   // measured at 8 rows and at 1 (us; widths 1024, 1536, 2048, 2560, 4096):
@@ -1249,7 +1179,8 @@ extern "C" int za_gemm_bf16_rows16_gated_conv(const float* x, const int* rows,
 #define ZA_GC_LAUNCH(NW, TILES)                                                               \
   {                                                                                           \
     const size_t lds = rows16_stage_bytes(NW, M);                                             \
-    auto kernel = gemm_bf16_rows16_gated_conv_kernel<NW, TILES>;                              \
+    auto kernel = M <= ROWS16_STAGE_ROWS ? gemm_bf16_rows16_gated_conv_kernel<NW, TILES, 8>   \
+                                         : gemm_bf16_rows16_gated_conv_kernel<NW, TILES, 16>; \
     if (const int rc = rows16_allow_lds((const void*)kernel, lds)) return rc;                 \
     hipLaunchKernelGGL(kernel, grid, dim3(NW * 64), lds, stream, normed, (const bf16_t*)W,    \
                        taps, conv_bias, state, slot_stride, slot_id, (bf16_t*)y, M, H, K, L); \

@@ -255,17 +255,16 @@ def normed_rows_fusable(rows: int, width: int) -> bool:
 
 
 def _takes_normed_rows(x, weight: torch.Tensor, M: int, K: int) -> bool:
-    """Whether the product's kernel runs the norm itself.  Every workgroup reads the rows
-    in 32-bit, which costs more the more rows there are (measured at K = 2048 against the
-    norm kernel followed by the product: 2 to 2.6 us saved per product up to 8 rows, even
-    at 16), unless a workgroup walks many row groups with them (the gate|up projection:
-    2.7 us saved at 16 rows; the output head: 5 to 7 us)."""
+    """Whether the product's kernel runs the norm itself: every workgroup then reads the
+    step's rows in 32-bit (whole lines, staged through LDS) and a kernel is saved.  Measured
+    at K = 2048 against the norm kernel followed by the product: 2 to 2.5 us saved per
+    product at every row count up to 16."""
     return (isinstance(x, NormedRows) and x.dtype == torch.bfloat16
             and weight.dtype == torch.bfloat16 and normed_rows_pay(M, weight.shape[0], K))
 
 
 def normed_rows_pay(M: int, N: int, K: int) -> bool:
-    return normed_rows_fusable(M, K) and (M <= 8 or N >= 16384)
+    return normed_rows_fusable(M, K)
 
 
 # --------------------------------------------------------------------- gemm
@@ -775,12 +774,12 @@ def paged_attention_decode_mfma(q: torch.Tensor, kv_cache: torch.Tensor,
 
 
 # ---------------------------------------------------------------- short conv
-GATED_CONV_MAX_ROWS = 8
+GATED_CONV_MAX_ROWS = 16
 
 
 def gated_conv_fusable(x, w_in: torch.Tensor, taps: torch.Tensor) -> bool:
     """Whether ``in_proj_gated_conv`` takes these operands: rows that still await their
-    norm, at most eight of them, bfloat16 weights whose K the fused norm covers, and a
+    norm, at most sixteen of them, bfloat16 weights whose K the fused norm covers, and a
     width that is a multiple of 16."""
     if not isinstance(x, NormedRows) or x.dtype != torch.bfloat16 or w_in.dtype != torch.bfloat16:
         return False
