@@ -19,10 +19,9 @@
 // the first answer, 76 with the eighteenth; on [2048, 2048] 29 against 25; 64 rows on
 // [3072, 2048] 15.4 against 9.0, on [6144, 2048] 13.5 against 11.0), so with `tune` the first
 // call of a shape times the first TUNE_CANDIDATES answers on the call's own operands and
-// keeps the fastest.  In a model every weight comes from memory: between the timed runs
-// TUNE_EVICT_BYTES of a buffer allocated for the occasion are cleared, so that the weights
-// do not lie in a cache (timed warm, the ranking is another one: a decode step of 64 rows
-// got slower).  Shapes whose row counts fall into the same block (of
+// keeps the fastest.  In a model every weight comes from memory: the timed runs take turns
+// over copies of the weight, so that a run's weights do not lie in a cache (timed warm, the
+// ranking is another one: a decode step of 64 rows got slower).  Shapes whose row counts fall into the same block (of
 // TUNE_BUCKET rows from TUNE_BUCKET rows on, between two powers of two below) share the
 // choice, so a server that sees every batch size and portion length times a few dozen
 // shapes, some 10 ms each, not thousands.  (Naming the winner to the library by its index
@@ -64,7 +63,7 @@ constexpr int TUNE_MIN_ROWS = 17;      // (up to 16 rows this package's own kern
 constexpr size_t TUNE_MIN_WEIGHT = (size_t)1 << 19;   // elements: a megabyte of bfloat16; below, nothing to gain
 constexpr int TUNE_BUCKET = 256;
 constexpr int TUNE_CANDIDATES = 24;
-constexpr size_t TUNE_EVICT_BYTES = (size_t)320 << 20;   // more than the caches hold
+constexpr size_t TUNE_COPY_BYTES = (size_t)512 << 20;    // room for copies of a weight
 
 bool tune_log() {
   static const bool on = [] {
@@ -185,59 +184,78 @@ bool make_plan(hipblasLtHandle_t handle, int M, int N, int K, int out_f32, int P
 
 // Times the plan's candidates on the call's operands (y is overwritten by every one of
 // them, and by the product proper afterwards) and returns the fastest: one run to load
-// the kernel, then TUNE_RUNS timed ones, each alone behind a pass over a buffer larger
-// than the caches.  The stream is waited for; this happens once per block of row counts.
-// A candidate that fails, or takes three times the best so far in its first timed run,
-// is out.
+// the kernel, then TUNE_RUNS timed ones.  In a model a product's weights come from
+// memory, so the timed runs take turns over copies of the weight made for the occasion
+// (as many as fit TUNE_COPY_BYTES, at most TUNE_COPIES; the weight itself is one of the
+// turns): a run's weights were last touched several runs ago and have left the caches.
+// (Clearing a large buffer before every run instead left its write-backs in the timed
+// run's way and ranked the candidates differently from a loop over many weights.)  The
+// stream is waited for; this happens once per block of row counts.  A candidate that
+// fails is out.
 constexpr int TUNE_RUNS = 3;
+constexpr int TUNE_COPIES = 7;
 int fastest_candidate(hipblasLtHandle_t handle, const Plan& plan, const void* x, const void* w,
-                      void* y, void* workspace, size_t workspace_bytes, hipStream_t stream) {
-  void* evict = nullptr;
-  if (hipMalloc(&evict, TUNE_EVICT_BYTES) != hipSuccess) {
+                      size_t weight_bytes, void* y, void* workspace, size_t workspace_bytes,
+                      hipStream_t stream) {
+  int copies = (int)(TUNE_COPY_BYTES / weight_bytes);
+  if (copies > TUNE_COPIES) copies = TUNE_COPIES;
+  char* room = nullptr;
+  if (copies > 0 && hipMalloc((void**)&room, (size_t)copies * weight_bytes) != hipSuccess) {
     (void)hipGetLastError();
-    return 0;                     // no room to time it properly: the first answer
+    copies = 0;                   // no room: every run on the weight itself
   }
   struct Release {
     void* p;
     ~Release() { if (p) (void)hipFree(p); }
-  } release{evict};
+  } release{room};
+  for (int c = 0; c < copies; ++c)
+    if (hipMemcpyAsync(room + (size_t)c * weight_bytes, w, weight_bytes, hipMemcpyDeviceToDevice,
+                       stream) != hipSuccess) {
+      (void)hipGetLastError();
+      copies = c;
+      break;
+    }
   hipEvent_t t0 = nullptr, t1 = nullptr;
   if (hipEventCreate(&t0) != hipSuccess || hipEventCreate(&t1) != hipSuccess) {
     if (t0) (void)hipEventDestroy(t0);
     (void)hipGetLastError();
+    (void)hipStreamSynchronize(stream);
     return 0;
   }
+  int turn = 0;
+  auto next_weight = [&]() -> const void* {
+    const int c = turn++ % (copies + 1);
+    return c == copies ? w : (const void*)(room + (size_t)c * weight_bytes);
+  };
   int best = 0;
   float best_ms = -1.f;
   {
     // (the clocks come up under the first runs: the first candidate is not to pay for that)
     hipblasLtMatmulAlgo_t algo = plan.candidates[0].algo;
     for (int r = 0; r < 4; ++r)
-      (void)hipblasLtMatmul(handle, plan.op, &kOne, w, plan.a, x, plan.b, &kZero, y, plan.c, y, plan.c,
-                            &algo, workspace, workspace_bytes, stream);
+      (void)hipblasLtMatmul(handle, plan.op, &kOne, next_weight(), plan.a, x, plan.b, &kZero, y, plan.c,
+                            y, plan.c, &algo, workspace, workspace_bytes, stream);
   }
   for (size_t i = 0; i < plan.candidates.size(); ++i) {
     hipblasLtMatmulAlgo_t algo = plan.candidates[i].algo;
     auto run = [&]() {
-      return hipblasLtMatmul(handle, plan.op, &kOne, w, plan.a, x, plan.b, &kZero, y, plan.c, y,
-                             plan.c, &algo, workspace, workspace_bytes, stream) == HIPBLAS_STATUS_SUCCESS;
+      return hipblasLtMatmul(handle, plan.op, &kOne, next_weight(), plan.a, x, plan.b, &kZero, y,
+                             plan.c, y, plan.c, &algo, workspace, workspace_bytes,
+                             stream) == HIPBLAS_STATUS_SUCCESS;
     };
-    // one run to load the kernel, then every timed run alone, its weights out of the caches
-    float ms = 0.f, total = 0.f;
-    bool fine = run();
-    for (int r = 0; r < TUNE_RUNS && fine; ++r) {
-      fine = hipMemsetAsync(evict, 0, TUNE_EVICT_BYTES, stream) == hipSuccess &&
-             hipEventRecord(t0, stream) == hipSuccess && run() &&
-             hipEventRecord(t1, stream) == hipSuccess && hipEventSynchronize(t1) == hipSuccess &&
-             hipEventElapsedTime(&ms, t0, t1) == hipSuccess;
-      total += ms;
-      if (fine && r == 0 && best_ms > 0.f && ms > 3.f * best_ms) fine = false;
-    }
+    float ms = 0.f;
+    bool fine = run() && hipEventRecord(t0, stream) == hipSuccess;
+    for (int r = 0; r < TUNE_RUNS && fine; ++r) fine = run();
+    fine = fine && hipEventRecord(t1, stream) == hipSuccess && hipEventSynchronize(t1) == hipSuccess &&
+           hipEventElapsedTime(&ms, t0, t1) == hipSuccess;
     if (!fine) {
       (void)hipGetLastError();
       continue;
     }
-    ms = total / TUNE_RUNS;
+    ms /= TUNE_RUNS;
+    if (tune_log())
+      fprintf(stderr, "[zig_ai_amd]   answer %zu (the library's index %d): %.1f us\n", i,
+              hipblaslt_ext::getIndexFromAlgo(algo), ms * 1e3f);
     if (best_ms < 0.f || ms < best_ms) {
       best_ms = ms;
       best = (int)i;
@@ -305,7 +323,8 @@ ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int
           }
       } else if (!recording) {
         const auto began = std::chrono::steady_clock::now();
-        const int best = fastest_candidate(handle, kept, x, w, y, workspace, workspace_bytes, stream);
+        const int best = fastest_candidate(handle, kept, x, w, (size_t)N * K * sizeof(uint16_t), y,
+                                           workspace, workspace_bytes, stream);
         choose((size_t)best);
         if (tune_log())
           fprintf(stderr, "[zig_ai_amd] timed %zu candidates for M=%d N=%d K=%d P=%d %s: answer %d in %.1f ms\n",
