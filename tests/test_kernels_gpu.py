@@ -320,12 +320,12 @@ def _normed_operands(x: torch.Tensor, weight: torch.Tensor, eps: float):
 
 
 @pytest.mark.parametrize("K", [8, 512, 520, 1024, 1536, 2048, 2560, 3584, 4096, 4608])
-@pytest.mark.parametrize("M,N", [(1, 48), (8, 50), (16, 33), (16, 16400), (11, 16385)])
+@pytest.mark.parametrize("M,N", [(1, 48), (8, 50), (16, 33), (16, 16400), (11, 16385), (9, 200), (13, 96)])
 def test_gemm_bf16_decode_rows_normalised_by_the_kernel(M, N, K):
     """A norm that has not run yet as the product's input: every K the fused form takes
-    (multiples of 512 up to 4096, also those that leave waves idle; up to 8 rows, or up
-    to 16 with many outputs) and some it does not, with a bias, and rows picked out of a
-    longer stream.  The
+    (multiples of 512 up to 4096, also those that leave waves idle; up to 16 rows, nine
+    and more in two turns through LDS) and some it does not, with a bias, and rows picked
+    out of a longer stream.  The
     row's scale is applied to the 32-bit sums, so against the same operands the error
     is that of 32-bit summation; against the norm as a kernel of its own (which rounds
     after scaling) it is one bfloat16 rounding."""
