@@ -257,8 +257,8 @@ def test_gemm_bf16_partial_sums(M, N, K):
     stack = ops().linear(x.to(dev()), w.to(dev()), b.to(dev()), partial_ok=True)
     assert stack.dim() == 3 and stack.dtype == torch.float32 and stack.shape[0] in (2, 4)
     assert rel_err(stack.sum(0), x.double() @ w.double().T + b.double()) < F32_TOL
-    many = ops().linear(rand((600, K), torch.bfloat16, 33).to(dev()), w.to(dev()), partial_ok=True)
-    assert many.dim() == 2                                  # only small batches are split
+    many = ops().linear(rand((1100, K), torch.bfloat16, 33).to(dev()), w.to(dev()), partial_ok=True)
+    assert many.dim() == 2                                  # beyond 1,024 rows nothing is split
 
 
 def test_library_product_again_on_the_same_operands():
@@ -452,17 +452,17 @@ def test_gemm_bf16_decode_rows_added_to_the_stream(M, N, K):
 
 def library_ranges(M, N, K):
     """The documented choice: with few outputs, K >= 4096 goes in 8 ranges up to 256 rows
-    and in 4 up to 512, K >= 2048 in 4 ranges up to 128 rows; a range is a multiple of
+    and in 4 up to 1,024, K >= 2048 in 4 ranges up to 128 rows; a range is a multiple of
     128 elements."""
     choices = ()
-    if N <= 4096 and K >= 4096 and M <= 512:
+    if N <= 4096 and K >= 4096 and M <= 1024:
         choices = (8, 4, 2) if M <= 256 else (4, 2)
     elif N <= 4096 and K >= 2048 and M <= 128:
         choices = (4, 2)
     return next((p for p in choices if K % (p * 128) == 0), 1)
 
 
-@pytest.mark.parametrize("M", [17, 40, 64, 128, 200, 300])
+@pytest.mark.parametrize("M", [17, 40, 64, 128, 200, 300, 700, 1100])
 @pytest.mark.parametrize("N,K", [(2048, 8192), (2048, 2048), (300, 4096), (1024, 4608), (2048, 4160),
                                  (6144, 2048), (64, 1024)])
 def test_gemm_bf16_library_partial_sums(M, N, K):

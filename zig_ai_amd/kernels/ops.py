@@ -272,8 +272,8 @@ def normed_rows_pay(M: int, N: int, K: int) -> bool:
 # (measured: the decode kernel wins up to 16 rows, the library from there on).
 LIBRARY_GEMM_ROWS = 16
 # Up to this many rows the library is given K in ranges when the consumer takes
-# partial sums (a decode batch is too few rows to fill the chip with tiles of N alone).
-LIBRARY_SPLIT_ROWS = 512
+# partial sums (too few tiles of M x N to fill the chip when N is small).
+LIBRARY_SPLIT_ROWS = 1024
 
 
 def check_projection_weight(weight: torch.Tensor, what: str) -> None:
@@ -294,10 +294,14 @@ def _k_splits(M: int, N: int, K: int) -> int:
       instead of 19.5), 2 ranges from 2048 on (8.3 instead of 8.9);
     * more rows (the library, as one batched product over the ranges, its algorithm
       timed at first use): from K = 4096 on 8 ranges up to 256 rows and 4 up to
-      ``LIBRARY_SPLIT_ROWS`` (K = 8192, 64 rows: 16.5 us instead of 19.9; 128 rows: 19.4
-      instead of 26.0; 512 rows: 32.2 instead of 40.7), and from K = 2048 on 4 ranges
-      up to 128 rows (64 rows: 11.4 instead of 11.7, 8 ranges 12.6; 128 rows: 13.5
-      instead of 15.8; 512 rows: one product is fastest)."""
+      ``LIBRARY_SPLIT_ROWS`` (K = 8192 with the norm that adds the stack, 64 rows: 16.5 us
+      instead of 19.9; 512 rows: 32.9 instead of 42.0; 1,024 rows: 47.7 instead of 59.9; the
+      same order at N = 1024, K = 4608 and N = 2560, K = 10752; a whole step of the 1.2B
+      shape: 640 rows 2.72 -> 2.56 ms, 768 rows 3.28 -> 3.14, 1,024 rows 3.40 -> 3.29; with 2
+      ranges 1,280 rows 3.98 -> 3.95, 1,536 rows 4.32 -> 4.37, 2,048 rows 5.17 -> 5.14: left
+      as one product), and
+      from K = 2048 on 4 ranges up to 128 rows (64 rows: 11.4 instead of 11.7, 8 ranges
+      12.6; 128 rows: 13.5 instead of 15.8; from 192 rows on one product is fastest)."""
     if N > 4096:
         return 1
     if M <= 16:
