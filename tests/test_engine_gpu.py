@@ -429,7 +429,7 @@ def test_real_layer_sizes_every_way_of_cutting(kind, dtype):
         assert stats["pages_reused"] > 0, "the pool was too large to reuse a page"
     if dtype == "bfloat16":
         kernels = forms.kernels
-        assert "mfma" in kernels and ("decode_mfma" in kernels or kind in ("whole", "far portion"))
+        assert "mfma" in kernels and ("decode_mfma_rope" in kernels or kind in ("whole", "far portion"))
 
 
 def test_reproducible_decoding_at_real_layer_sizes():

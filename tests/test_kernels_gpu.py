@@ -916,6 +916,69 @@ def test_paged_attention_window_skips_freed_pages():
     assert rel_err(out, expect) < F32_TOL
 
 
+def decode_step_case(nh, nkv, d, page_size, positions, seed):
+    """A decode step: request i holds positions[i] cached tokens and brings one more.
+    Returns qkv [T, (nh + 2 nkv) d], the cache with random contents in the requests' pages
+    (the new tokens' places included: what was there before must not count), block table,
+    positions and the new tokens' places, all on the device."""
+    T = len(positions)
+    ks = [rand((p + 1, nkv, d), torch.bfloat16, seed + 2 * i) for i, p in enumerate(positions)]
+    vs = [rand((p + 1, nkv, d), torch.bfloat16, seed + 2 * i + 1) for i, p in enumerate(positions)]
+    cache, table = paged_from_dense(ks, vs, page_size, torch.bfloat16, seed=seed)
+    slots = torch.tensor([int(table[i, p // page_size]) * page_size + p % page_size
+                          for i, p in enumerate(positions)], dtype=torch.int32)
+    qkv = rand((T, (nh + 2 * nkv) * d), torch.bfloat16, seed + 100)
+    pos = torch.tensor(positions, dtype=torch.int32)
+    return qkv.to(dev()), cache.to(dev()), table.to(dev()), pos.to(dev()), slots.to(dev())
+
+
+@pytest.mark.parametrize("nh,nkv,d,page_size", [(8, 2, 64, 16), (3, 3, 64, 4), (16, 1, 64, 32),
+                                                (5, 1, 64, 12), (32, 8, 64, 16), (4, 2, 128, 16),
+                                                (6, 1, 128, 8), (2, 2, 128, 20)])
+@pytest.mark.parametrize("keys_per_split,nsplit,window", [(0, 1, 0), (256, 5, 0), (0, 1, 100),
+                                                          (128, 9, 70)])
+@pytest.mark.parametrize("norms", [True, False])
+def test_rope_attention_decode_is_the_two_kernels_in_one(nh, nkv, d, page_size, keys_per_split,
+                                                         nsplit, window, norms):
+    """A decode step's norm, rotation and cache write inside its attention kernel: the bits
+    of qk_norm_rope_kv_write followed by paged_attention_decode_mfma, in the result and in
+    the cache; positions at the edges of tiles (64 keys), of pages and of the ranges."""
+    o = ops()
+    positions = [0, 1, 3, 62, 63, 64, 65, 127, 128, 255, 256, 257, 700, 1023, 1100]
+    qkv, cache, table, pos, slots = decode_step_case(nh, nkv, d, page_size, positions, 900 + nh + d)
+    T = len(positions)
+    qw = (rand((d,), torch.float32, 901) * 0.3 + 1.0).to(dev()) if norms else None
+    kw = (rand((d,), torch.float32, 902) * 0.3 + 1.0).to(dev()) if norms else None
+    inv = (1.0 / torch.pow(torch.tensor(1e6, dtype=torch.float64),
+                           2.0 * torch.arange(0, d // 2, dtype=torch.float64) / d)).float().to(dev())
+    eps, scale = 1e-5, 1.0 / math.sqrt(d)
+    two = cache.clone()
+    q = o.qk_norm_rope_kv_write(qkv, pos, slots, qw, kw, inv, two, nh, nkv, d, d, False, eps)
+    want = o.paged_attention_decode_mfma(q, two, table, pos, None, None, None, T, scale, window,
+                                         keys_per_split, nsplit)
+    one = cache.clone()
+    got = o.rope_attention_decode(qkv, pos, slots, qw, kw, inv, one, table, nh, eps, scale, window,
+                                  keys_per_split, nsplit)
+    assert torch.equal(one, two)
+    assert torch.equal(got, want)
+    assert not torch.equal(one, cache)            # something was stored
+
+
+def test_rope_attention_decode_refuses_what_it_cannot_take():
+    o = ops()
+    qkv, cache, table, pos, slots = decode_step_case(4, 2, 64, 16, [5, 9], 950)
+    inv = torch.ones(32, device=dev())
+    assert not o.decode_rope_fusable(qkv, 4, 2, 64, 32, False, 16, 0.125)     # a partial rotation
+    assert not o.decode_rope_fusable(qkv, 4, 2, 64, 64, True, 16, 0.125)      # adjacent pairs
+    assert not o.decode_rope_fusable(qkv.float(), 4, 2, 64, 64, False, 16, 0.125)
+    assert not o.decode_rope_fusable(qkv, 4, 2, 64, 64, False, 6, 0.125)      # the page size
+    assert o.decode_rope_fusable(qkv, 4, 2, 64, 64, False, 16, 0.125)
+    with pytest.raises(ops().KernelError):
+        o.rope_attention_decode(qkv[:, :-64], pos, slots, None, None, inv, cache, table, 4, 1e-5, 0.125)
+    with pytest.raises(ops().KernelError):
+        o.rope_attention_decode(qkv, pos, slots[:1], None, None, inv, cache, table, 4, 1e-5, 0.125)
+
+
 # ------------------------------------------------------------------ short conv
 def conv_reference(z, w, b, H):
     B, C, x = z[:, :H], z[:, H:2 * H], z[:, 2 * H:]

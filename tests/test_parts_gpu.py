@@ -237,12 +237,18 @@ def test_short_conv_part_decoding_from_the_stream(bias, monkeypatch):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("nh,nkv,d,window", [(4, 2, 16, 0), (3, 1, 32, 0), (8, 2, 64, 0), (8, 2, 64, 20)])
-def test_attention_part(dtype, nh, nkv, d, window):
+def test_attention_part(dtype, nh, nkv, d, window, monkeypatch):
     """The mixer with its pages: a prompt portion, then single tokens, against the
-    plain mixer on the whole sequence."""
+    plain mixer on the whole sequence.  In bfloat16 with a head size the matrix cores take,
+    a step of single tokens runs norm, rotation and cache write inside its attention."""
     from zig_ai_amd.cache import CacheManager
     from zig_ai_amd.config.spec import PartSpec
+    from zig_ai_amd.kernels import ops
     from zig_ai_amd.parts import lookup
+    calls = []
+    fused = ops.rope_attention_decode
+    monkeypatch.setattr(ops, "rope_attention_decode",
+                        lambda *a, **k: (calls.append(a[0].shape[0]), fused(*a, **k))[1])
     cls = lookup("mixer", "gqa_attention")
     H, theta, eps = 80, 10000.0, 1e-5
     rope = PartSpec("rope", {"head_dim": d, "rotary_dim": d, "theta": theta, "pairing": "half"})
@@ -269,6 +275,7 @@ def test_attention_part(dtype, nh, nkv, d, window):
         done += n
     assert done == T
     assert rel_err(torch.cat(got), expect) < TOL[dtype]
+    assert calls == ([1] * 10 if dtype == torch.bfloat16 and d == 64 else [])
 
 
 @pytest.mark.parametrize("T", [12, 20])

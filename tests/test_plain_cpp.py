@@ -286,6 +286,7 @@ def test_kernel_attention_path_against_twin(dtype, nh, nkv, d, rot, adjacent, pa
     gpu_cache = torch.zeros((n_pages, 2, nkv, page_size, d), dtype=dtype, device=dev())
     G = nh // nkv
     mfma = ops().attention_mfma_supported(dtype, nh, nkv, d, page_size, 1.0)
+    fused_steps = []
     for step_no, step in enumerate(steps):
         pos, seq, slots, counts = [], [], [], []
         for s, lo, n in step:
@@ -295,6 +296,7 @@ def test_kernel_attention_path_against_twin(dtype, nh, nkv, d, rot, adjacent, pa
             counts.append(n)
         T = len(pos)
         qkv = rand((T, (nh + 2 * nkv) * d), 70 + step_no).to(dtype)
+        before = gpu_cache.clone()
         want_q = twin.qk_norm_rope_kv_write(qkv.float(), i32(pos), i32(slots), qw, kw, inv_freq, host_cache,
                                             nh, nkv, d, rot, adjacent, eps)
         got_q = ops().qk_norm_rope_kv_write(qkv.to(dev()), i32(pos).to(dev()), i32(slots).to(dev()),
@@ -319,6 +321,16 @@ def test_kernel_attention_path_against_twin(dtype, nh, nkv, d, rot, adjacent, pa
             got = fn(got_q, gpu_cache, step_table, i32(pos).to(dev()), item_seq, row0, cnt,
                      item_seq.numel(), 1.0 / math.sqrt(d), window)
             assert rel_err(got, want) < tol_of(dtype), (step_no, kind)
+        if max(counts) == 1 and ops().decode_rope_fusable(qkv, nh, nkv, d, rot, adjacent, page_size,
+                                                          1.0 / math.sqrt(d)):
+            # the two kernels in one, from the cache as it was before the step
+            got = ops().rope_attention_decode(qkv.to(dev()), i32(pos).to(dev()), i32(slots).to(dev()),
+                                              qw.to(dev()), kw.to(dev()), inv_freq.to(dev()), before,
+                                              step_table, nh, eps, 1.0 / math.sqrt(d), window)
+            assert rel_err(got, want) < tol_of(dtype), (step_no, "both in one")
+            assert rel_err(before, host_cache) < tol_of(dtype)
+            fused_steps.append(step_no)
+    assert fused_steps == ([2] if dtype == torch.bfloat16 and d in (64, 128) and rot == d else [])
 
 
 @pytest.mark.gpu

@@ -27,6 +27,7 @@
 #include <math.h>
 
 #include "common.h"
+#include "rope_math.h"
 
 #define AT_WAVES 4
 #define AT_RPW 8                     // rows per wave, at most
@@ -620,20 +621,41 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
 // side).  At the end the waves' partial (m, l, O) are merged in LDS; with
 // `nsplit` > 1 the merged partial goes to `attention_combine_kernel` like those of
 // the plain kernel.
-template <int D, int NWV>
+// ROPE: the kernel prepares its token's queries, key and value itself, from the step's fused
+// q|k|v projection: per-head RMSNorm of q and k, the rotation (half pairing over the whole
+// head), with rope_math.h's expressions and the order of additions of
+// qk_norm_rope_kv_write_pow2_kernel, so the bits are those of that kernel followed by this
+// one.  Every workgroup of a (request, key/value head) works the key out; the wave whose
+// tile holds the token's own position puts key and value into its fragments (the cache does
+// not hold them yet) and stores them to the cache for the steps to come.  One token a
+// work item only.
+struct DecodeRope {
+  const bf16_t* qkv;        // [tokens][nh + 2 nkv][D]
+  const int* slots;         // a token's place in the cache (page * page_size + offset), -1: none
+  const float* q_norm_w;    // [D] each, or null: no norm
+  const float* k_norm_w;
+  const float* inv_freq;    // [D / 2]
+  bf16_t* kv_write;         // the cache, to store the token's key and value
+  float eps;
+  int write_kv;
+};
+
+template <int D, int NWV, bool ROPE>
 __global__ void __launch_bounds__(NWV * 64)
 paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
-                                   const bf16_t* __restrict__ kv,
+                                   const bf16_t* kv,
                                    const int* __restrict__ block_table, int bt_stride,
                                    const int* __restrict__ positions,
                                    const int* __restrict__ wi_seq, const int* __restrict__ wi_row0,
                                    const int* __restrict__ wi_count, float* __restrict__ part_acc,
                                    float* __restrict__ part_ml, int nh, int nkv, int page_size,
-                                   float scale_log2e, int window, int keys_per_split, int nsplit) {
+                                   float scale_log2e, int window, int keys_per_split, int nsplit,
+                                   DecodeRope rope) {
   constexpr int KSTEPS = D / 32;
   constexpr int DBLK = D / 16;
   __shared__ float mg_m[NWV][16], mg_l[NWV][16];
   __shared__ float mg_o[NWV][DBLK][64][4];
+  [[maybe_unused]] __shared__ float rope_cs[ROPE ? D / 2 : 1], rope_sn[ROPE ? D / 2 : 1];
 
   const int item = blockIdx.x, gkv = blockIdx.y, z = blockIdx.z;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -653,11 +675,26 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
   const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 
   bf16x8_t qf[KSTEPS];
+  [[maybe_unused]] bf16x8_t knew[KSTEPS];     // ROPE: the token's key, as this lane's fragments
+  [[maybe_unused]] bf16_t vnew[DBLK];         // and its value at head-dim elements db * 16 + r16
+  [[maybe_unused]] float xq[KSTEPS][8], xk[KSTEPS][8];
+  if constexpr (ROPE) {
+    // the raw rows are requested first of all; they are worked on once the position is known
+    const bf16_t* row = rope.qkv + (size_t)tok * (nh + 2 * nkv) * D;
 #pragma unroll
-  for (int ks = 0; ks < KSTEPS; ++ks)
-    qf[ks] = row_valid ? *reinterpret_cast<const bf16x8_t*>(
-                             q + ((size_t)tok * nh + head) * D + ks * 32 + grp * 8)
-                       : zero8;
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      load8<bf16_t>(row + (size_t)head * D + ks * 32 + grp * 8, xq[ks]);
+      load8<bf16_t>(row + (size_t)(nh + gkv) * D + ks * 32 + grp * 8, xk[ks]);
+    }
+#pragma unroll
+    for (int db = 0; db < DBLK; ++db) vnew[db] = row[(size_t)(nh + nkv + gkv) * D + db * 16 + r16];
+  } else {
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks)
+      qf[ks] = row_valid ? *reinterpret_cast<const bf16x8_t*>(
+                               q + ((size_t)tok * nh + head) * D + ks * 32 + grp * 8)
+                         : zero8;
+  }
 
   f32x4_t o[DBLK];
 #pragma unroll
@@ -782,6 +819,53 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
     if (ps_shift >= 4) load_entries(tile0);
     fetch(tile0, 0, kf, vf);
   }
+  if constexpr (ROPE) {
+    if (tid < D / 2) rope_angle(pos_last, rope.inv_freq[tid], &rope_cs[tid], &rope_sn[tid]);
+    __syncthreads();
+    // chunk ks * 4 + grp of a head is this lane's x[ks]; the sums of squares meet as in the
+    // kernel this replaces: partners half the head apart first, then ever closer ones
+    auto finish = [&](float (&x)[KSTEPS][8], const float* nw, bf16x8_t (&frag)[KSTEPS]) {
+      if (nw) {
+        float ss[KSTEPS];
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) ss[ks] = rope_sum_squares8(x[ks]);
+#pragma unroll
+        for (int o = KSTEPS / 2; o > 0; o >>= 1)
+#pragma unroll
+          for (int ks = 0; ks < o; ++ks) ss[ks] += ss[ks + o];
+        float t = ss[0];
+        t += __shfl_xor(t, 32, ZA_WAVE);
+        t += __shfl_xor(t, 16, ZA_WAVE);
+        const float norm_scale = rope_rms_scale(t, D, rope.eps);
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          float w8[8];
+          load8<float>(nw + ks * 32 + grp * 8, w8);
+          rope_scale8(x[ks], norm_scale, w8);
+        }
+      }
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS / 2; ++ks)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int p = ks * 32 + grp * 8 + i;
+          const float cs = rope_cs[p], sn = rope_sn[p];
+          const float lo = x[ks][i], hi = x[ks + KSTEPS / 2][i];
+          x[ks][i] = rope_rotate_low(lo, hi, cs, sn);
+          x[ks + KSTEPS / 2][i] = rope_rotate_high(hi, lo, cs, sn);
+        }
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) frag[ks][i] = (bf16_t)x[ks][i];
+    };
+    finish(xq, rope.q_norm_w, qf);
+    if (!row_valid) {
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) qf[ks] = zero8;
+    }
+    finish(xk, rope.k_norm_w, knew);
+  }
   int nth = 0;
   for (; tile0 <= range_hi; tile0 += NWV * AM_KT) {
     bf16x8_t kfn[4][KSTEPS];
@@ -793,6 +877,43 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
         if (ps_shift >= 4) load_entries(next);
       }
       fetch(next, nth, kfn, vfn);
+    }
+    if constexpr (ROPE) {
+      // the tile with the token's own position (one wave of one workgroup meets it): key
+      // and value are not in the cache yet, they go into the fragments here and from here
+      // into the cache
+      const int own = pos_last - tile0;
+      if (own >= 0 && own < AM_KT) {
+#pragma unroll
+        for (int jb = 0; jb < 4; ++jb)
+          if ((jb >> 1) * 32 + (jb & 1) * 4 + krow_in_pair == own) {
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) kf[jb][ks] = knew[ks];
+          }
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (kk * 32 + grp * 8 + e == own) {
+#pragma unroll
+              for (int db = 0; db < DBLK; ++db) vf[db][kk][e] = vnew[db];
+            }
+        const int slot = rope.write_kv ? rope.slots[tok] : -1;
+        if (slot >= 0) {
+          const int page = slot / page_size, off = slot % page_size;
+          if (r16 == 0) {
+            bf16_t* dst = rope.kv_write + ((((size_t)page * 2) * nkv + gkv) * page_size + off) * D;
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks)
+              *reinterpret_cast<bf16x8_t*>(dst + ks * 32 + grp * 8) = knew[ks];
+          }
+          if (grp == 0) {
+            bf16_t* dst = rope.kv_write + (((size_t)page * 2 + 1) * nkv + gkv) * page_size * D + off;
+#pragma unroll
+            for (int db = 0; db < DBLK; ++db) dst[(size_t)(db * 16 + r16) * page_size] = vnew[db];
+          }
+        }
+      }
     }
     // A key that must not count is masked in the scores, whatever its row holds; its
     // values are cleared, since 0 * (not a number) would not be 0.  (Keys whose page is
@@ -1049,6 +1170,41 @@ extern "C" int za_paged_attention_mfma(const void* q, void* out, const void* kv,
 #undef ZA_AM_ARGS
 }
 
+template <bool ROPE>
+static int launch_decode_mfma(const void* q, void* out, const void* kv, const int* block_table,
+                              int bt_stride, const int* positions, const int* wi_seq,
+                              const int* wi_row0, const int* wi_count, int n_items, int n_tokens,
+                              float* part_acc, float* part_ml, int nh, int nkv, int d,
+                              int page_size, float scale, int window, int keys_per_split,
+                              int nsplit, const DecodeRope& rope, hipStream_t stream) {
+  dim3 grid(n_items, nkv, nsplit), block(256);
+  // Few workgroups (a small batch): eight waves each, so that a compute unit that
+  // gets one workgroup still has eight waves' loads in flight.
+  const long long workgroups = (long long)n_items * nkv * nsplit;
+  if (d == 64 && workgroups <= ZA_DECODE_WIDE_BELOW) {
+    hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<64, 8, ROPE>), grid, dim3(512), 0, stream,
+                       (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
+                       positions, wi_seq, wi_row0, wi_count, part_acc, part_ml, nh, nkv,
+                       page_size, scale * 1.44269504088896341f, window, keys_per_split, nsplit, rope);
+  } else if (d == 64) {
+    hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<64, 4, ROPE>), grid, block, 0, stream,
+                       (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
+                       positions, wi_seq, wi_row0, wi_count, part_acc, part_ml, nh, nkv,
+                       page_size, scale * 1.44269504088896341f, window, keys_per_split, nsplit, rope);
+  } else {
+    hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<128, 4, ROPE>), grid, block, 0, stream,
+                       (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
+                       positions, wi_seq, wi_row0, wi_count, part_acc, part_ml, nh, nkv,
+                       page_size, scale * 1.44269504088896341f, window, keys_per_split, nsplit, rope);
+  }
+  int rc = za_launch_status();
+  if (rc != 0 || nsplit == 1) return rc;
+  dim3 cgrid((unsigned)((size_t)n_tokens * nh)), cblock(64);
+  hipLaunchKernelGGL((attention_combine_kernel<bf16_t>), cgrid, cblock, 0, stream, part_acc,
+                     part_ml, (bf16_t*)out, d, nsplit, 1);
+  return za_launch_status();
+}
+
 // Matrix-core decode variant: bfloat16, head_dim 64 or 128, page sizes that are
 // multiples of 4, work items of at most 16 / (nh / nkv) query tokens, contexts
 // optionally cut as in
@@ -1073,30 +1229,37 @@ extern "C" int za_paged_attention_decode_mfma(const void* q, void* out, const vo
     return ZA_ERR_UNSUPPORTED;
   if (nsplit > 1 && (!part_acc || !part_ml || keys_per_split <= 0 || keys_per_split % 64 != 0))
     return ZA_ERR_ARG;
-  dim3 grid(n_items, nkv, nsplit), block(256);
-  // Few workgroups (a small batch): eight waves each, so that a compute unit that
-  // gets one workgroup still has eight waves' loads in flight.
-  const long long workgroups = (long long)n_items * nkv * nsplit;
-  if (d == 64 && workgroups <= ZA_DECODE_WIDE_BELOW) {
-    hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<64, 8>), grid, dim3(512), 0, stream,
-                       (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
-                       positions, wi_seq, wi_row0, wi_count, part_acc, part_ml, nh, nkv,
-                       page_size, scale * 1.44269504088896341f, window, keys_per_split, nsplit);
-  } else if (d == 64) {
-    hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<64, 4>), grid, block, 0, stream,
-                       (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
-                       positions, wi_seq, wi_row0, wi_count, part_acc, part_ml, nh, nkv,
-                       page_size, scale * 1.44269504088896341f, window, keys_per_split, nsplit);
-  } else {
-    hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<128, 4>), grid, block, 0, stream,
-                       (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
-                       positions, wi_seq, wi_row0, wi_count, part_acc, part_ml, nh, nkv,
-                       page_size, scale * 1.44269504088896341f, window, keys_per_split, nsplit);
-  }
-  int rc = za_launch_status();
-  if (rc != 0 || nsplit == 1) return rc;
-  dim3 cgrid((unsigned)((size_t)n_tokens * nh)), cblock(64);
-  hipLaunchKernelGGL((attention_combine_kernel<bf16_t>), cgrid, cblock, 0, stream, part_acc,
-                     part_ml, (bf16_t*)out, d, nsplit, 1);
-  return za_launch_status();
+  const DecodeRope none = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0};
+  return launch_decode_mfma<false>(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0,
+                                   wi_count, n_items, n_tokens, part_acc, part_ml, nh, nkv, d,
+                                   page_size, scale, window, keys_per_split, nsplit, none, stream);
+}
+
+// The same for a step in which every request brings one token, with the token's part of
+// qk_norm_rope_kv_write in the kernel's prologue: `qkv` is the fused projection
+// [n_tokens][nh + 2 nkv][d] as it leaves the product; queries and key get their per-head
+// RMSNorm (weights may be null) and the rotation over the whole head with half pairing
+// (rotary_dim == d, pairs (p, p + d / 2)), key and value go to the cache at `slots`
+// (page * page_size + offset, -1: not stored).  The result and the cache hold the bits that
+// za_qk_norm_rope_kv_write followed by za_paged_attention_decode_mfma leave.
+extern "C" int za_paged_attention_decode_mfma_rope(
+    const void* qkv, void* out, void* kv, const int* block_table, int bt_stride,
+    const int* positions, const int* slots, const float* q_norm_w, const float* k_norm_w,
+    const float* inv_freq, float eps, int n_tokens, float* part_acc, float* part_ml, int nh,
+    int nkv, int d, int page_size, float scale, int window, int keys_per_split, int nsplit,
+    hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  if (n_tokens < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || page_size <= 0 || bt_stride <= 0 ||
+      nsplit < 1 || !qkv || !out || !kv || !block_table || !positions || !slots || !inv_freq)
+    return ZA_ERR_ARG;
+  const int G = nh / nkv;
+  if ((d != 64 && d != 128) || G > 16 || page_size % 4 != 0 || nkv > 65535 || nsplit > 65535)
+    return ZA_ERR_UNSUPPORTED;
+  if (nsplit > 1 && (!part_acc || !part_ml || keys_per_split <= 0 || keys_per_split % 64 != 0))
+    return ZA_ERR_ARG;
+  const DecodeRope rope = {(const bf16_t*)qkv, slots, q_norm_w, k_norm_w, inv_freq, (bf16_t*)kv,
+                           eps, 1};
+  return launch_decode_mfma<true>(nullptr, out, kv, block_table, bt_stride, positions, nullptr,
+                                  nullptr, nullptr, n_tokens, n_tokens, part_acc, part_ml, nh, nkv,
+                                  d, page_size, scale, window, keys_per_split, nsplit, rope, stream);
 }

@@ -16,6 +16,7 @@
 //        read, for one head-dimension element, consecutive keys side by side)
 //   q    -> q_out[token][head][head_dim]
 #include "common.h"
+#include "rope_math.h"
 
 #define RK_MAX_D 256
 
@@ -164,9 +165,8 @@ qk_norm_rope_kv_write_pow2_kernel(const T* __restrict__ qkv, const int* __restri
   if ((int)threadIdx.x / LPH < heads_here)
     load8<T>(qkv + ((size_t)t * total + threadIdx.x / LPH) * D + e0, xn);
   if ((int)threadIdx.x < half) {
-    const float angle = (float)positions[t] * inv_freq[threadIdx.x];
     float sn, cs;
-    sincosf(angle, &sn, &cs);
+    rope_angle(positions[t], inv_freq[threadIdx.x], &cs, &sn);
     cs_tab[threadIdx.x] = cs;
     sn_tab[threadIdx.x] = sn;
   }
@@ -181,16 +181,15 @@ qk_norm_rope_kv_write_pow2_kernel(const T* __restrict__ qkv, const int* __restri
       load8<T>(qkv + ((size_t)t * total + head + 256 / LPH) * D + e0, xn);
     const float* nw = is_q ? q_norm_w : (is_k ? k_norm_w : nullptr);
     if (nw) {
-      float ss = 0.f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) ss += x[i] * x[i];
+      // (the decode attention's prologue adds the lanes' sums up in this order too:
+      // partners 4 lanes apart first, then 2, then 1)
+      float ss = rope_sum_squares8(x);
 #pragma unroll
       for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
-      const float scale = 1.0f / sqrtf(ss / (float)D + eps);
+      const float scale = rope_rms_scale(ss, D, eps);
       float w8[8];
       load8<float>(nw + e0, w8);     // two 16-byte loads, not eight of 4 bytes
-#pragma unroll
-      for (int i = 0; i < 8; ++i) x[i] = x[i] * scale * w8[i];
+      rope_scale8(x, scale, w8);
     }
     if ((is_q || is_k) && rot > 0) {
       if (adjacent) {
@@ -212,7 +211,7 @@ qk_norm_rope_kv_write_pow2_kernel(const T* __restrict__ qkv, const int* __restri
           if (in_rot) {
             const int p = low ? e0 + i : e0 + i - half;
             const float cs = cs_tab[p], sn = sn_tab[p];
-            x[i] = low ? x[i] * cs - other * sn : other * sn + x[i] * cs;
+            x[i] = low ? rope_rotate_low(x[i], other, cs, sn) : rope_rotate_high(x[i], other, cs, sn);
           }
         }
       }

@@ -39,7 +39,8 @@ HIPCC_FLAGS = [
 ]
 
 EXTRA_FLAGS = {"blaslt": ["-lhipblaslt"]}   # host code around the GEMM library, no kernels
-EXTRA_HEADERS = {"sampling": ["no_alloc.h"]}    # headers a source includes beside common.h
+# headers a source includes beside common.h
+EXTRA_HEADERS = {"sampling": ["no_alloc.h"], "rope_kv": ["rope_math.h"], "attention": ["rope_math.h"]}
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()

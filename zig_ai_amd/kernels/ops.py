@@ -47,6 +47,10 @@ _SIGNATURES = {
                                                       c_void_p, c_int, c_int, c_void_p, c_void_p,
                                                       c_int, c_int, c_int, c_int, c_float, c_int,
                                                       c_int, c_int, c_void_p],
+    ("attention", "za_paged_attention_decode_mfma_rope"): [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+        c_void_p, c_float, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int,
+        c_int, c_int, c_void_p],
     ("shortconv", "za_short_conv"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                      c_longlong, c_void_p],
@@ -774,6 +778,65 @@ def paged_attention_decode_mfma(q: torch.Tensor, kv_cache: torch.Tensor,
         int(keys_per_split), int(nsplit), _stream())
     _check(rc, "paged_attention_decode_mfma")
     _note("attention", kernel="decode_mfma", rows=T, dtype=q.dtype, nsplit=int(nsplit))
+    return out
+
+
+def decode_rope_fusable(qkv, num_heads: int, num_kv_heads: int, head_dim: int, rotary_dim: int,
+                        adjacent_pairs: bool, page_size: int, scale: float) -> bool:
+    """Whether ``rope_attention_decode`` takes the step: bfloat16, the rotation over the whole
+    head with half pairing, and what the matrix-core decode kernel takes."""
+    return (qkv.dtype == torch.bfloat16 and rotary_dim == head_dim and not adjacent_pairs
+            and attention_mfma_supported(qkv.dtype, num_heads, num_kv_heads, head_dim, page_size,
+                                         scale)
+            and num_heads // num_kv_heads <= ATTENTION_MFMA_DECODE_ROWS)
+
+
+def rope_attention_decode(qkv: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor,
+                          q_norm_w: Optional[torch.Tensor], k_norm_w: Optional[torch.Tensor],
+                          inv_freq: torch.Tensor, kv_cache: torch.Tensor,
+                          block_table: torch.Tensor, num_heads: int, eps: float, scale: float,
+                          window: int = 0, keys_per_split: int = 0,
+                          nsplit: int = 1) -> torch.Tensor:
+    """A step in which request ``i`` brings the one token of row ``i``: what
+    ``qk_norm_rope_kv_write`` followed by ``paged_attention_decode_mfma`` does, in the
+    attention's kernel (its prologue normalises and rotates the token's queries and key;
+    the workgroup that meets the token's own position stores key and value to the cache).
+    The same bits in the result and in the cache, one kernel and one trip through memory
+    less.  Returns the attention's output ``[T, heads, head_dim]``."""
+    if kv_cache.dim() != 5 or kv_cache.shape[1] != 2:
+        raise KernelError(f"kv_cache has shape {tuple(kv_cache.shape)}, expected "
+                          f"[pages, 2, kv_heads, page_size, head_dim]")
+    nkv, page_size, d = kv_cache.shape[2], kv_cache.shape[3], kv_cache.shape[4]
+    T = qkv.shape[0]
+    nh = int(num_heads)
+    _need(qkv, "qkv", torch.bfloat16, (T, (nh + 2 * nkv) * d))
+    _need(kv_cache, "kv_cache", torch.bfloat16)
+    if nh % nkv or not decode_rope_fusable(qkv, nh, nkv, d, d, False, page_size, scale):
+        raise KernelError(f"rope_attention_decode does not take {nh} heads, {nkv} key/value "
+                          f"heads, head_dim {d}, page size {page_size}, scale {scale}")
+    _need(block_table, "block_table", torch.int32)
+    if block_table.dim() != 2 or block_table.shape[0] < T:
+        raise KernelError("block_table must be [requests, max_pages] with a row per token")
+    _need(positions, "positions", torch.int32, (T,))
+    _need(slots, "slots", torch.int32, (T,))
+    _need(inv_freq, "inv_freq", torch.float32, (d // 2,))
+    for name, w in (("q_norm_w", q_norm_w), ("k_norm_w", k_norm_w)):
+        if w is not None:
+            _need(w, name, torch.float32, (d,))
+    out = torch.empty((T, nh, d), dtype=torch.bfloat16, device=qkv.device)
+    part_acc = part_ml = None
+    if nsplit > 1:
+        if keys_per_split <= 0 or keys_per_split % 64:
+            raise KernelError("keys_per_split must be a positive multiple of 64")
+        part_acc = torch.empty((T, nh, nsplit, d), dtype=torch.float32, device=qkv.device)
+        part_ml = torch.empty((T, nh, nsplit, 2), dtype=torch.float32, device=qkv.device)
+    rc = _fn("attention", "za_paged_attention_decode_mfma_rope")(
+        _ptr(qkv), _ptr(out), _ptr(kv_cache), _ptr(block_table), block_table.shape[1],
+        _ptr(positions), _ptr(slots), _ptr(q_norm_w), _ptr(k_norm_w), _ptr(inv_freq), float(eps),
+        T, _ptr(part_acc), _ptr(part_ml), nh, nkv, d, page_size, float(scale), int(window),
+        int(keys_per_split), int(nsplit), _stream())
+    _check(rc, "rope_attention_decode")
+    _note("attention", kernel="decode_mfma_rope", rows=T, dtype=qkv.dtype, nsplit=int(nsplit))
     return out
 
 

@@ -124,6 +124,10 @@ class GroupedQueryAttention(Mixer):
         if pos is not None:
             self.position = lookup("position", pos.kind)(pos.params, {}, runtime)
         self.fused_rotation = bool(getattr(self.position, "fused_rotation", False))
+        # a decode step's norm, rotation and cache write can run inside its attention kernel
+        self.rotation_in_attention = (
+            self.fused_rotation and runtime.dtype == torch.bfloat16
+            and self.position.rotary_dim == self.head_dim and self.position.pairing != "adjacent")
         ops.check_projection_weight(self.w_qkv, "attention w_qkv")
         ops.check_projection_weight(self.w_out, "attention w_out")
 
@@ -132,6 +136,22 @@ class GroupedQueryAttention(Mixer):
         T = x.shape[0]
         qkv = ops.linear(x, self.w_qkv, self.b_qkv)
         slots = step.slot_mapping[cache.group]
+        if self.rotation_in_attention and step.n_tokens == step.n_seqs and cache.writes \
+                and ops.decode_rope_fusable(qkv, nh, nkv, d, d, False, cache.kv.shape[3], self.scale):
+            # single tokens only: the attention kernel prepares queries, key and value itself
+            keys, nsplit = plan_split(step.n_seqs, nkv, step.max_keys)
+            o = ops.rope_attention_decode(qkv, step.positions, slots, self.q_norm, self.k_norm,
+                                          self.position.inv_freq, cache.kv,
+                                          step.block_tables[cache.group], nh, self.eps, self.scale,
+                                          self.window, keys, nsplit)
+            if getattr(step, "taps", None) is not None:
+                # (diagnostics want the queries too: from the kernel the attention replaced)
+                q = ops.qk_norm_rope_kv_write(qkv, step.positions, None, self.q_norm, self.k_norm,
+                                              self.position.inv_freq, None, nh, nkv, d, d, False,
+                                              self.eps, write_kv=False)
+                self._leave_taps(step, cache, q, o)
+            return ops.linear(o.view(T, nh * d), self.w_out, self.b_out, partial_ok=True,
+                              accumulate=stream)
         if self.position is None or self.fused_rotation:
             rot = self.position.rotary_dim if self.position is not None else 0
             q = ops.qk_norm_rope_kv_write(
