@@ -678,16 +678,22 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
   [[maybe_unused]] bf16x8_t knew[KSTEPS];     // ROPE: the token's key, as this lane's fragments
   [[maybe_unused]] bf16_t vnew[DBLK];         // and its value at head-dim elements db * 16 + r16
   [[maybe_unused]] float xq[KSTEPS][8], xk[KSTEPS][8];
+  [[maybe_unused]] float wq[KSTEPS][8], wk[KSTEPS][8];
+  [[maybe_unused]] float freq = 0.f;
   if constexpr (ROPE) {
-    // the raw rows are requested first of all; they are worked on once the position is known
+    // the raw rows, the norms' weights and the frequencies are requested first of all: none
+    // of them waits for anything, and the norm is done by the time the position has arrived
     const bf16_t* row = rope.qkv + (size_t)tok * (nh + 2 * nkv) * D;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       load8<bf16_t>(row + (size_t)head * D + ks * 32 + grp * 8, xq[ks]);
       load8<bf16_t>(row + (size_t)(nh + gkv) * D + ks * 32 + grp * 8, xk[ks]);
+      if (rope.q_norm_w) load8<float>(rope.q_norm_w + ks * 32 + grp * 8, wq[ks]);
+      if (rope.k_norm_w) load8<float>(rope.k_norm_w + ks * 32 + grp * 8, wk[ks]);
     }
 #pragma unroll
     for (int db = 0; db < DBLK; ++db) vnew[db] = row[(size_t)(nh + nkv + gkv) * D + db * 16 + r16];
+    freq = rope.inv_freq[tid & (D / 2 - 1)];
   } else {
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks)
@@ -820,30 +826,28 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
     fetch(tile0, 0, kf, vf);
   }
   if constexpr (ROPE) {
-    if (tid < D / 2) rope_angle(pos_last, rope.inv_freq[tid], &rope_cs[tid], &rope_sn[tid]);
-    __syncthreads();
     // chunk ks * 4 + grp of a head is this lane's x[ks]; the sums of squares meet as in the
     // kernel this replaces: partners half the head apart first, then ever closer ones
-    auto finish = [&](float (&x)[KSTEPS][8], const float* nw, bf16x8_t (&frag)[KSTEPS]) {
-      if (nw) {
-        float ss[KSTEPS];
+    auto normalise = [&](float (&x)[KSTEPS][8], const float (&w)[KSTEPS][8]) {
+      float ss[KSTEPS];
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) ss[ks] = rope_sum_squares8(x[ks]);
+      for (int ks = 0; ks < KSTEPS; ++ks) ss[ks] = rope_sum_squares8(x[ks]);
 #pragma unroll
-        for (int o = KSTEPS / 2; o > 0; o >>= 1)
+      for (int o = KSTEPS / 2; o > 0; o >>= 1)
 #pragma unroll
-          for (int ks = 0; ks < o; ++ks) ss[ks] += ss[ks + o];
-        float t = ss[0];
-        t += __shfl_xor(t, 32, ZA_WAVE);
-        t += __shfl_xor(t, 16, ZA_WAVE);
-        const float norm_scale = rope_rms_scale(t, D, rope.eps);
+        for (int ks = 0; ks < o; ++ks) ss[ks] += ss[ks + o];
+      float t = ss[0];
+      t += __shfl_xor(t, 32, ZA_WAVE);
+      t += __shfl_xor(t, 16, ZA_WAVE);
+      const float norm_scale = rope_rms_scale(t, D, rope.eps);
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-          float w8[8];
-          load8<float>(nw + ks * 32 + grp * 8, w8);
-          rope_scale8(x[ks], norm_scale, w8);
-        }
-      }
+      for (int ks = 0; ks < KSTEPS; ++ks) rope_scale8(x[ks], norm_scale, w[ks]);
+    };
+    if (rope.q_norm_w) normalise(xq, wq);
+    if (rope.k_norm_w) normalise(xk, wk);
+    if (tid < D / 2) rope_angle(pos_last, freq, &rope_cs[tid], &rope_sn[tid]);
+    __syncthreads();
+    auto rotate = [&](float (&x)[KSTEPS][8], bf16x8_t (&frag)[KSTEPS]) {
 #pragma unroll
       for (int ks = 0; ks < KSTEPS / 2; ++ks)
 #pragma unroll
@@ -859,12 +863,12 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
 #pragma unroll
         for (int i = 0; i < 8; ++i) frag[ks][i] = (bf16_t)x[ks][i];
     };
-    finish(xq, rope.q_norm_w, qf);
+    rotate(xq, qf);
     if (!row_valid) {
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) qf[ks] = zero8;
     }
-    finish(xk, rope.k_norm_w, knew);
+    rotate(xk, knew);
   }
   int nth = 0;
   for (; tile0 <= range_hi; tile0 += NWV * AM_KT) {
