@@ -964,6 +964,25 @@ def test_rope_attention_decode_is_the_two_kernels_in_one(nh, nkv, d, page_size, 
     assert not torch.equal(one, cache)            # something was stored
 
 
+def test_rope_attention_decode_stores_the_token_whatever_the_ranges():
+    """Ranges that end before a token's position (a caller's mistake) must not leave its key
+    and value out of the cache: the last range takes the keys that are left."""
+    o = ops()
+    nh, nkv, d, page_size = 8, 2, 64, 16
+    positions = [5, 300, 700]
+    qkv, cache, table, pos, slots = decode_step_case(nh, nkv, d, page_size, positions, 970)
+    inv = (1.0 / torch.pow(torch.tensor(1e4, dtype=torch.float64),
+                           2.0 * torch.arange(0, d // 2, dtype=torch.float64) / d)).float().to(dev())
+    two = cache.clone()
+    q = o.qk_norm_rope_kv_write(qkv, pos, slots, None, None, inv, two, nh, nkv, d, d, False, 1e-5)
+    want = o.paged_attention_decode_mfma(q, two, table, pos, None, None, None, 3, 0.125)
+    one = cache.clone()
+    got = o.rope_attention_decode(qkv, pos, slots, None, None, inv, one, table, nh, 1e-5, 0.125,
+                                  0, 128, 2)                   # two ranges of 128 keys: 256 < 700
+    assert torch.equal(one, two)
+    assert rel_err(got, want.double().cpu()) < 2e-2
+
+
 def test_rope_attention_decode_refuses_what_it_cannot_take():
     o = ops()
     qkv, cache, table, pos, slots = decode_step_case(4, 2, 64, 16, [5, 9], 950)

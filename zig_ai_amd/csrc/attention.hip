@@ -817,6 +817,9 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
   int range_hi = range_lo + keys_per_split - 1;
   if (nsplit == 1) { range_lo = 0; range_hi = hi; }
   if (range_hi > hi) range_hi = hi;
+  // (the token's own key and value are stored by whoever meets its position: ranges that
+  // end before it would leave them out of the cache, so the last range takes what is left)
+  if (ROPE && z == nsplit - 1) range_hi = hi;
   int tile_first = (lo / AM_KT) * AM_KT;
   if (tile_first < range_lo) tile_first = range_lo;
 
