@@ -243,7 +243,7 @@ def main() -> int:
     prefill_flops = 2.0 * T * matmul_params(model) + n_attn * 2.0 * T * T * qdim \
         + 2.0 * vocab * cfg["hidden_size"]
 
-    def prefill_run(portion, reps=3):
+    def prefill_run(portion, reps=8, warm=4):
         runner = ModelRunner(model, page_size=page, num_pages=4 * (T // page + 1), num_slots=4)
 
         def one(name):
@@ -254,7 +254,7 @@ def main() -> int:
                 runner.step([StepEntry(name, toks[lo:hi], [hi - lo - 1] if hi == T else [])])
             runner.release(name)
 
-        for r in range(2):                                  # warm-up
+        for r in range(warm):                               # warm-up
             one(("w", r))
         torch.cuda.synchronize()
         t0 = time.perf_counter()
