@@ -37,3 +37,16 @@ def test_the_kernel_that_runs_the_norm_covers_k_alone():
     assert ops.accumulate_plan(8, 2048, 2048, True) == 1
     assert ops.normed_rows_pay(8, 2048, 2048) and not ops.normed_rows_pay(8, 2048, 4608)
     assert ops.normed_rows_pay(16, 2048, 2048) and not ops.normed_rows_pay(17, 16384, 2048)
+
+
+def test_when_the_output_projection_merges_the_context_ranges():
+    """Few rows in few ranges: every workgroup of the projection merges its slice of every
+    row, which pays while rows x ranges stays small."""
+    from zig_ai_amd.kernels import ops
+    assert ops.merged_rows_pay(1, 8) and ops.merged_rows_pay(3, 8) and ops.merged_rows_pay(8, 2)
+    assert ops.merged_rows_pay(2, 2) and ops.merged_rows_pay(4, 4) and ops.merged_rows_pay(8, 3)
+    assert not ops.merged_rows_pay(8, 4) and not ops.merged_rows_pay(5, 8) and not ops.merged_rows_pay(4, 8)
+    assert ops.merged_rows_pay(1, 12) and ops.merged_rows_pay(2, 12) and not ops.merged_rows_pay(2, 16)
+    assert not ops.merged_rows_pay(3, 12)
+    assert not ops.merged_rows_pay(1, 1) and not ops.merged_rows_pay(1, 17) and not ops.merged_rows_pay(9, 2)
+

@@ -983,6 +983,74 @@ def test_rope_attention_decode_stores_the_token_whatever_the_ranges():
     assert rel_err(got, want.double().cpu()) < 2e-2
 
 
+@pytest.mark.parametrize("nh,nkv,d,H", [(32, 8, 64, 2048), (16, 8, 64, 1024), (8, 2, 128, 512), (24, 8, 64, 1536)])
+@pytest.mark.parametrize("T,keys_per_split,nsplit", [(1, 256, 8), (3, 256, 5), (4, 128, 8), (8, 1024, 2), (7, 512, 3),
+                                                     (1, 128, 12), (2, 128, 16), (3, 128, 11)])
+def test_output_projection_merges_the_context_ranges_itself(nh, nkv, d, H, T, keys_per_split, nsplit):
+    """The decode attention may leave its ranges' partial results unmerged (MergedRows) and
+    the output projection merge them on its way in: the merge has the combine kernel's bits,
+    the product stored has the bits of the product of the merged rows, and added to a stream
+    it agrees to rounding (the additions of the ranges of K arrive in any order)."""
+    o = ops()
+    positions = [1100, 3, 700, 64, 1023, 255, 256, 900][:T]
+    qkv, cache, table, pos, slots = decode_step_case(nh, nkv, d, 16, positions, 980 + T)
+    inv = (1.0 / torch.pow(torch.tensor(1e6, dtype=torch.float64),
+                           2.0 * torch.arange(0, d // 2, dtype=torch.float64) / d)).float().to(dev())
+    scale = 1.0 / math.sqrt(d)
+    want = o.rope_attention_decode(qkv, pos, slots, None, None, inv, cache.clone(), table, nh, 1e-5,
+                                   scale, 0, keys_per_split, nsplit)
+    parts = o.rope_attention_decode(qkv, pos, slots, None, None, inv, cache.clone(), table, nh, 1e-5,
+                                    scale, 0, keys_per_split, nsplit, combine=False)
+    assert isinstance(parts, o.MergedRows) and parts.shape == (T, nh * d) and parts.ranges == nsplit
+    assert torch.equal(parts.materialise().view(T, nh, d), want)
+    w = rand((H, nh * d), torch.bfloat16, 985).to(dev())
+    stored = o.linear(want.view(T, nh * d), w, out_dtype=torch.float32)
+    direct = torch.empty((T, H), dtype=torch.float32, device=dev())
+    rc = o._fn("gemm", "za_gemm_bf16_rows16_merged")(
+        o._ptr(parts.acc), o._ptr(parts.ml), nsplit, d, o._ptr(w), o._ptr(direct), T, H, nh * d, 1, 0,
+        o._stream())
+    assert rc == 0
+    assert torch.equal(direct, stored)
+    base = rand((T, H), torch.float32, 986).to(dev())
+    a, b = base.clone(), base.clone()
+    o.form_log = []
+    try:
+        assert o.linear(parts, w, partial_ok=True, accumulate=a) is None
+        took_the_merge = any(r.get("merged_ranges") for r in o.form_log if r["op"] == "linear")
+    finally:
+        o.form_log = None
+    assert o.linear(want.view(T, nh * d), w, partial_ok=True, accumulate=b) is None
+    assert rel_err(a, b.double().cpu()) < 1e-5
+    assert took_the_merge == o.merged_rows_pay(T, nsplit)     # (every width here is a multiple of 512)
+
+
+def test_merged_rows_fall_back_to_the_combine_kernel():
+    """What the merging product does not take (a bias, a product that is stored, many rows)
+    goes through the combine kernel and the ordinary product."""
+    o = ops()
+    T, nh, d, nsplit = 12, 4, 64, 3
+    acc = rand((T, nh, nsplit, d), torch.float32, 990).to(dev())
+    ml = torch.stack([torch.randint(-3, 4, (T, nh, nsplit)).float(), torch.rand(T, nh, nsplit) + 0.5],
+                     dim=-1).contiguous().to(dev())
+    ml[0, 0, 1, 0] = float("-inf")                  # a range without keys
+    ml[0, 0, 1, 1] = 0.0
+    parts = o.MergedRows(acc, ml)
+    rows = parts.materialise()
+    m, l = ml[..., 0].double().cpu(), ml[..., 1].double().cpu()
+    wgt = torch.exp2(m - m.max(dim=-1, keepdim=True).values)
+    expect = ((acc.double().cpu() * wgt[..., None]).sum(2) / (l * wgt).sum(-1, keepdim=True)).reshape(T, nh * d)
+    assert rel_err(rows, expect) < 1e-2
+    w = rand((96, nh * d), torch.bfloat16, 991).to(dev())
+    bias = rand((96,), torch.float32, 992).to(dev())
+    assert torch.equal(o.linear(parts, w, bias), o.linear(rows, w, bias))
+    stream = torch.zeros((T, 96), device=dev())
+    assert not o.merged_rows_pay(T, nsplit)
+    got = o.linear(parts, w, partial_ok=True, accumulate=stream)       # twelve rows: not merged on the way in
+    expect_y = rows.double().cpu() @ w.double().cpu().T
+    y = stream if got is None else (got.sum(0) if got.dim() == 3 else got)
+    assert rel_err(y, expect_y) < 1e-2
+
+
 def test_rope_attention_decode_refuses_what_it_cannot_take():
     o = ops()
     qkv, cache, table, pos, slots = decode_step_case(4, 2, 64, 16, [5, 9], 950)

@@ -1183,7 +1183,8 @@ static int launch_decode_mfma(const void* q, void* out, const void* kv, const in
                               const int* wi_row0, const int* wi_count, int n_items, int n_tokens,
                               float* part_acc, float* part_ml, int nh, int nkv, int d,
                               int page_size, float scale, int window, int keys_per_split,
-                              int nsplit, const DecodeRope& rope, hipStream_t stream) {
+                              int nsplit, const DecodeRope& rope, bool combine,
+                              hipStream_t stream) {
   dim3 grid(n_items, nkv, nsplit), block(256);
   // Few workgroups (a small batch): eight waves each, so that a compute unit that
   // gets one workgroup still has eight waves' loads in flight.
@@ -1205,10 +1206,22 @@ static int launch_decode_mfma(const void* q, void* out, const void* kv, const in
                        page_size, scale * 1.44269504088896341f, window, keys_per_split, nsplit, rope);
   }
   int rc = za_launch_status();
-  if (rc != 0 || nsplit == 1) return rc;
+  if (rc != 0 || nsplit == 1 || !combine) return rc;
   dim3 cgrid((unsigned)((size_t)n_tokens * nh)), cblock(64);
   hipLaunchKernelGGL((attention_combine_kernel<bf16_t>), cgrid, cblock, 0, stream, part_acc,
                      part_ml, (bf16_t*)out, d, nsplit, 1);
+  return za_launch_status();
+}
+
+// The merge alone: `rows` (token, head) rows of bfloat16 `out` [rows][d] from the partial
+// results of `nsplit` context ranges, maxima on the base-2 scale (the matrix-core kernels').
+extern "C" int za_attention_combine(const float* part_acc, const float* part_ml, void* out,
+                                    int rows, int d, int nsplit, hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || d <= 0 || d > AT_MAX_D || nsplit < 1 || !part_acc || !part_ml || !out)
+    return ZA_ERR_ARG;
+  hipLaunchKernelGGL((attention_combine_kernel<bf16_t>), dim3((unsigned)rows), dim3(64), 0, stream,
+                     part_acc, part_ml, (bf16_t*)out, d, nsplit, 1);
   return za_launch_status();
 }
 
@@ -1239,7 +1252,8 @@ extern "C" int za_paged_attention_decode_mfma(const void* q, void* out, const vo
   const DecodeRope none = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0};
   return launch_decode_mfma<false>(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0,
                                    wi_count, n_items, n_tokens, part_acc, part_ml, nh, nkv, d,
-                                   page_size, scale, window, keys_per_split, nsplit, none, stream);
+                                   page_size, scale, window, keys_per_split, nsplit, none, true,
+                                   stream);
 }
 
 // The same for a step in which every request brings one token, with the token's part of
@@ -1248,16 +1262,20 @@ extern "C" int za_paged_attention_decode_mfma(const void* q, void* out, const vo
 // RMSNorm (weights may be null) and the rotation over the whole head with half pairing
 // (rotary_dim == d, pairs (p, p + d / 2)), key and value go to the cache at `slots`
 // (page * page_size + offset, -1: not stored).  The result and the cache hold the bits that
-// za_qk_norm_rope_kv_write followed by za_paged_attention_decode_mfma leave.
+// za_qk_norm_rope_kv_write followed by za_paged_attention_decode_mfma leave.  With
+// nsplit > 1 and `combine` 0 the partial results stay as they are in part_acc / part_ml
+// (`out` is not written and may be null): whoever reads them merges them
+// (za_attention_combine, or za_gemm_bf16_rows16_merged on its way in).
 extern "C" int za_paged_attention_decode_mfma_rope(
     const void* qkv, void* out, void* kv, const int* block_table, int bt_stride,
     const int* positions, const int* slots, const float* q_norm_w, const float* k_norm_w,
     const float* inv_freq, float eps, int n_tokens, float* part_acc, float* part_ml, int nh,
     int nkv, int d, int page_size, float scale, int window, int keys_per_split, int nsplit,
-    hipStream_t stream) {
+    int combine, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   if (n_tokens < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || page_size <= 0 || bt_stride <= 0 ||
-      nsplit < 1 || !qkv || !out || !kv || !block_table || !positions || !slots || !inv_freq)
+      nsplit < 1 || !qkv || !kv || !block_table || !positions || !slots || !inv_freq ||
+      (!out && (combine || nsplit == 1)))
     return ZA_ERR_ARG;
   const int G = nh / nkv;
   if ((d != 64 && d != 128) || G > 16 || page_size % 4 != 0 || nkv > 65535 || nsplit > 65535)
@@ -1268,5 +1286,6 @@ extern "C" int za_paged_attention_decode_mfma_rope(
                            eps, 1};
   return launch_decode_mfma<true>(nullptr, out, kv, block_table, bt_stride, positions, nullptr,
                                   nullptr, nullptr, n_tokens, n_tokens, part_acc, part_ml, nh, nkv,
-                                  d, page_size, scale, window, keys_per_split, nsplit, rope, stream);
+                                  d, page_size, scale, window, keys_per_split, nsplit, rope,
+                                  combine != 0, stream);
 }

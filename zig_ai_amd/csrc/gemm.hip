@@ -457,12 +457,82 @@ __device__ __forceinline__ void stage_normed_rows(bf16x8_t (&xa)[KSTEPS],
   __syncthreads();
 }
 
-template <int NW, int KSTEPS, typename TC, bool NORM, bool STAGED, bool ROLL>
+// Rows that are an attention's output while it still lies in the partial results of its
+// context ranges (MergedRowsArg): for range z of row (token, head), an accumulator of `d`
+// head-dim elements and (maximum on the base-2 scale, sum).  The product's kernel merges
+// them on the way in, with the arithmetic of attention_combine_kernel in its order (the
+// same bits), and a kernel between the attention and its output projection is saved.
+// K = heads * d; up to 16 ranges, up to 8 rows.
+struct MergedRowsArg {
+  const float* acc;     // [rows][heads][nsplit][d]
+  const float* ml;      // [rows][heads][nsplit][2]
+  int nsplit;
+  int d;
+};
+
+template <int KSTEPS, int Z, typename Prefetch>
+__device__ __forceinline__ void stage_merged_rows(bf16x8_t (&xa)[KSTEPS], const MergedRowsArg& mg,
+                                                  int M, int K, int kslice, bf16_t* mine, int lane,
+                                                  Prefetch&& prefetch) {
+  static_assert(KSTEPS == 16, "one lane takes eight elements of a row's slice of 512");
+  constexpr int RB = 16 / Z;                 // rows whose partial results are in flight at once
+  static_assert(Z == 2 || Z == 4 || Z == 8 || Z == 16, "ranges in flight");
+  const int k = kslice + lane * 8;
+  const int heads = K / mg.d, head = k / mg.d, dim = k % mg.d;
+#pragma unroll
+  for (int rb = 0; rb < ROWS16_STAGE_ROWS; rb += RB) {
+    if (rb > 0 && M <= rb) break;
+    float2 ml[RB][Z];
+    f32x4_t pa[RB][Z][2];
+#pragma unroll
+    for (int r = 0; r < RB; ++r)
+#pragma unroll
+      for (int z = 0; z < Z; ++z)
+        if (rb + r < M && z < mg.nsplit) {
+          const size_t part = ((size_t)(rb + r) * heads + head) * mg.nsplit + z;
+          ml[r][z] = *reinterpret_cast<const float2*>(mg.ml + part * 2);
+          pa[r][z][0] = *reinterpret_cast<const f32x4_t*>(mg.acc + part * mg.d + dim);
+          pa[r][z][1] = *reinterpret_cast<const f32x4_t*>(mg.acc + part * mg.d + dim + 4);
+        }
+    if (rb == 0) {
+      __builtin_amdgcn_sched_barrier(0);
+      prefetch();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int r = 0; r < RB; ++r)
+      if (rb + r < M) {
+        float mx = -INFINITY;
+#pragma unroll
+        for (int z = 0; z < Z; ++z)
+          if (z < mg.nsplit) mx = fmaxf(mx, ml[r][z].x);
+        float total = 0.f, acc[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+#pragma unroll
+        for (int z = 0; z < Z; ++z)
+          if (z < mg.nsplit && ml[r][z].x > -INFINITY) {
+            const float w = ldexpf(1.0f, (int)(ml[r][z].x - mx));
+            total += ml[r][z].y * w;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] = fmaf(pa[r][z][e >> 2][e & 3], w, acc[e]);
+          }
+        const float inv = total > 0.f ? 1.0f / total : 0.f;
+        bf16x8_t v;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = (bf16_t)(acc[e] * inv);
+        *reinterpret_cast<bf16x8_t*>(mine + (rb + r) * ROWS16_STAGE_STRIDE + lane * 8) = v;
+      }
+  }
+  staged_fragments<KSTEPS>(xa, mine, M, lane, 0);
+}
+
+template <int NW, int KSTEPS, typename TC, bool NORM, bool STAGED, bool ROLL, bool MERGED = false>
 __global__ void __launch_bounds__(NW * 64, 2)
 gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
                         const bf16_t* __restrict__ W, const float* __restrict__ bias,
                         TC* __restrict__ C, int M, int N, int K, int groups_per_block,
-                        int accumulate) {
+                        int accumulate, MergedRowsArg merged) {
   __shared__ float red[2][NW][64][4];
   __shared__ float ssw[NW][16];
   const int tid = threadIdx.x;
@@ -498,9 +568,20 @@ gemm_bf16_rows16_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
                                       staged, [&]() { load_first(S0, S2); });
   } else if constexpr (STAGED) {
     if (inside) {
-      stage_rows<KSTEPS>(xa, A, M, K, (blockIdx.y * NW + wave) * KSTEPS * 32,
-                         staged + (size_t)wave * rows16_stage_places(M) * ROWS16_STAGE_STRIDE, lane,
-                         [&]() { load_first(S0, S2); });
+      bf16_t* mine = staged + (size_t)wave * rows16_stage_places(M) * ROWS16_STAGE_STRIDE;
+      const int kslice = (blockIdx.y * NW + wave) * KSTEPS * 32;
+      if constexpr (MERGED) {
+        if (merged.nsplit <= 2)
+          stage_merged_rows<KSTEPS, 2>(xa, merged, M, K, kslice, mine, lane, [&]() { load_first(S0, S2); });
+        else if (merged.nsplit <= 4)
+          stage_merged_rows<KSTEPS, 4>(xa, merged, M, K, kslice, mine, lane, [&]() { load_first(S0, S2); });
+        else if (merged.nsplit <= 8)
+          stage_merged_rows<KSTEPS, 8>(xa, merged, M, K, kslice, mine, lane, [&]() { load_first(S0, S2); });
+        else
+          stage_merged_rows<KSTEPS, 16>(xa, merged, M, K, kslice, mine, lane, [&]() { load_first(S0, S2); });
+      } else {
+        stage_rows<KSTEPS>(xa, A, M, K, kslice, mine, lane, [&]() { load_first(S0, S2); });
+      }
     } else {
 #pragma unroll
       for (int s = 0; s < KSTEPS; ++s) xa[s] = zero8;
@@ -941,12 +1022,18 @@ static bool rows16_takes_norm(int K, int ksplit) {
 
 static int launch_rows16(const bf16_t* a, const NormedRowsArg* normed, const bf16_t* w,
                          const float* bias, void* C, int c_dtype, int M, int N, int K, int ksplit,
-                         int accumulate, hipStream_t stream, int groups_per_block = 0) {
+                         int accumulate, hipStream_t stream, int groups_per_block = 0,
+                         const MergedRowsArg* merged_rows = nullptr) {
   if (ksplit < 1 || (ksplit > 1 && (c_dtype != 0 || K % (ksplit * 32) != 0))) return ZA_ERR_ARG;
   if (accumulate && c_dtype != 0) return ZA_ERR_ARG;
   const bool norm = normed && normed->x;
   if (norm && (!normed->weight || !rows16_takes_norm(K, ksplit))) return ZA_ERR_UNSUPPORTED;
-  if (!norm && !a) return ZA_ERR_ARG;
+  const bool merge = merged_rows && merged_rows->acc;
+  if (merge && (norm || c_dtype != 0 || M > ROWS16_STAGE_ROWS || K % 512 != 0 || merged_rows->nsplit > 16 ||
+                merged_rows->nsplit < 1 || merged_rows->d % 8 != 0 || K % merged_rows->d != 0 ||
+                K / ksplit % 512 != 0 || K / ksplit > 4096))
+    return ZA_ERR_UNSUPPORTED;
+  if (!norm && !a && !merge) return ZA_ERR_ARG;
   const int kper = (K + ksplit - 1) / ksplit;   // K range of one workgroup
   if (kper > 8192) return ZA_ERR_UNSUPPORTED;
   const int groups = (N + 15) / 16;
@@ -963,6 +1050,7 @@ static int launch_rows16(const bf16_t* a, const NormedRowsArg* normed, const bf1
   if (groups_per_block > 0) per_block = groups_per_block;
   dim3 grid((groups + per_block - 1) / per_block, ksplit);
   const NormedRowsArg none = {nullptr, nullptr, nullptr, 0.f};
+  const MergedRowsArg unmerged = {nullptr, nullptr, 0, 0};
   // the rows go through LDS (16 steps a wave only; without the norm: only where K is a
   // multiple of a wave's slice, the condition of the kernel's loads without conditions)
   const bool stage = norm || K % 512 == 0;
@@ -972,7 +1060,15 @@ static int launch_rows16(const bf16_t* a, const NormedRowsArg* normed, const bf1
     auto kernel = gemm_bf16_rows16_kernel<NW, KS, TC, NORM, STAGED, ROLL>;                    \
     if (const int rc = rows16_allow_lds((const void*)kernel, lds)) return rc;                         \
     hipLaunchKernelGGL(kernel, grid, dim3(NW * 64), lds, stream, a, NORM ? *normed : none, w, \
-                       bias, (TC*)C, M, N, K, per_block, accumulate);                         \
+                       bias, (TC*)C, M, N, K, per_block, accumulate, unmerged);               \
+  }
+#define ZA_R16_MERGED(NW, KS, ROLL)                                                           \
+  {                                                                                           \
+    const size_t lds = rows16_stage_bytes(NW, M);                                             \
+    auto kernel = gemm_bf16_rows16_kernel<NW, KS, float, false, true, ROLL, true>;            \
+    if (const int rc = rows16_allow_lds((const void*)kernel, lds)) return rc;                 \
+    hipLaunchKernelGGL(kernel, grid, dim3(NW * 64), lds, stream, a, none, w, bias, (float*)C, \
+                       M, N, K, per_block, accumulate, *merged_rows);                         \
   }
 #define ZA_R16_TYPES(NW, KS, NORM, STAGED, ROLL)                                              \
   {                                                                                           \
@@ -987,6 +1083,10 @@ static int launch_rows16(const bf16_t* a, const NormedRowsArg* normed, const bf1
 #define ZA_R16_CASE(NW, KS)                                                                   \
   {                                                                                           \
     if constexpr (KS == 16) {                                                                 \
+      if (merge) {                                                                            \
+        if (per_block <= 2) ZA_R16_MERGED(NW, KS, true)                                       \
+        else ZA_R16_MERGED(NW, KS, false)                                                     \
+      } else                                                                                  \
       if (norm) ZA_R16_ROLL(NW, KS, true)                                                     \
       else if (stage) ZA_R16_ROLL(NW, KS, false)                                              \
       else ZA_R16_TYPES(NW, KS, false, false, false)                                          \
@@ -1005,6 +1105,7 @@ static int launch_rows16(const bf16_t* a, const NormedRowsArg* normed, const bf1
 #undef ZA_R16_ROLL
 #undef ZA_R16_TYPES
 #undef ZA_R16_LAUNCH
+#undef ZA_R16_MERGED
 }
 
 // ------------------------------------------------------------------ launchers
@@ -1100,6 +1201,22 @@ extern "C" int za_gemm_bf16_rows16_stream(const void* A, const float* x, const i
   const NormedRowsArg normed = {A ? nullptr : x, rows, norm_weight, eps};
   return launch_rows16((const bf16_t*)A, &normed, (const bf16_t*)W, bias, C, c_dtype, M, N, K,
                        ksplit, accumulate ? 1 : 0, stream);
+}
+
+// The decode kernel on rows that are an attention's output still in the partial results of
+// `nsplit` context ranges (part_acc [M][K / d][nsplit][d], part_ml [M][K / d][nsplit][2], as
+// za_paged_attention_decode_mfma leaves them): merged on the way in as
+// attention_combine_kernel would, then multiplied and added to (or stored in) the 32-bit C.
+// M <= 8, nsplit <= 16, K and K / ksplit multiples of 512.
+extern "C" int za_gemm_bf16_rows16_merged(const float* part_acc, const float* part_ml, int nsplit,
+                                          int d, const void* W, void* C, int M, int N, int K,
+                                          int ksplit, int accumulate, hipStream_t stream) {
+  if (M == 0 || N == 0) return 0;
+  if (M < 0 || N < 0 || K <= 0 || !W || !C || !part_acc || !part_ml || d <= 0) return ZA_ERR_ARG;
+  if (!accumulate && ksplit != 1) return ZA_ERR_ARG;
+  const MergedRowsArg merged = {part_acc, part_ml, nsplit, d};
+  return launch_rows16(nullptr, nullptr, (const bf16_t*)W, nullptr, C, 0, M, N, K, ksplit,
+                       accumulate ? 1 : 0, stream, 0, &merged);
 }
 
 // Fused gate|up projection with the SwiGLU gate applied to the accumulators:

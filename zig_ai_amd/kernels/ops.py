@@ -50,7 +50,11 @@ _SIGNATURES = {
     ("attention", "za_paged_attention_decode_mfma_rope"): [
         c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
         c_void_p, c_float, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int,
-        c_int, c_int, c_void_p],
+        c_int, c_int, c_int, c_void_p],
+    ("attention", "za_attention_combine"): [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                            c_void_p],
+    ("gemm", "za_gemm_bf16_rows16_merged"): [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p,
+                                             c_int, c_int, c_int, c_int, c_int, c_void_p],
     ("shortconv", "za_short_conv"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                      c_longlong, c_void_p],
@@ -271,6 +275,52 @@ def normed_rows_pay(M: int, N: int, K: int) -> bool:
     return normed_rows_fusable(M, K)
 
 
+class MergedRows:
+    """An attention's output ``[T, heads * head_dim]`` while it still lies in the partial
+    results of its context ranges (``acc [T, heads, ranges, head_dim]``, ``ml [T, heads,
+    ranges, 2]``: accumulator, maximum on the base-2 scale and sum).  ``linear`` merges them
+    on the product's way in where that pays (a kernel less); ``materialise`` runs the merge
+    as a kernel of its own.  The same bits either way."""
+
+    def __init__(self, acc: torch.Tensor, ml: torch.Tensor):
+        _need(acc, "acc", torch.float32)
+        T, nh, nsplit, d = acc.shape
+        _need(ml, "ml", torch.float32, (T, nh, nsplit, 2))
+        self.acc, self.ml = acc, ml
+        self.rows, self.heads, self.ranges, self.head_dim = T, nh, nsplit, d
+        self.shape = (T, nh * d)
+        self.dtype = torch.bfloat16
+
+    @property
+    def device(self) -> torch.device:
+        return self.acc.device
+
+    def materialise(self) -> torch.Tensor:
+        out = torch.empty(self.shape, dtype=torch.bfloat16, device=self.acc.device)
+        rc = _fn("attention", "za_attention_combine")(
+            _ptr(self.acc), _ptr(self.ml), _ptr(out), self.rows * self.heads, self.head_dim,
+            self.ranges, _stream())
+        _check(rc, "attention_combine")
+        _note("attention_combine", rows=self.rows, ranges=self.ranges)
+        return out
+
+
+MERGED_ROWS_MAX_ROWS = 8
+MERGED_ROWS_MAX_RANGES = 16
+
+
+def merged_rows_pay(rows: int, ranges: int) -> bool:
+    """Whether the output projection should merge the ranges itself.  Measured against the
+    combine kernel followed by the projection, hidden 2048 (1024): one row in 8 ranges 4.6
+    (3.4) against 8.0 (6.7) us, four rows in 8 ranges 6.7 (5.3) against 8.1 (6.7), eight rows
+    in 2 ranges 5.5 (4.6) against 6.8 (5.3), eight rows in 4 ranges 7.1 (5.9) against 7.3
+    (5.8): every workgroup of the projection merges its slice of every row.  In a decode step
+    of the 1.2B shape: batch 1 (12 ranges) 0.731 -> 0.704 ms, batch 2 0.735 -> 0.716, batch 4
+    (8 ranges) 0.750 -> 0.762: up to 24 rows x ranges."""
+    return (1 < ranges <= MERGED_ROWS_MAX_RANGES and 0 < rows <= MERGED_ROWS_MAX_ROWS
+            and rows * ranges <= 24)
+
+
 # --------------------------------------------------------------------- gemm
 # Above this many rows a bfloat16 projection without bias goes to the library
 # (measured: the decode kernel wins up to 16 rows, the library from there on).
@@ -389,6 +439,16 @@ def _accumulate_splits(N: int, K: int) -> int:
     return 0
 
 
+def _merged_splits(N: int, K: int) -> int:
+    """The same for rows that are merged on the way in: a workgroup's range of K is then a
+    multiple of a wave's 512 and at most 4096.  0: no such cut."""
+    groups = (N + 15) // 16
+    for split in (8, 4, 3, 2, 1):
+        if K % (split * 512) == 0 and K // split <= 4096 and (groups * split <= 640 or split == 1):
+            return split
+    return 0
+
+
 def accumulate_plan(M: int, N: int, K: int, normed: bool) -> int:
     """How a decode batch's product reaches the stream: the number of ranges of K whose
     partial products are added there with atomics, or 0 when the kernel that adds takes
@@ -427,6 +487,23 @@ def linear(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
                           f"{tuple(weight.shape)}")
     M, K = x.shape
     N = weight.shape[0]
+    if isinstance(x, MergedRows):
+        splits = 0
+        if accumulate is not None and bias is None and weight.dtype == torch.bfloat16 \
+                and not force_tiled and merged_rows_pay(M, x.ranges):
+            splits = _merged_splits(N, K)
+        if not splits:
+            x = x.materialise()
+        else:
+            _need(weight, "weight", torch.bfloat16, (N, K))
+            _need(accumulate, "accumulate", torch.float32, (M, N))
+            rc = _fn("gemm", "za_gemm_bf16_rows16_merged")(
+                _ptr(x.acc), _ptr(x.ml), x.ranges, x.head_dim, _ptr(weight), _ptr(accumulate),
+                M, N, K, splits, 1, _stream())
+            _check(rc, "gemm_bf16_rows16_merged", f"M={M} N={N} K={K} splits={splits}")
+            _note("linear", M=M, N=N, K=K, norm_in_product=False, added_to_stream=True,
+                  partial_sums=1, out=accumulate.dtype, merged_ranges=x.ranges)
+            return None
     normed = None
     if isinstance(x, NormedRows):
         if _takes_normed_rows(x, weight, M, K) and not force_tiled:
@@ -796,13 +873,14 @@ def rope_attention_decode(qkv: torch.Tensor, positions: torch.Tensor, slots: tor
                           inv_freq: torch.Tensor, kv_cache: torch.Tensor,
                           block_table: torch.Tensor, num_heads: int, eps: float, scale: float,
                           window: int = 0, keys_per_split: int = 0,
-                          nsplit: int = 1) -> torch.Tensor:
+                          nsplit: int = 1, combine: bool = True):
     """A step in which request ``i`` brings the one token of row ``i``: what
     ``qk_norm_rope_kv_write`` followed by ``paged_attention_decode_mfma`` does, in the
     attention's kernel (its prologue normalises and rotates the token's queries and key;
     the workgroup that meets the token's own position stores key and value to the cache).
     The same bits in the result and in the cache, one kernel and one trip through memory
-    less.  Returns the attention's output ``[T, heads, head_dim]``."""
+    less.  Returns the attention's output ``[T, heads, head_dim]``, or, with ``nsplit`` > 1 and
+    ``combine=False``, the ranges' partial results unmerged as ``MergedRows``."""
     if kv_cache.dim() != 5 or kv_cache.shape[1] != 2:
         raise KernelError(f"kv_cache has shape {tuple(kv_cache.shape)}, expected "
                           f"[pages, 2, kv_heads, page_size, head_dim]")
@@ -823,7 +901,8 @@ def rope_attention_decode(qkv: torch.Tensor, positions: torch.Tensor, slots: tor
     for name, w in (("q_norm_w", q_norm_w), ("k_norm_w", k_norm_w)):
         if w is not None:
             _need(w, name, torch.float32, (d,))
-    out = torch.empty((T, nh, d), dtype=torch.bfloat16, device=qkv.device)
+    unmerged = nsplit > 1 and not combine
+    out = None if unmerged else torch.empty((T, nh, d), dtype=torch.bfloat16, device=qkv.device)
     part_acc = part_ml = None
     if nsplit > 1:
         if keys_per_split <= 0 or keys_per_split % 64:
@@ -834,10 +913,11 @@ def rope_attention_decode(qkv: torch.Tensor, positions: torch.Tensor, slots: tor
         _ptr(qkv), _ptr(out), _ptr(kv_cache), _ptr(block_table), block_table.shape[1],
         _ptr(positions), _ptr(slots), _ptr(q_norm_w), _ptr(k_norm_w), _ptr(inv_freq), float(eps),
         T, _ptr(part_acc), _ptr(part_ml), nh, nkv, d, page_size, float(scale), int(window),
-        int(keys_per_split), int(nsplit), _stream())
+        int(keys_per_split), int(nsplit), 0 if unmerged else 1, _stream())
     _check(rc, "rope_attention_decode")
-    _note("attention", kernel="decode_mfma_rope", rows=T, dtype=qkv.dtype, nsplit=int(nsplit))
-    return out
+    _note("attention", kernel="decode_mfma_rope", rows=T, dtype=qkv.dtype, nsplit=int(nsplit),
+          combine_kernel=nsplit > 1 and not unmerged)
+    return MergedRows(part_acc, part_ml) if unmerged else out
 
 
 # ---------------------------------------------------------------- short conv

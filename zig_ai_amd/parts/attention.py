@@ -140,18 +140,22 @@ class GroupedQueryAttention(Mixer):
                 and ops.decode_rope_fusable(qkv, nh, nkv, d, d, False, cache.kv.shape[3], self.scale):
             # single tokens only: the attention kernel prepares queries, key and value itself
             keys, nsplit = plan_split(step.n_seqs, nkv, step.max_keys)
+            # few rows in few ranges: the output projection merges the ranges on its way in
+            unmerged = stream is not None and self.b_out is None and ops.merged_rows_pay(T, nsplit)
             o = ops.rope_attention_decode(qkv, step.positions, slots, self.q_norm, self.k_norm,
                                           self.position.inv_freq, cache.kv,
                                           step.block_tables[cache.group], nh, self.eps, self.scale,
-                                          self.window, keys, nsplit)
+                                          self.window, keys, nsplit, combine=not unmerged)
             if getattr(step, "taps", None) is not None:
                 # (diagnostics want the queries too: from the kernel the attention replaced)
                 q = ops.qk_norm_rope_kv_write(qkv, step.positions, None, self.q_norm, self.k_norm,
                                               self.position.inv_freq, None, nh, nkv, d, d, False,
                                               self.eps, write_kv=False)
-                self._leave_taps(step, cache, q, o)
-            return ops.linear(o.view(T, nh * d), self.w_out, self.b_out, partial_ok=True,
-                              accumulate=stream)
+                merged = o.materialise() if isinstance(o, ops.MergedRows) else o
+                self._leave_taps(step, cache, q, merged.view(T, nh, d))
+            if not isinstance(o, ops.MergedRows):
+                o = o.view(T, nh * d)
+            return ops.linear(o, self.w_out, self.b_out, partial_ok=True, accumulate=stream)
         if self.position is None or self.fused_rotation:
             rot = self.position.rotary_dim if self.position is not None else 0
             q = ops.qk_norm_rope_kv_write(
