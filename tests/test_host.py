@@ -182,3 +182,7 @@ def test_context_split_plan():
     keys, nsplit = plan_split(1, 8, 131072)               # one long request: ~SPLIT_TARGET groups
     assert (keys, nsplit) == (4096, 32) and 8 * nsplit >= SPLIT_TARGET
     assert plan_split(16, 8, 4608) == (2304, 2)           # ranges of the same length
+    assert plan_split(12, 8, 3072) == (1536, 2)           # never more workgroups than SPLIT_TARGET
+    assert plan_split(20, 8, 8192) == (0, 1) and plan_split(7, 8, 3072)[1] == 4
+    assert plan_split(1, 8, 1024) == (256, 4)             # short contexts are cut finer
+    assert plan_split(1, 8, 3072) == (512, 6) and plan_split(1, 8, 512) == (0, 1)

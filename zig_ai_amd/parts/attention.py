@@ -29,8 +29,8 @@ from .feed_forward import fuse_rows
 # machine idle (decoding few requests, or a portion of a prompt far into a long
 # request).  Measured on one MI355X with 8 key/value heads, contexts from 2,048 to
 # 131,072 keys and 1 to 64 requests: from 512 workgroups on nothing is gained; below,
-# as few ranges as still yield SPLIT_TARGET workgroups are best or within a few
-# percent of it (fewer partial results to merge), all of the same length.
+# as many ranges as still stay within SPLIT_TARGET workgroups (one decode workgroup of
+# eight waves a compute unit) are best or within a few percent of it, all of the same length.
 BUSY_WORKGROUPS = 512
 SPLIT_TARGET = 256
 SPLIT_KEYS_MIN = 512
@@ -48,7 +48,10 @@ def plan_split(n_items: int, num_kv_heads: int, max_keys: int, target: int = SPL
     keys_min = SPLIT_KEYS_MIN if max_keys > 4 * SPLIT_KEYS_MIN else SPLIT_KEYS_MIN // 2
     if groups >= BUSY_WORKGROUPS or max_keys <= 2 * keys_min:
         return 0, 1
-    wanted = (target + groups - 1) // groups                # ranges that fill the machine
+    # as many ranges as keep the launch within `target` workgroups (one more range would send
+    # part of them into a second round: 12 requests at 2,048 keys, 2 ranges 0.862 ms a step, 3
+    # ranges 0.878; 20 requests uncut 1.18, in 2 ranges 1.27)
+    wanted = target // groups
     nsplit = min(wanted, max_keys // keys_min, SPLIT_MAX)
     if nsplit <= 1:
         return 0, 1
