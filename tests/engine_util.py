@@ -158,6 +158,8 @@ class Forms:
         for r in log:
             if r["op"] == "attention":
                 self.kernels.add(r["kernel"])
+            if r["op"] == "linear" and r.get("merged_ranges"):
+                self.kernels.add("output projection that merges the ranges")
         if products:
             L = self.n_layers
             assert len(products) == 4 * L + (1 if wanted_rows else 0), \

@@ -430,6 +430,8 @@ def test_real_layer_sizes_every_way_of_cutting(kind, dtype):
     if dtype == "bfloat16":
         kernels = forms.kernels
         assert "mfma" in kernels and ("decode_mfma_rope" in kernels or kind in ("whole", "far portion"))
+        if kind == "bulk":        # single tokens of one request, its context cut into ranges
+            assert "output projection that merges the ranges" in kernels
 
 
 def test_reproducible_decoding_at_real_layer_sizes():
