@@ -12,11 +12,16 @@ greedy sampler, issued as generation issues them (the tokens of a step reach the
 next one on the device; the host reads them every 8 steps).  Prints ONE JSON line: decoded tokens per second as ``value``,
 a 2,048-token prefill under ``prefill``, the decode step against the HBM
 roofline under ``roofline``, and batch 1 / batch 64 decoding under ``points`` (tokens per
-second) with their step times, bytes and fractions under ``points_detail``.  Further keys:
+second) with their step times, bytes and fractions under ``points_detail``, where batch 8
+at contexts of 4,096 and 8,192 tokens and batch 64 at 4,096 stand too.  Further keys:
 ``prefill_chunked_512`` (the same 2,048 tokens in four steps of 512, the reference's
-``-ub 512``, /root/reference/src/main.zig:57-61), and ``calibration``: what this GPU
-does at best, measured here (a kernel that only reads 1 GiB; matrix-core instructions
-issued back to back), with every fraction also given against those (``frac_measured``).
+``-ub 512``, /root/reference/src/main.zig:57-61), ``shapes`` (batch 8 decoding and the
+2,048-token prefill of the LFM2-350M and LFM2-2.6B layer sizes, the latter at its context
+of 8,192), and ``calibration``: what this GPU does at best, measured here (a kernel that
+only reads 1 GiB; matrix-core instructions issued back to back), with every fraction also
+given against those (``frac_measured``).  ``--phase prefill|decode`` runs that phase alone
+for a profiler: no calibration kernels, and the GEMM library's first answer for every
+shape (no timing of candidates, which allocates, frees and waits inside the first steps).
 The model is ``DecoderModel.from_random(cfg, seed=0)``: the tensors that
 ``write_random_model(cfg, folder, seed=0)`` stores, drawn on the device.
 """
@@ -66,7 +71,7 @@ SHAPES = {
 }
 
 
-def serve(cfg, name, n_requests, new_tokens, portion_graphs=False) -> int:
+def serve(cfg, name, n_requests, new_tokens, portion_graphs=False, chunk_size=None) -> int:
     """Requests with prompts of 128 to 2,048 tokens through the scheduler, the step
     function and the sampler (temperature 0.7), all admitted at once."""
     import random
@@ -82,9 +87,10 @@ def serve(cfg, name, n_requests, new_tokens, portion_graphs=False) -> int:
                for _ in range(n_requests)]
     with tempfile.TemporaryDirectory(prefix="zigai_bench_") as folder:
         write_random_model(config_from_dict(cfg), folder, seed=0, dtype=torch.bfloat16)
+        more = {} if chunk_size is None else {"chunk_size": chunk_size}   # (else the engine's default)
         engine = Engine(folder, dtype="bfloat16", page_size=16, max_num_seqs=64,
-                        max_num_batched_tokens=4096, chunk_size=2048, max_model_len=4096,
-                        portion_graphs=portion_graphs)
+                        max_num_batched_tokens=4096, max_model_len=4096,
+                        portion_graphs=portion_graphs, **more)
         # warm-up: every kind of step once (more than 16 rows of logits among them),
         # so that no library loads its kernels inside the timed run
         engine.generate([p[:64] for p in prompts[:20]], max_new_tokens=4, temperature=0.7, seed=3,
@@ -105,6 +111,7 @@ def serve(cfg, name, n_requests, new_tokens, portion_graphs=False) -> int:
         "prompt_tokens": prompt_tokens, "generated_tokens": generated, "seconds": dt,
         "generated_per_s": generated / dt, "tokens_per_s": (prompt_tokens + generated) / dt,
         "steps": stats["steps"], "preemptions": stats["preemptions"], "dtype": "bf16",
+        "chunk_size": engine.scheduler.chunk_size,
         "data": "synthetic token ids; random weights N(0, 0.02)"}), flush=True)
     return 0
 
@@ -160,6 +167,9 @@ def main() -> int:
     ap.add_argument("--new-tokens", type=int, default=256, help="new tokens per request of "
                     "--workload serve")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points")
+    ap.add_argument("--chunk-size", type=int, default=None,
+                    help="--workload serve: the longest portion of a prompt in one step "
+                         "(default: the engine's own)")
     ap.add_argument("--portion-graphs", action="store_true",
                     help="--workload serve: also record steps with prompt portions")
     ap.add_argument("--phase", choices=["all", "prefill", "decode"], default="all",
@@ -177,133 +187,178 @@ def main() -> int:
     torch.cuda.set_device(0)
     cfg = dict(SHAPES[args.shape])
     if args.workload == "serve":
-        return serve(cfg, args.shape.upper(), args.requests, args.new_tokens, args.portion_graphs)
+        return serve(cfg, args.shape.upper(), args.requests, args.new_tokens, args.portion_graphs,
+                     args.chunk_size)
     full_layers = cfg["num_hidden_layers"]
     if args.layers is not None and args.layers < full_layers:
         cfg["num_hidden_layers"] = args.layers
         cfg["layer_types"] = cfg["layer_types"][:args.layers]
-    model = DecoderModel.from_random(cfg, seed=0, dtype="bfloat16")
-    vocab = cfg["vocab_size"]
     page = 16
     gen = torch.Generator().manual_seed(1234)
+    profiled = args.phase != "all"
 
-    def tokens(n):
+    def tokens(n, vocab):
         return torch.randint(0, vocab, (n,), generator=gen).tolist()
 
-    def decode_run(batch, prompt_len, steps, warmup):
-        """Prefill ``batch`` requests, then time ``steps`` decode steps."""
-        need = batch * ((prompt_len + steps + warmup + 2 + page - 1) // page + 1)
-        runner = ModelRunner(model, page_size=page, num_pages=need, num_slots=batch)
-        last = []
-        for r in range(batch):
-            runner.admit(r)
-            logits = runner.step([StepEntry(r, tokens(prompt_len), [prompt_len - 1])])
-            last.append(int(ops.argmax(logits)[0]))
+    class Measured:
+        """One shape's model with what is measured on it."""
 
-        requests = list(range(batch))
+        def __init__(self, cfg):
+            self.cfg = cfg
+            # (a profiled phase takes the library's first answer for every shape)
+            self.model = DecoderModel.from_random(cfg, seed=0, dtype="bfloat16",
+                                                  library_tuning=False if profiled else None)
+            self.vocab = cfg["vocab_size"]
+            self.n_attn = sum(1 for k in cfg["layer_types"] if k != "conv")
+            self.hd = cfg["hidden_size"] // cfg["num_attention_heads"]
+            self.kv_bytes_per_token = self.n_attn * 2 * cfg["num_key_value_heads"] * self.hd * 2
+            self.weight_bytes = count_bytes(self.model)
 
-        def run(cur, n):
-            """``n`` decode steps the way generation issues them: greedy tokens handed
-            from step to step on the device, the host reading them every 8 steps."""
-            done = 0
-            while done < n:
-                k = min(8, n - done)
-                drawn = runner.decode_steps(requests, cur, k, lambda logits, i: ops.argmax(logits))
-                cur = drawn[-1].tolist()
-                done += drawn.shape[0]
-            return cur
+        def decode_run(self, batch, prompt_len, steps, warmup):
+            """Prefill ``batch`` requests, then time ``steps`` decode steps.  Returns the
+            seconds and the mean context length over the timed steps."""
+            model, vocab = self.model, self.vocab
+            need = batch * ((prompt_len + steps + warmup + 2 + page - 1) // page + 1)
+            runner = ModelRunner(model, page_size=page, num_pages=need, num_slots=batch)
+            last = []
+            for r in range(batch):
+                runner.admit(r)
+                toks = tokens(prompt_len, vocab)
+                for lo in range(0, prompt_len, 2048):            # prompts in steps of 2,048
+                    hi = min(prompt_len, lo + 2048)
+                    logits = runner.step([StepEntry(r, toks[lo:hi],
+                                                    [hi - lo - 1] if hi == prompt_len else [])])
+                last.append(int(ops.argmax(logits)[0]))
+            requests = list(range(batch))
 
-        last = run(last, warmup)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        last = run(last, steps)
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-        ctx_mid = prompt_len + warmup + steps / 2.0
-        for r in range(batch):
-            runner.release(r)
-        del runner
-        torch.cuda.empty_cache()
-        return dt, ctx_mid
+            def run(cur, n):
+                """``n`` decode steps the way generation issues them: greedy tokens handed
+                from step to step on the device, the host reading them every 8 steps."""
+                done = 0
+                while done < n:
+                    k = min(8, n - done)
+                    drawn = runner.decode_steps(requests, cur, k, lambda logits, i: ops.argmax(logits))
+                    cur = drawn[-1].tolist()
+                    done += drawn.shape[0]
+                return cur
+
+            last = run(last, warmup)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            last = run(last, steps)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            ctx_mid = prompt_len + warmup + steps / 2.0
+            for r in range(batch):
+                runner.release(r)
+            del runner
+            torch.cuda.empty_cache()
+            return dt, ctx_mid
+
+        def prefill_flops(self, T):
+            cfg = self.cfg
+            qdim = cfg["num_attention_heads"] * self.hd
+            return 2.0 * T * matmul_params(self.model) + self.n_attn * 2.0 * T * T * qdim \
+                + 2.0 * self.vocab * cfg["hidden_size"]
+
+        def prefill_run(self, T, portion, calibration, reps=8, warm=4):
+            model, vocab = self.model, self.vocab
+            runner = ModelRunner(model, page_size=page, num_pages=4 * (T // page + 1), num_slots=4)
+
+            def one(name):
+                runner.admit(name)
+                toks = tokens(T, vocab)
+                for lo in range(0, T, portion):
+                    hi = min(T, lo + portion)
+                    runner.step([StepEntry(name, toks[lo:hi], [hi - lo - 1] if hi == T else [])])
+                runner.release(name)
+
+            for r in range(warm):                               # warm-up
+                one(("w", r))
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for r in range(reps):
+                one(("p", r))
+            torch.cuda.synchronize()
+            seconds = (time.perf_counter() - t0) / reps
+            del runner
+            torch.cuda.empty_cache()
+            rate = self.prefill_flops(T) / seconds
+            out = {"value": T / seconds, "tokens": T, "ms": seconds * 1e3,
+                   "frac": rate / PEAK_FLOPS["bf16"]}
+            if calibration:
+                out["frac_measured"] = rate / (calibration["mfma_bf16_TFLOPs"] * 1e12)
+            return out
+
+        def against_memory(self, batch, seconds_per_step, ctx, calibration):
+            """A decode step against the memory it has to read: every weight once and the
+            cache of the live requests."""
+            step_bytes = self.weight_bytes + batch * self.kv_bytes_per_token * ctx
+            rate = step_bytes / seconds_per_step
+            out = {"ms_per_step": seconds_per_step * 1e3, "ctx": ctx, "bytes": step_bytes,
+                   "achieved_GBps": rate / 1e9, "frac": rate / HBM_BYTES_PER_S}
+            if calibration:
+                out["frac_measured"] = rate / (calibration["read_GBps"] * 1e9)
+            return out
+
+    T = 2048
+    main_shape = Measured(cfg)
+    ffn_width = main_shape.model.config.intermediate_size
+    # ---- one phase alone, for a profiler: nothing else runs
+    if args.phase == "decode":
+        dt, ctx_mid = main_shape.decode_run(args.batch, args.prompt_len, args.steps, args.warmup)
+        print(json.dumps({"phase": "decode", "batch": args.batch, "steps": args.steps,
+                          "ms_per_step": dt / args.steps * 1e3,
+                          "value": args.batch * args.steps / dt, "unit": "tokens/s"}), flush=True)
+        return 0
+    if args.phase == "prefill":
+        print(json.dumps({"phase": "prefill", **main_shape.prefill_run(T, T, None)}), flush=True)
+        return 0
 
     # ---- what this GPU does at best
     calibration = {"read_GBps": ops.measured_read_bandwidth() / 1e9,
                    "mfma_bf16_TFLOPs": ops.measured_mfma_rate() / 1e12}
 
     # ---- prefill of 2,048 tokens, one request: in one step, and in four steps of 512
-    T = 2048
-    if args.phase == "decode":
-        dt, ctx_mid = decode_run(args.batch, args.prompt_len, args.steps, args.warmup)
-        print(json.dumps({"phase": "decode", "batch": args.batch, "steps": args.steps,
-                          "ms_per_step": dt / args.steps * 1e3,
-                          "value": args.batch * args.steps / dt, "unit": "tokens/s"}), flush=True)
-        return 0
-    n_attn = sum(1 for k in cfg["layer_types"] if k != "conv")
-    qdim = cfg["num_attention_heads"] * (cfg["hidden_size"] // cfg["num_attention_heads"])
-    prefill_flops = 2.0 * T * matmul_params(model) + n_attn * 2.0 * T * T * qdim \
-        + 2.0 * vocab * cfg["hidden_size"]
-
-    def prefill_run(portion, reps=8, warm=4):
-        runner = ModelRunner(model, page_size=page, num_pages=4 * (T // page + 1), num_slots=4)
-
-        def one(name):
-            runner.admit(name)
-            toks = tokens(T)
-            for lo in range(0, T, portion):
-                hi = min(T, lo + portion)
-                runner.step([StepEntry(name, toks[lo:hi], [hi - lo - 1] if hi == T else [])])
-            runner.release(name)
-
-        for r in range(warm):                               # warm-up
-            one(("w", r))
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for r in range(reps):
-            one(("p", r))
-        torch.cuda.synchronize()
-        seconds = (time.perf_counter() - t0) / reps
-        del runner
-        torch.cuda.empty_cache()
-        rate = prefill_flops / seconds
-        return {"value": T / seconds, "tokens": T, "ms": seconds * 1e3,
-                "frac": rate / PEAK_FLOPS["bf16"],
-                "frac_measured": rate / (calibration["mfma_bf16_TFLOPs"] * 1e12)}
-
-    prefill = prefill_run(T)
-    if args.phase == "prefill":
-        print(json.dumps({"phase": "prefill", **prefill}), flush=True)
-        return 0
-    prefill_chunked = prefill_run(512)
+    prefill = main_shape.prefill_run(T, T, calibration)
+    prefill_chunked = main_shape.prefill_run(T, 512, calibration)
 
     # ---- the headline: batch 8 decoding from a 2,048-token context
-    hd = cfg["hidden_size"] // cfg["num_attention_heads"]
-    kv_bytes_per_token = n_attn * 2 * cfg["num_key_value_heads"] * hd * 2
-    weight_bytes = count_bytes(model)
-
-    def against_memory(batch, seconds_per_step, ctx):
-        """A decode step against the memory it has to read: every weight once and the
-        cache of the live requests."""
-        step_bytes = weight_bytes + batch * kv_bytes_per_token * ctx
-        rate = step_bytes / seconds_per_step
-        return {"ms_per_step": seconds_per_step * 1e3, "bytes": step_bytes,
-                "achieved_GBps": rate / 1e9, "frac": rate / HBM_BYTES_PER_S,
-                "frac_measured": rate / (calibration["read_GBps"] * 1e9)}
-
-    dt, ctx_mid = decode_run(args.batch, args.prompt_len, args.steps, args.warmup)
+    dt, ctx_mid = main_shape.decode_run(args.batch, args.prompt_len, args.steps, args.warmup)
     ms_per_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
-    headline = against_memory(args.batch, dt / args.steps, ctx_mid)
+    headline = main_shape.against_memory(args.batch, dt / args.steps, ctx_mid, calibration)
     roofline = {"bound": "hbm", "achieved": headline["achieved_GBps"], "peak": HBM_BYTES_PER_S / 1e9,
                 "unit": "GB/s", "frac": headline["frac"], "frac_measured": headline["frac_measured"]}
 
-    points, points_detail = {}, {}
+    points, points_detail, shapes = {}, {}, {}
     if not args.no_points:
         for b in (1, 64):
             steps = max(16, args.steps // 2)
-            d, ctx = decode_run(b, args.prompt_len, steps, 4)
+            d, ctx = main_shape.decode_run(b, args.prompt_len, steps, 4)
             points[f"decode_b{b}"] = b * steps / d
-            points_detail[f"decode_b{b}"] = against_memory(b, d / steps, ctx)
+            points_detail[f"decode_b{b}"] = main_shape.against_memory(b, d / steps, ctx, calibration)
+        # further contexts (prefilled to there, 16 steps each)
+        for b, ctx0 in ((8, 4096), (8, 8192), (64, 4096)):
+            d, ctx = main_shape.decode_run(b, ctx0, 16, 4)
+            points_detail[f"decode_b{b}_ctx{ctx0}"] = main_shape.against_memory(b, d / 16, ctx, calibration)
+        # the other shapes: batch 8 decoding and a 2,048-token prefill each
+        if args.shape == "1.2b" and args.layers is None:
+            del main_shape.model
+            torch.cuda.empty_cache()
+            for name, ctx0 in (("350m", 2048), ("2.6b", 8192)):
+                other = Measured(dict(SHAPES[name]))
+                d, ctx = other.decode_run(8, ctx0, 16, 4)
+                detail = other.against_memory(8, d / 16, ctx, calibration)
+                detail.update(value=8 * 16 / d, unit="tokens/s", batch=8,
+                              layers=other.cfg["num_hidden_layers"],
+                              weights_GB=other.weight_bytes / 1e9,
+                              prefill=other.prefill_run(T, T, calibration, reps=4, warm=2))
+                shapes[name] = detail
+                del other
+                torch.cuda.empty_cache()
 
+    vocab, hd, n_attn = cfg["vocab_size"], main_shape.hd, main_shape.n_attn
     line = {
         "metric": f"decode tok/s @ batch {args.batch} (LFM2-{args.shape.upper()} shape, context "
                   f"{args.prompt_len} prompt + decode)",
@@ -313,19 +368,20 @@ def main() -> int:
         "data": "synthetic token ids uniform over the vocabulary; random weights N(0, 0.02)",
         "config": {
             "model": f"LFM2-{args.shape.upper()} shape", "global_batch": args.batch,
-            "seq_len": args.prompt_len + 2048,
+            # the context the timed steps really reach
+            "seq_len": args.prompt_len + args.warmup + args.steps,
             "prompt_len": args.prompt_len, "parallelism": "single GPU",
             "layers": cfg["num_hidden_layers"], "layers_of_config": full_layers,
             "attention_layers": n_attn, "hidden_size": cfg["hidden_size"],
             "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
-            "head_dim": hd, "ffn_width": model.config.intermediate_size, "vocab": vocab,
+            "head_dim": hd, "ffn_width": ffn_width, "vocab": vocab,
             "conv_L_cache": cfg["conv_L_cache"], "rope_theta": cfg["rope_theta"],
             "norm_eps": cfg["norm_eps"], "tied_embeddings": cfg["tie_embedding"],
-            "page_size": page, "weights_GB": count_bytes(model) / 1e9,
+            "page_size": page, "weights_GB": main_shape.weight_bytes / 1e9,
         },
         "prefill": prefill, "roofline": roofline, "points": points,
         "points_detail": points_detail, "prefill_chunked_512": prefill_chunked,
-        "calibration": calibration,
+        "shapes": shapes, "calibration": calibration,
     }
     print(json.dumps(line), flush=True)
     return 0

@@ -142,6 +142,7 @@ class Forms:
         self.lengths = list(lengths)
         self.by_shape = {}
         self.kernels = set()
+        self.seen = set()        # further forms a test may ask about (see note_step)
         self._torch = _torch
 
     def _mask(self, i, key):
@@ -160,6 +161,13 @@ class Forms:
                 self.kernels.add(r["kernel"])
             if r["op"] == "linear" and r.get("merged_ranges"):
                 self.kernels.add("output projection that merges the ranges")
+            if r["op"] == "attention_combine" or (r["op"] == "attention" and r.get("combine_kernel")):
+                self.seen.add("ranges merged by the combine kernel")
+            if r["op"] == "attention" and r["kernel"].startswith("decode_mfma") and r["rows"] > 16 \
+                    and r["nsplit"] == 1:
+                self.seen.add("decode attention of many rows, contexts uncut")
+            if r["op"] == "linear" and r["M"] > 16 and r["partial_sums"] > 1:
+                self.seen.add("library product with ranges of K")
         if products:
             L = self.n_layers
             assert len(products) == 4 * L + (1 if wanted_rows else 0), \

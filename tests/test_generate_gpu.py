@@ -12,7 +12,7 @@ import torch
 
 import engine_util as eu
 import plain_lfm2 as plain
-from tiny_configs import TINY_A, TINY_B
+from tiny_configs import TINY_A, TINY_B, TINY_D
 
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -86,6 +86,83 @@ def test_sampled_generation_tiny_b(params):
     for number, (p, g) in enumerate(zip(prompts, got)):
         assert len(g) == 10
         follow_sampling(oracle, p, g, params, number)
+
+
+# A bfloat16 run's logits lie within about one percent of the plain implementation's
+# (of the largest logit); what is drawn from them is held to that.
+BF16_NEAR = 1e-2
+
+
+def follow_bfloat16(oracle, prompt, tokens, params, number):
+    """A continuation generated in bfloat16, token by token along the ENGINE's tokens, against
+    the plain implementation's 64-bit logits for the same history.  Greedy: the chosen token's
+    plain logit is within ``BF16_NEAR`` (of the largest logit) of the plain maximum.  Sampled:
+    with the request's own uniform number ``u`` for that token, ``u`` lies in the chosen
+    token's interval of the plain cumulative distribution, widened by what logits off by
+    ``BF16_NEAR`` can move the distribution's edges.  Returns the largest distance seen."""
+    from zig_ai_amd.sampling import UniformStream
+    stream = UniformStream(params.get("seed", 42), number)
+    seq = list(prompt)
+    worst = 0.0
+    T = params["temperature"]
+    for k, tok in enumerate(tokens):
+        logits = oracle.logits(seq)[-1].double()
+        scale = float(logits.abs().max())
+        if T <= 0:
+            gap = float(logits.max() - logits[tok]) / scale
+            assert gap <= BF16_NEAR, f"token {k}: engine chose {tok}, {gap:.2e} below the plain maximum"
+            worst = max(worst, gap)
+        else:
+            p = torch.softmax(logits / T, dim=0)
+            hi = float(p[:tok + 1].sum())
+            lo = hi - float(p[tok])
+            # every logit off by at most e: every probability by a factor within exp(+-2e/T)
+            slack = float(torch.expm1(torch.tensor(2.0 * BF16_NEAR * scale / T)))
+            u = stream.at(k)
+            assert lo - slack <= u <= hi + slack, \
+                f"token {k}: u = {u:.4f} outside [{lo:.4f}, {hi:.4f}] +- {slack:.3f} of token {tok}"
+            worst = max(worst, lo - u, u - hi, 0.0)
+        seq.append(tok)
+    return worst
+
+
+@pytest.mark.parametrize("temperature", [0.0, 0.7])
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_generation_in_bfloat16_through_scheduler_and_graphs(name, temperature):
+    """bfloat16 through everything serving uses at once: the scheduler (prompts in portions,
+    requests that join late), up to eight decode steps issued ahead with the tokens handed
+    over on the device, recorded graphs, the sampler on the device.  Each generated token
+    is checked against the plain implementation given the same history."""
+    from zig_ai_amd.engine import Engine
+    cfg, seed, lens = {"B": (TINY_B, 1, (1, 8, 31, 64, 100)), "D": (TINY_D, 3, (150, 9, 66, 40))}[name]
+    # tiny-B's weights as its workload writes them; D (matrix-core attention) with the
+    # weights under which a misplaced key would show
+    folder = folder_for(cfg, seed, torch.bfloat16, weights="as written" if name == "B" else "sharp")
+    oracle = plain.PlainLfm2(folder)
+    prompts = [eu.random_tokens(n, cfg["vocab_size"], 500 + n) for n in lens]
+    engine = Engine(folder, dtype="bfloat16", page_size=8, num_pages=128, max_num_seqs=3,
+                    chunk_size=16, max_num_batched_tokens=40, multi_step=8)
+    params = dict(temperature=temperature, seed=1234)
+    got = engine.generate(prompts, max_new_tokens=24, eos_token_id=-1, **params)
+    for number, (p, g) in enumerate(zip(prompts, got)):
+        assert len(g) == 24
+        follow_bfloat16(oracle, p, g, params, number)
+    graphs = engine.runner.graphs
+    assert graphs is not None and graphs.replays >= 24, "the decode steps were not replayed"
+    stats = engine.stats()
+    assert stats["requests"] == 0 and all(g["pages_free"] == g["pages"] for g in stats["groups"])
+
+
+def test_an_engine_takes_a_model_that_is_already_built():
+    """``Engine`` around ``DecoderModel.from_random``: no folder on the way."""
+    from zig_ai_amd.engine import DecoderModel, Engine
+    model = DecoderModel.from_random(TINY_A, seed=0, dtype="float32", **eu.sharp_kwargs())
+    folder = folder_for(TINY_A, 0)
+    oracle = plain.PlainLfm2(folder)
+    prompts = [eu.random_tokens(n, 256, 200 + n) for n in (5, 17)]
+    engine = Engine(model, page_size=4, num_pages=64, max_num_seqs=4)
+    got = engine.generate(prompts, max_new_tokens=8, temperature=0.0, eos_token_id=-1)
+    assert got == [oracle.greedy(p, 8) for p in prompts]
 
 
 def test_tokens_do_not_depend_on_scheduling():

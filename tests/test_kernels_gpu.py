@@ -2,7 +2,7 @@
 sizes other than the engine's (odd widths, tails in every dimension, head sizes
 from 16 to 256, any group size).
 
-Tolerances, fixed beforehand: a kernel computing in 32-bit must agree with the
+Tolerances, set from the arithmetic and confirmed by measurement: a kernel computing in 32-bit must agree with the
 float64 formula to 2e-5 of the result's largest magnitude (accumulation order);
 a kernel that stores bfloat16 adds one rounding of the stored value, 2^-8
 relative, so 6e-3 of the largest magnitude.

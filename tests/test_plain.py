@@ -147,16 +147,37 @@ def test_conv_identity_and_causality():
 
 
 def test_short_conv_mixer_order_of_gates():
-    """(B, C, x) in that order: B gates the input of the convolution, C its output."""
-    H, T = 4, 5
-    x = rnd(T, H, seed=25)
-    w = {"in_proj": rnd(3 * H, H, seed=26), "conv": rnd(H, 3, seed=27), "out_proj": torch.eye(H, dtype=D)}
-    z = x @ w["in_proj"].T
-    B, C, xx = z[:, :H], z[:, H:2 * H], z[:, 2 * H:]
-    want = C * plain.causal_depthwise_conv(B * xx, w["conv"], None)
-    assert torch.allclose(plain.short_conv_mixer(x, w), want)
-    wrong = B * plain.causal_depthwise_conv(C * xx, w["conv"], None)
-    assert not torch.allclose(want, wrong)
+    """(B, C, x) in that order: B gates the input of the convolution, C its output.
+    Seen by what each gate can reach, not by the formula again: in_proj is chosen so
+    that B[t] is feature 0 of token t, C[t] feature 1 and x[t] feature 2, and the filter
+    is all ones.  A token whose B is zero then vanishes from the L outputs that its
+    input reaches (and those outputs no longer depend on its x); a token whose C is zero
+    has a zero output of its own and nothing else changes."""
+    H, T, L = 4, 9, 3
+    x = rnd(T, H, seed=25) + 2.0                       # no accidental zeros
+    in_proj = torch.zeros((3 * H, H), dtype=D)
+    in_proj[0:H, 0] = 1.0                              # B[t, c] = x[t, 0]
+    in_proj[H:2 * H, 1] = 1.0                          # C[t, c] = x[t, 1]
+    in_proj[2 * H:3 * H, 2] = 1.0                      # xx[t, c] = x[t, 2]
+    w = {"in_proj": in_proj, "conv": torch.ones((H, L), dtype=D), "out_proj": torch.eye(H, dtype=D)}
+    y = plain.short_conv_mixer(x, w)
+    for t in range(T):                                 # the definition, token by token
+        want = x[t, 1] * sum(x[s, 0] * x[s, 2] for s in range(max(0, t - L + 1), t + 1))
+        assert torch.allclose(y[t], want.expand(H))
+    t0 = 4
+    xb = x.clone()
+    xb[t0, 0] = 0.0                                    # B of token t0 is zero
+    yb = plain.short_conv_mixer(xb, w)
+    xb2 = xb.clone()
+    xb2[t0, 2] = 123.0                                 # ... so its x reaches nothing
+    assert torch.equal(plain.short_conv_mixer(xb2, w), yb)
+    changed = [t for t in range(T) if not torch.equal(yb[t], y[t])]
+    assert changed == list(range(t0, t0 + L))          # the outputs its input reached
+    xc = x.clone()
+    xc[t0, 1] = 0.0                                    # C of token t0 is zero
+    yc = plain.short_conv_mixer(xc, w)
+    assert yc[t0].abs().max() == 0
+    assert [t for t in range(T) if not torch.equal(yc[t], y[t])] == [t0]
 
 
 # ------------------------------------------------------------------------- ffn

@@ -372,6 +372,96 @@ def test_toy_routing_and_position_parts_step_through_the_engine():
             assert eu.rel_err(g, e) < 1e-4
 
 
+# ------------------- a position encoding inside a mixer decides whether steps are recorded
+class WavedLfm2Config:
+    """LFM2's own parts with the attention's rotary encoding replaced by the position part
+    named under ``position_kind``."""
+
+    def __init__(self, data):
+        self.data = dict(data)
+
+    @classmethod
+    def from_dict(cls, data):
+        return cls(data)
+
+    def to_dict(self):
+        return dict(self.data)
+
+    def to_spec(self):
+        import dataclasses
+
+        from zig_ai_amd.config.lfm2 import Lfm2Config
+        from zig_ai_amd.config.spec import LayerSpec, PartSpec
+        inner = dict(self.data, architectures=["Lfm2ForCausalLM"])
+        kind = inner.pop("position_kind")
+        spec = Lfm2Config.from_dict(inner).to_spec()
+        waves = PartSpec(kind, {"head_dim": spec.layers[0].mixer.params.get("head_dim", 16),
+                                "rate": 0.7, "amplitude": 0.5})
+        layers = []
+        for layer in spec.layers:
+            parts = dict(layer.parts)
+            if parts["mixer"].kind == "gqa_attention":
+                parts["mixer"] = parts["mixer"].with_params(position=waves)
+            layers.append(LayerSpec(parts, layer.arrangement))
+        return dataclasses.replace(spec, architecture=self.data["architectures"][0], layers=tuple(layers))
+
+
+WAVED = {"architectures": ["ToyWavedForCausalLM"], "model_type": "lfm2", "hidden_size": 64,
+         "num_hidden_layers": 3, "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 16,
+         "vocab_size": 97, "layer_types": ["full_attention", "conv", "full_attention"],
+         "intermediate_size": 96, "rope_theta": 10000.0, "norm_eps": 1e-5, "conv_L_cache": 3,
+         "conv_bias": False, "tie_embedding": True, "max_position_embeddings": 512}
+
+
+def test_a_nested_position_part_decides_whether_steps_are_recorded():
+    """The attention mixer holds its position encoding inside it.  The model asks nested
+    parts too whether a step may be recorded: with a position part that declares nothing
+    (``graph_safe`` is false unless a part says otherwise) no graph is ever made, although
+    every other part of the model is the framework's own and safe; the same encoding
+    declared safe is recorded, and replayed steps give the logits of steps issued one
+    kernel at a time.  Nothing under the package changes for either."""
+    from zig_ai_amd.config import register_architecture
+    from zig_ai_amd.engine import DecoderModel, ModelRunner, StepEntry
+    from zig_ai_amd.parts import lookup, register_position
+    routed_classes()
+    looking = lookup("position", "toy_added_waves")
+    assert not looking.graph_safe
+
+    class RecordableWaves(looking):
+        """The same arithmetic; it only uses the positions on the device."""
+        kind = "toy_added_waves_recordable"
+        graph_safe = True
+
+    register_position(RecordableWaves.kind, RecordableWaves)
+    register_architecture("ToyWavedForCausalLM", WavedLfm2Config)
+    tokens = eu.random_tokens(60, 97, 5)
+    outs = {}
+    for kind in ("toy_added_waves", RecordableWaves.kind):
+        folder = eu.model_folder(dict(WAVED, position_kind=kind), 21, torch.float32, **eu.sharp_kwargs())
+        model = DecoderModel.from_folder(folder, "float32")
+        assert model.graph_safe == (kind == RecordableWaves.kind)
+        runner = ModelRunner(model, page_size=4, num_pages=20, num_slots=2)
+        assert (runner.graphs is not None) == model.graph_safe
+        runner.admit("r")
+        out = [runner.step([StepEntry("r", tokens[:20], [19])]).cpu()]
+        for p in range(20, 60):
+            out.append(runner.step([StepEntry("r", tokens[p:p + 1], [0])]).cpu())
+            if p % 7 == 0:
+                torch.cuda.synchronize()
+        outs[kind] = torch.cat(out)
+        if runner.graphs is not None:
+            assert runner.graphs.captures >= 1 and runner.graphs.replays >= 35
+    # the two models have the same tensors (same seed, same names): recorded or not, the
+    # same logits
+    assert eu.rel_err(outs[RecordableWaves.kind], outs["toy_added_waves"].double()) < 2e-5
+    # and they are the model's: the rotary model with these weights gives other logits
+    # (the encoding is really applied)
+    plain_folder = eu.model_folder({k: v for k, v in dict(WAVED, architectures=["Lfm2ForCausalLM"]).items()},
+                                   21, torch.float32, **eu.sharp_kwargs())
+    rotary = plain.PlainLfm2(plain_folder).logits(tokens)[19:]
+    assert eu.rel_err(outs["toy_added_waves"], rotary) > 1e-2
+
+
 # ---------- another arrangement (four norms, two mixers), a mixer that pages ONE vector
 def sandwich_classes():
     from zig_ai_amd.kernels import ops

@@ -84,6 +84,13 @@ REAL_2L = {
 # hundreds of tokens under every way of cutting them
 REAL_3L = dict(REAL_2L, num_hidden_layers=3, layer_types=["conv", "full_attention", "conv"])
 
+# two layers at the LFM2-350M shape's sizes (hidden 1024, two query heads per key/value
+# head, feed-forward 6656 -> 4608) and at the LFM2-2.6B shape's feed-forward width
+# (10752 -> 7168): the sizes the other measured shapes add to the 1.2B shape's
+REAL_350M_2L = dict(REAL_2L, hidden_size=1024, num_attention_heads=16, num_key_value_heads=8,
+                    block_ff_dim=6656)
+REAL_26B_2L = dict(REAL_2L, block_ff_dim=10752)
+
 # widths that are multiples of neither 8 nor 16: fine in 32-bit, refused in bfloat16
 TINY_E = {
     "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",

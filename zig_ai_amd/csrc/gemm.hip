@@ -1011,10 +1011,15 @@ static int rows16_allow_lds(const void* kernel, size_t bytes) {
   return 0;
 }
 
-// For tuning runs: row groups per workgroup of the decode products that take no such
-// argument (0: the launchers choose).
+// Only in a build made for tuning runs (-DZA_TUNING_BUILD): row groups per workgroup of
+// the decode products that take no such argument (0: the launchers choose).  The
+// library the engine loads has no such switch: nothing process-wide steers its launches.
+#ifdef ZA_TUNING_BUILD
 static int rows16_groups_override = 0;
 extern "C" void za_gemm_rows16_set_groups_per_block(int groups) { rows16_groups_override = groups; }
+#else
+static constexpr int rows16_groups_override = 0;
+#endif
 
 static bool rows16_takes_norm(int K, int ksplit) {
   return ksplit == 1 && K <= 4096 && K % 512 == 0;

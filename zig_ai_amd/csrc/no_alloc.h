@@ -1,7 +1,6 @@
 // An entry point for callers that cannot allocate device memory: code under HIP graph
 // capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart
-// in the reference (whose sampler runs on the host after copying every logit back:
-// /root/reference/src/main.zig:1273,1340).
+// in the reference.
 //
 // za_argmax_no_alloc is za_argmax (sampling.hip) with the workspace of the chunked form
 // taken from an array that lives in the library's own device image instead of from the
@@ -13,9 +12,10 @@
 //
 //   * Nothing is allocated or freed, on the device or through any library, by the call.
 //   * Returns 0, ZA_ERR_ARG (-1: a null pointer, a count below zero, chunks < 1),
-//     ZA_ERR_UNSUPPORTED (-2: n_rows * chunks exceeds the maximum, or chunks > 65535),
-//     or a hipError_t; za_no_alloc_last_error() gives the reason as text for the calling
-//     thread's last failed call.
+//     ZA_ERR_UNSUPPORTED (-2: n_rows * chunks exceeds the maximum, chunks > 65535, or a
+//     device number of 64 and more), or the hipError_t of the HIP call that failed (a
+//     launch, hipGetDevice, hipGetSymbolAddress); za_no_alloc_last_error() gives the
+//     reason as text for the calling thread's last failed call.
 //   * Every partial result the merge reads is written by the same call first, so
 //     nothing has to be cleared between calls.
 //   * All calls on one GPU share that GPU's array: calls that overlap there (two

@@ -605,29 +605,39 @@ static thread_local char no_alloc_error[192];
 
 extern "C" const char* za_no_alloc_last_error(void) { return no_alloc_error; }
 
-// The current device's copy of `scratch`, or null with the reason in no_alloc_error.
-static void* scratch_address() {
+// The current device's copy of `scratch` into *out.  0, or the failed call's hipError_t
+// (ZA_ERR_UNSUPPORTED for a device number beyond the table) with the reason in
+// no_alloc_error.
+static int scratch_address(void** out) {
+  *out = nullptr;
   int device = -1;
   hipError_t e = hipGetDevice(&device);
-  if (e != hipSuccess || device < 0 || device >= ZA_NO_ALLOC_MAX_DEVICES) {
+  if (e != hipSuccess) {
+    snprintf(no_alloc_error, sizeof no_alloc_error, "za_argmax_no_alloc: hipGetDevice: %s",
+             hipGetErrorString(e));
+    return (int)e;
+  }
+  if (device < 0 || device >= ZA_NO_ALLOC_MAX_DEVICES) {
     snprintf(no_alloc_error, sizeof no_alloc_error,
-             "za_argmax_no_alloc: no current device below %d (hipGetDevice: %s)",
-             ZA_NO_ALLOC_MAX_DEVICES, hipGetErrorString(e));
-    return nullptr;
+             "za_argmax_no_alloc: device %d is beyond the %d this library keeps an address for",
+             device, ZA_NO_ALLOC_MAX_DEVICES);
+    return ZA_ERR_UNSUPPORTED;
   }
   std::lock_guard<std::mutex> hold(scratch_lock);
   if (!scratch_of_device[device]) {
     void* ptr = nullptr;
     e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
-    if (e != hipSuccess || !ptr) {
+    if (e == hipSuccess && !ptr) e = hipErrorInvalidSymbol;
+    if (e != hipSuccess) {
       snprintf(no_alloc_error, sizeof no_alloc_error,
                "za_argmax_no_alloc: hipGetSymbolAddress on device %d: %s", device,
                hipGetErrorString(e));
-      return nullptr;
+      return (int)e;
     }
     scratch_of_device[device] = ptr;
   }
-  return scratch_of_device[device];
+  *out = scratch_of_device[device];
+  return 0;
 }
 
 extern "C" int za_argmax_no_alloc(const float* logits, int n_rows, int vocab, int* out,
@@ -652,8 +662,9 @@ extern "C" int za_argmax_no_alloc(const float* logits, int n_rows, int vocab, in
              n_rows, chunks, (long long)n_rows * chunks, ZA_ARGMAX_NO_ALLOC_MAX_PARTIALS);
     return ZA_ERR_UNSUPPORTED;
   }
-  void* base = scratch_address();
-  if (!base) return ZA_ERR_ARG;
+  void* base = nullptr;
+  const int found = scratch_address(&base);
+  if (found != 0) return found;
   float* part_v = reinterpret_cast<float*>(base);
   int* part_i = reinterpret_cast<int*>(reinterpret_cast<unsigned char*>(base) +
                                        (size_t)ZA_ARGMAX_NO_ALLOC_MAX_PARTIALS * sizeof(float));

@@ -23,14 +23,17 @@ from .scheduler import RUNNING, Request, ScheduledEntry, Scheduler
 
 
 class Engine:
-    def __init__(self, model_dir: str, dtype: str = "bfloat16", page_size: int = 16,
+    def __init__(self, model_dir, dtype: str = "bfloat16", page_size: int = 16,
                  num_pages: Optional[int] = None, max_num_seqs: int = 64,
                  max_num_batched_tokens: int = 2048, chunk_size: int = 512,
                  max_model_len: Optional[int] = None, use_graphs: bool = True,
                  portion_graphs: bool = False,
                  on_step=None, memory_fraction: float = 0.85, multi_step: int = 8,
-                 reproducible: bool = False):
-        """``num_pages``: pages per cache group; by default enough for
+                 reproducible: bool = False, warm_up: bool = True):
+        """``model_dir``: a model folder, or a ``DecoderModel`` that is already built (from a
+        folder or ``DecoderModel.from_random``; ``dtype`` and ``reproducible`` are then the
+        model's own).
+        ``num_pages``: pages per cache group; by default enough for
         ``max_num_seqs`` requests of ``max_model_len`` tokens (the model's
         ``max_position_embeddings`` if not given, capped at 8192), but no more than
         fit into ``memory_fraction`` of the device memory that is free once the
@@ -51,8 +54,12 @@ class Engine:
         stream with atomics, several ranges of K to one element in the hardware's order,
         so two runs agree to 32-bit rounding of the stream only; ``True`` keeps every sum
         in a fixed order (some 10 % slower decoding), and the same requests scheduled the
-        same way then give the same bits."""
-        self.model = DecoderModel.from_folder(model_dir, dtype, reproducible=reproducible)
+        same way then give the same bits.
+        ``warm_up``: see ``Engine.warm_up``; done here, before the first request."""
+        if isinstance(model_dir, DecoderModel):
+            self.model = model_dir
+        else:
+            self.model = DecoderModel.from_folder(model_dir, dtype, reproducible=reproducible)
         limit = max_model_len or self.model.spec.max_position or 8192
         if max_model_len is None:
             limit = min(limit, 8192)
@@ -84,6 +91,54 @@ class Engine:
                                    chunk_size, limit)
         self._next_id = 0
         self.timings = {"steps": 0, "step_seconds": 0.0, "tokens_run": 0, "tokens_generated": 0}
+        self.max_num_batched_tokens = int(max_num_batched_tokens)
+        self.max_num_seqs = int(max_num_seqs)
+        self.warm_up_steps = self.warm_up() if warm_up else 0
+
+    # ----------------------------------------------------------------- warm-up
+    WARM_UP_MIN_WEIGHT = 1 << 19      # elements; smaller products are never timed
+
+    def warm_up(self) -> int:
+        """The GEMM library times its candidates for a shape at the shape's first call
+        (some 10 ms a shape, shared by the row counts of a block: 17-32, 33-64, 65-128,
+        129-255, then blocks of 256).  Run one step of every block up to
+        ``max_num_batched_tokens`` now, with a request of its own that is released again,
+        so that no request pays for it.  Nothing to do, and nothing done, for 32-bit
+        models, models that take the library's first answer (``reproducible``,
+        ZIG_AI_GEMM_TUNE=0) and models without a projection large enough to be timed.
+        Returns the number of steps run."""
+        from .model import walk_parts
+        model, runner = self.model, self.runner
+        rt = model.runtime
+        wanted = ops.library_tuning if rt.tune is None else rt.tune
+        if rt.dtype != torch.bfloat16 or not wanted:
+            return 0
+        top = [model.embedding, model.head] + [p for b in model.blocks for p in b.parts.values()]
+        large = any(isinstance(v, torch.Tensor) and v.dim() == 2 and v.dtype == torch.bfloat16
+                    and v.numel() >= self.WARM_UP_MIN_WEIGHT
+                    for part in top for q in walk_parts(part) for v in vars(q).values())
+        if not large:
+            return 0
+        sizes = [m for m in (32, 64, 128, 255) if m <= self.max_num_batched_tokens]
+        sizes += list(range(256, self.max_num_batched_tokens + 1, 256))
+        name = ("warm-up", id(self))
+        steps = 0
+        for m in sizes:
+            if m > self.max_model_len:
+                break
+            # (steps of up to max_num_seqs rows want every row's logits, as a decode batch
+            # of that many requests does: the head's shapes are met too)
+            want = list(range(m)) if m <= max(self.max_num_seqs, 16) else [m - 1]
+            runner.admit(name)
+            try:
+                if not runner.cache.can_reserve(name, m):
+                    break
+                runner.step([StepEntry(name, [0] * m, want)])
+                steps += 1
+            finally:
+                runner.release(name)
+        torch.cuda.synchronize(rt.device)
+        return steps
 
     # ---------------------------------------------------------------- requests
     def add_request(self, prompt: Sequence[int], max_new_tokens: int,

@@ -52,6 +52,25 @@ def arrangement_slots(arrangement, layer) -> Dict[str, str]:
     return slots
 
 
+def walk_parts(part):
+    """``part`` and every part nested in it (an attribute that is itself a part, as the
+    position encoding inside an attention mixer), at any depth."""
+    seen, todo = set(), [part]
+    while todo:
+        p = todo.pop()
+        if id(p) in seen:
+            continue
+        seen.add(id(p))
+        yield p
+        for v in getattr(p, "__dict__", {}).values():
+            if isinstance(v, parts.Part):
+                todo.append(v)
+            elif isinstance(v, (list, tuple)):
+                todo.extend(e for e in v if isinstance(e, parts.Part))
+            elif isinstance(v, dict):
+                todo.extend(e for e in v.values() if isinstance(e, parts.Part))
+
+
 class DecoderModel:
     def __init__(self, spec: ModelSpec, tensors: Mapping[Any, Mapping[str, torch.Tensor]],
                  runtime: parts.Runtime):
@@ -64,8 +83,9 @@ class DecoderModel:
 
         sources = set()
 
-        def note(cls_or_obj) -> None:
-            sources.update(getattr(cls_or_obj, "kernel_sources", ()))
+        def note(part) -> None:
+            for p in walk_parts(part):
+                sources.update(getattr(p, "kernel_sources", ()))
 
         self.embedding = make("embedding", spec.embedding, ("embedding",))
         note(self.embedding)
@@ -108,9 +128,11 @@ class DecoderModel:
             for key, _ in self.cache_keys(call):
                 if self.cache_needs[key] is not None and key not in writers:
                     raise ValueError(f"cache {key} is read but no run-order entry writes it")
-        every = [self.embedding, self.final_norm, self.head]
+        # (what a part holds inside it, a mixer's position encoding for one, is asked too)
+        top = [self.embedding, self.final_norm, self.head]
         for b in self.blocks:
-            every += list(b.parts.values())
+            top += list(b.parts.values())
+        every = [q for p in top for q in walk_parts(p)]
         self.item_granularities = sorted({
             g for p in every for g in getattr(p, "item_granularities", ())})
         self.kernel_sources = sorted(sources)
@@ -128,12 +150,14 @@ class DecoderModel:
     # ------------------------------------------------------------- construction
     @classmethod
     def from_folder(cls, model_dir: str, dtype="bfloat16", device: Optional[torch.device] = None,
-                    reproducible: bool = False):
-        """``reproducible``: every sum in a fixed order (see ``Runtime.stream_additions``)."""
+                    reproducible: bool = False, library_tuning: Optional[bool] = None):
+        """``reproducible``: every sum in a fixed order (see ``Runtime.stream_additions``).
+        ``library_tuning``: see ``Runtime.library_tuning``."""
         device = device or require_gpu()
         config = load_config(model_dir)
         spec = config.to_spec()
-        rt = parts.Runtime(device=device, dtype=run_dtype(dtype), stream_additions=not reproducible)
+        rt = parts.Runtime(device=device, dtype=run_dtype(dtype), stream_additions=not reproducible,
+                           library_tuning=library_tuning)
         tensors = load_tensors(model_dir, spec, rt.dtype, device)
         model = cls(spec, tensors, rt)
         model.config = config
@@ -143,7 +167,8 @@ class DecoderModel:
     def from_random(cls, config, seed: int = 0, dtype="bfloat16",
                     device: Optional[torch.device] = None, std: float = 0.02,
                     norm_init: str = "ones", reproducible: bool = False,
-                    role_std: Optional[Mapping[str, float]] = None):
+                    role_std: Optional[Mapping[str, float]] = None,
+                    library_tuning: Optional[bool] = None):
         """The model that ``write_random_model(config, folder, seed, ...)`` followed by
         ``from_folder`` gives, without the trip through a file: every tensor is drawn on the
         device by the same keyed generator (a value depends on seed, tensor name and element
@@ -156,7 +181,8 @@ class DecoderModel:
         if isinstance(config, Mapping):
             config = config_from_dict(config)
         spec = config.to_spec()
-        rt = parts.Runtime(device=device, dtype=run_dtype(dtype), stream_additions=not reproducible)
+        rt = parts.Runtime(device=device, dtype=run_dtype(dtype), stream_additions=not reproducible,
+                           library_tuning=library_tuning)
         tensors: Dict[Any, Dict[str, torch.Tensor]] = {}
         for exp in expected_tensors(spec):
             stored = random_tensor(seed, exp.names[0], exp.rule.stored_shape or exp.rule.shapes[0],
@@ -207,14 +233,7 @@ class DecoderModel:
         entry's parts left under ``step.taps`` (the attention mixer: its queries, the
         keys and values it stored, its output); all copies that later kernels do not
         touch."""
-        # a model that keeps every sum in a fixed order also keeps the GEMM library's first
-        # answer for every shape: which of its candidates is fastest is decided by a clock
-        wanted = ops.library_tuning
-        ops.library_tuning = wanted and self.runtime.stream_additions
-        try:
-            return self._forward(step, views, taps)
-        finally:
-            ops.library_tuning = wanted
+        return self._forward(step, views, taps)
 
     def _forward(self, step: StepContext, views: Sequence[CacheView],
                  taps: Optional[List[Dict[str, torch.Tensor]]]) -> torch.Tensor:

@@ -383,14 +383,15 @@ def _k_splits(M: int, N: int, K: int) -> int:
 LIBRARY_WORKSPACE_BYTES = 64 << 20
 _library_workspace = {}
 # Whether the GEMM library's candidates for a shape of many rows are timed at the shape's
-# first call (csrc/blaslt.hip).  Which candidate wins can differ from run to run; a model
-# that promises the same bits run after run switches this off around its steps, and
-# ZIG_AI_GEMM_TUNE=0 switches it off for a whole process.
+# first call (csrc/blaslt.hip), for calls that do not say (``linear(..., tune=None)``).
+# Which candidate wins can differ from run to run; a model that promises the same bits run
+# after run passes ``tune=False`` with every product (``Runtime.tune``), and
+# ZIG_AI_GEMM_TUNE=0 switches the default off for a whole process.
 library_tuning = os.environ.get("ZIG_AI_GEMM_TUNE", "1") != "0"
 
 
 def _library_matmul(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype,
-                    splits: int) -> Optional[torch.Tensor]:
+                    splits: int, tune: Optional[bool] = None) -> Optional[torch.Tensor]:
     """``x @ weight^T`` through the GEMM library (csrc/blaslt.hip): ``[M, N]``, or the
     stack ``[splits, M, N]`` of 32-bit partial sums over ranges of K.  ``None`` when
     the library names no algorithm for the shape (nothing was launched)."""
@@ -405,7 +406,8 @@ def _library_matmul(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtyp
     shape = (splits, M, N) if splits > 1 else (M, N)
     out = torch.empty(shape, dtype=torch.float32 if f32 else torch.bfloat16, device=x.device)
     rc = _fn("blaslt", "za_lt_matmul")(_ptr(x), _ptr(weight), _ptr(out), M, N, K, 1 if f32 else 0,
-                                       splits, 1 if library_tuning else 0, _ptr(work),
+                                       splits, 1 if (library_tuning if tune is None else tune) else 0,
+                                       _ptr(work),
                                        LIBRARY_WORKSPACE_BYTES, _stream())
     if rc == -2:
         return None
@@ -463,7 +465,8 @@ def accumulate_plan(M: int, N: int, K: int, normed: bool) -> int:
 def linear(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
            out_dtype: Optional[torch.dtype] = None, force_tiled: bool = False,
            partial_ok: bool = False,
-           accumulate: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+           accumulate: Optional[torch.Tensor] = None,
+           tune: Optional[bool] = None) -> Optional[torch.Tensor]:
     """``x [M, K] @ weight[N, K]^T + bias`` with 32-bit accumulation.
 
     bfloat16 weights use the matrix-core kernels of csrc/gemm.hip up to
@@ -481,7 +484,10 @@ def linear(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
     own kernel.  With ``accumulate`` (the 32-bit ``[M, N]`` residual stream) a decode
     batch's product is added to that tensor with atomics and ``None`` comes back (the
     additions of the ranges of K arrive in the hardware's order: reproducible to
-    rounding only); otherwise the product comes back as usual and the caller adds it."""
+    rounding only); otherwise the product comes back as usual and the caller adds it.
+
+    ``tune``: whether the GEMM library may time its candidates at this shape's first call
+    (``None``: the process's default, ``library_tuning``)."""
     if len(x.shape) != 2 or weight.dim() != 2:
         raise KernelError(f"linear takes x [M, K] and weight [N, K], got {tuple(x.shape)} and "
                           f"{tuple(weight.shape)}")
@@ -582,7 +588,7 @@ def linear(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
         return stack
     if library:
         # (with ranges of K: one batched product, [P, M, K/P] x [P, K/P, N])
-        out = _library_matmul(x, weight, out_dtype, splits)
+        out = _library_matmul(x, weight, out_dtype, splits, tune)
         if out is not None:
             _note("linear", M=M, N=N, K=K, norm_in_product=False, added_to_stream=False,
                   partial_sums=splits, out=out.dtype)

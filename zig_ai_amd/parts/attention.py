@@ -131,6 +131,9 @@ class GroupedQueryAttention(Mixer):
         if pos is not None:
             self.position = lookup("position", pos.kind)(pos.params, {}, runtime)
         self.fused_rotation = bool(getattr(self.position, "fused_rotation", False))
+        # recorded into a graph only if the position encoding, too, never looks at a
+        # step's numbers on the host
+        self.graph_safe = self.position is None or bool(getattr(self.position, "graph_safe", False))
         # a decode step's norm, rotation and cache write can run inside its attention kernel
         self.rotation_in_attention = (
             self.fused_rotation and runtime.dtype == torch.bfloat16
@@ -141,7 +144,7 @@ class GroupedQueryAttention(Mixer):
     def forward(self, x, step, cache, stream: Optional[torch.Tensor] = None):
         nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
         T = x.shape[0]
-        qkv = ops.linear(x, self.w_qkv, self.b_qkv)
+        qkv = ops.linear(x, self.w_qkv, self.b_qkv, tune=self.runtime.tune)
         slots = step.slot_mapping[cache.group]
         if self.rotation_in_attention and step.n_tokens == step.n_seqs and cache.writes \
                 and ops.decode_rope_fusable(qkv, nh, nkv, d, d, False, cache.kv.shape[3], self.scale):
@@ -162,7 +165,8 @@ class GroupedQueryAttention(Mixer):
                 self._leave_taps(step, cache, q, merged.view(T, nh, d))
             if not isinstance(o, ops.MergedRows):
                 o = o.view(T, nh * d)
-            return ops.linear(o, self.w_out, self.b_out, partial_ok=True, accumulate=stream)
+            return ops.linear(o, self.w_out, self.b_out, partial_ok=True, accumulate=stream,
+                              tune=self.runtime.tune)
         if self.position is None or self.fused_rotation:
             rot = self.position.rotary_dim if self.position is not None else 0
             q = ops.qk_norm_rope_kv_write(
@@ -214,7 +218,7 @@ class GroupedQueryAttention(Mixer):
         if getattr(step, "taps", None) is not None:
             self._leave_taps(step, cache, q, o)
         return ops.linear(o.view(T, nh * d), self.w_out, self.b_out, partial_ok=True,
-                          accumulate=stream)
+                          accumulate=stream, tune=self.runtime.tune)
 
     def _leave_taps(self, step, cache, q: torch.Tensor, o: torch.Tensor) -> None:
         """Diagnostics: the queries, the keys and values of the step's tokens as they lie in

@@ -78,8 +78,13 @@ class PagedNeed:
 
 @dataclass(frozen=True)
 class StateNeed:
-    """Per-request state of fixed size, zero for a new request; 32-bit floats unless
-    ``dtype`` says otherwise."""
+    """Per-request state of fixed size; 32-bit floats unless ``dtype`` says otherwise.
+    A new request's state is ZERO BYTES (the cache manager clears the slot at admission
+    and knows no other start).  A mixer whose state starts elsewhere (a running maximum
+    at -inf, a product at 1) stores it relative to that start, so that zero bytes mean
+    it (the maximum as ``exp(-m)`` or with a "seen anything" flag beside it, the product
+    minus one), or treats a request's first portion, ``step.ctx_lens_host[i] == 0``, as
+    the start itself."""
 
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
@@ -99,6 +104,16 @@ class Runtime:
     # and reproducible to 32-bit rounding only.  False keeps every sum in a fixed order
     # (bitwise the same result for the same step, run after run).
     stream_additions: bool = True
+    # Whether the GEMM library's candidates for a shape of many rows are timed at the
+    # shape's first call (the fastest is kept; which one wins can differ from run to
+    # run).  None: the process's default (on, unless ZIG_AI_GEMM_TUNE=0).  A runtime that
+    # keeps every sum in a fixed order takes the library's first answer.
+    library_tuning: Optional[bool] = None
+
+    @property
+    def tune(self) -> Optional[bool]:
+        """What parts hand to ``ops.linear(..., tune=)``."""
+        return False if not self.stream_additions else self.library_tuning
 
 
 class Part:
@@ -175,6 +190,11 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
+    # Held inside a mixer; the model asks nested parts, too, for ``graph_safe``,
+    # ``kernel_sources`` and ``item_granularities``.  ``graph_safe = True`` only if
+    # ``apply`` never looks at ``positions`` (or anything of the step) on the host.
+    graph_safe = False
+
     def apply(self, q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor):
         """Generic path: return encoded ``(q, k)`` of shape ``[T, heads, head_dim]``."""
         raise NotImplementedError

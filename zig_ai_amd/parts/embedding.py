@@ -53,7 +53,7 @@ class LinearHead(Part):
 
     def forward(self, x) -> torch.Tensor:
         ops.check_projection_weight(self.weight, "output head")
-        return ops.linear(x, self.weight, out_dtype=torch.float32)
+        return ops.linear(x, self.weight, out_dtype=torch.float32, tune=self.runtime.tune)
 
 
 register_embedding(TokenEmbedding.kind, TokenEmbedding)

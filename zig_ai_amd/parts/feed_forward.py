@@ -48,8 +48,8 @@ class SwiGLU(FeedForward):
         else:
             if isinstance(x, ops.NormedRows):
                 x = x.materialise()
-            a = ops.swiglu(ops.linear(x, self.gate_up))
-        return ops.linear(a, self.down, partial_ok=True, accumulate=stream)
+            a = ops.swiglu(ops.linear(x, self.gate_up, tune=self.runtime.tune))
+        return ops.linear(a, self.down, partial_ok=True, accumulate=stream, tune=self.runtime.tune)
 
 
 register_feed_forward(SwiGLU.kind, SwiGLU)

@@ -20,6 +20,7 @@ class RotaryEmbedding(PositionEncoding):
     kind = "rope"
     kernel_sources = ("rope_kv",)
     fused_rotation = True   # the mixer's kernel rotates; ``apply`` is not called
+    graph_safe = True       # constants only: nothing of a step is looked at on the host
 
     def __init__(self, params, tensors, runtime: Runtime):
         super().__init__(params, tensors, runtime)

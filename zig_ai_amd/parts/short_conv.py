@@ -68,10 +68,11 @@ class ShortConv(Mixer):
             y = ops.in_proj_gated_conv(x, self.w_in, self.w_conv, self.b_conv, cache.state,
                                        step.slot_id)
         else:
-            z = ops.linear(x, self.w_in, self.b_in)
+            z = ops.linear(x, self.w_in, self.b_in, tune=self.runtime.tune)
             y = ops.short_conv(z, self.w_conv, self.b_conv, cache.state, step.token_seq,
                                step.seq_start, step.slot_id)
-        return ops.linear(y, self.w_out, self.b_out, partial_ok=True, accumulate=stream)
+        return ops.linear(y, self.w_out, self.b_out, partial_ok=True, accumulate=stream,
+                          tune=self.runtime.tune)
 
 
 register_mixer(ShortConv.kind, ShortConv)
