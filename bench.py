@@ -175,6 +175,9 @@ def main() -> int:
     ap.add_argument("--phase", choices=["all", "prefill", "decode"], default="all",
                     help="measure only one phase (for profiling); the JSON line then holds "
                          "only that phase")
+    ap.add_argument("--tuned", action="store_true",
+                    help="with --phase: let the GEMM library time its candidates as a plain run "
+                         "does (not under a profiler's counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -195,7 +198,7 @@ def main() -> int:
         cfg["layer_types"] = cfg["layer_types"][:args.layers]
     page = 16
     gen = torch.Generator().manual_seed(1234)
-    profiled = args.phase != "all"
+    profiled = args.phase != "all" and not args.tuned
 
     def tokens(n, vocab):
         return torch.randint(0, vocab, (n,), generator=gen).tolist()

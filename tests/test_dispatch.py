@@ -50,3 +50,25 @@ def test_when_the_output_projection_merges_the_context_ranges():
     assert not ops.merged_rows_pay(3, 12)
     assert not ops.merged_rows_pay(1, 1) and not ops.merged_rows_pay(1, 17) and not ops.merged_rows_pay(9, 2)
 
+
+
+def test_where_the_kernel_for_17_to_64_rows_is_taken():
+    """The feed-forward's fused first product up to 32 rows, for widths whose K is spans of
+    512 (at least two) up to 4096; the mixer's closing product of such a step adds itself to
+    the stream when K is short and enough workgroups come of it."""
+    assert ops.rows64_swiglu_fusable(17, 2048) and ops.rows64_swiglu_fusable(32, 1024)
+    assert ops.rows64_swiglu_fusable(20, 1536) and ops.rows64_swiglu_fusable(24, 4096)
+    assert not ops.rows64_swiglu_fusable(16, 2048)      # the decode kernel's
+    assert not ops.rows64_swiglu_fusable(33, 2048)      # measured no faster than the library's path
+    assert not ops.rows64_swiglu_fusable(20, 512) and not ops.rows64_swiglu_fusable(20, 1280)
+    assert not ops.rows64_swiglu_fusable(20, 4608)
+    assert ops.rows64_add_splits(2048, 2048) == 2       # 32 tiles x 2 ranges of 1,024
+    assert ops.rows64_add_splits(2048, 4096) == 4
+    assert ops.rows64_add_splits(2048, 8192) == 0       # the library's ranges of K are faster
+    assert ops.rows64_add_splits(1024, 1024) == 0       # 16 workgroups: too few
+    assert ops.rows64_add_splits(4096, 1024) == 1
+    assert ops.rows64_add_splits(2048, 1280) == 0       # no cut into spans of 512
+    for K in range(512, 9000, 256):
+        for N in (1024, 2048, 4096):
+            ks = ops.rows64_add_splits(N, K)
+            assert ks == 0 or ops.rows64_takes(32, K, ks)

@@ -440,14 +440,130 @@ def test_gemm_bf16_decode_rows_added_to_the_stream(M, N, K):
     assert rel_err(stream, stream0.double() + product) < F32_TOL
     assert o.linear(x.to(dev()), w.to(dev()), b.to(dev()), accumulate=stream) is None
     assert rel_err(stream, stream0.double() + 2 * product) < F32_TOL
-    # more than a decode batch, or 32-bit weights: the product comes back instead
-    many = rand((20, K), torch.bfloat16, 64).to(dev())
-    kept = torch.zeros((20, N), dtype=torch.float32, device=dev())
+    # more rows than any kernel that adds takes, or 32-bit weights: the product comes back instead
+    many = rand((40, K), torch.bfloat16, 64).to(dev())
+    kept = torch.zeros((40, N), dtype=torch.float32, device=dev())
     back = o.linear(many, w.to(dev()), accumulate=kept)
     assert back is not None and not kept.any()
     kept = torch.zeros((M, N), dtype=torch.float32, device=dev())
     back = o.linear(x.float().to(dev()), w.float().to(dev()), accumulate=kept)
     assert back is not None and not kept.any()
+
+
+# ------------------------------------------------- products of 17 to 64 rows, fused forms
+@pytest.mark.parametrize("M", [1, 5, 17, 20, 32, 33, 47, 64])
+@pytest.mark.parametrize("N,K", [(50, 1024), (200, 1536), (6144, 2048), (130, 4096), (64, 2560)])
+def test_rows64_products(M, N, K):
+    """The kernel for steps of 17 to 64 rows, alone: every number of row blocks (and fewer
+    rows than a block), tiles with tails in N, two to eight spans of K, odd numbers of
+    spans; stored, with the norm run by the kernel (rows picked out of a longer stream),
+    through the SwiGLU gate, and added to a stream with K in ranges."""
+    o = ops()
+    eps = 1e-5
+    w = rand((N, K), torch.bfloat16, 80)
+    x = rand((M, K), torch.bfloat16, 81)
+    exact = x.double() @ w.double().T
+    got = o.linear_rows64(x.to(dev()), w.to(dev()))
+    assert got.dtype == torch.bfloat16 and rel_err(got, exact) < BF16_TOL
+    # the norm on the way in
+    stream = rand((M + 3, K), torch.float32, 82) * 3.0
+    nw = 1.0 + rand((K,), torch.float32, 83)
+    rows = torch.tensor([(5 * i + 2) % (M + 3) for i in range(M)], dtype=torch.int32)
+    for pick in (None, rows):
+        xs = stream[:M] if pick is None else stream[pick.long()]
+        src = stream[:M].contiguous() if pick is None else stream
+        normed = o.NormedRows(src.to(dev()), nw.to(dev()), eps, torch.bfloat16,
+                              None if pick is None else pick.to(dev()))
+        a, scale = _normed_operands(xs, nw, eps)
+        want = scale * (a @ w.double().T)
+        assert rel_err(o.linear_rows64(normed, w.to(dev())), want) < BF16_TOL
+        if N % 2 == 0:
+            I = N // 2
+            g, u = want[:, :I], want[:, I:]
+            gated = o.linear_rows64(normed, w.to(dev()), mode=o.ROWS64_SWIGLU)
+            assert gated.shape == (M, I) and rel_err(gated, g / (1 + torch.exp(-g)) * u) < BF16_TOL
+    # added to a stream, K in every number of ranges the kernel takes
+    for ks in (1, 2, 3, 4):
+        if not o.rows64_takes(M, K, ks):
+            continue
+        base = rand((M, N), torch.float32, 84)
+        on_device = base.clone().to(dev())
+        assert o.linear_rows64(x.to(dev()), w.to(dev()), mode=o.ROWS64_ADD, accumulate=on_device,
+                               ksplit=ks) is None
+        assert rel_err(on_device, base.double() + exact) < F32_TOL
+        o.linear_rows64(x.to(dev()), w.to(dev()), mode=o.ROWS64_ADD, accumulate=on_device, ksplit=ks)
+        assert rel_err(on_device, base.double() + 2 * exact) < F32_TOL
+
+
+def test_rows64_rows_do_not_depend_on_the_batch():
+    """A row's result is a function of that row: the same bits whichever rows stand beside
+    it and wherever it stands (the sums over K run in one order for every row)."""
+    o = ops()
+    N, K = 300, 2048
+    w = rand((N, K), torch.bfloat16, 85).to(dev())
+    x = rand((64, K), torch.bfloat16, 86)
+    whole = o.linear_rows64(x.to(dev()), w).cpu()
+    some = o.linear_rows64(x[10:30].contiguous().to(dev()), w).cpu()
+    assert torch.equal(some, whole[10:30])
+    one = o.linear_rows64(x[63:64].contiguous().to(dev()), w).cpu()
+    assert torch.equal(one, whole[63:64])
+
+
+def test_rows64_refuses_what_it_does_not_take():
+    o = ops()
+    w = rand((64, 1024), torch.bfloat16, 87).to(dev())
+    with pytest.raises(o.KernelError, match="64 rows"):
+        o.linear_rows64(rand((65, 1024), torch.bfloat16, 88).to(dev()), w)
+    for K in (512, 1000, 1280):                         # one span only; no multiple of 512
+        wk = rand((64, K), torch.bfloat16, 89).to(dev())
+        with pytest.raises(o.KernelError):
+            o.linear_rows64(rand((20, K), torch.bfloat16, 90).to(dev()), wk)
+    with pytest.raises(o.KernelError):                  # ranges of K only when adding
+        o.linear_rows64(rand((20, 2048), torch.bfloat16, 91).to(dev()),
+                        rand((64, 2048), torch.bfloat16, 92).to(dev()), ksplit=2)
+    # the norm's weight lies in LDS: K up to 4096
+    wide = o.NormedRows(rand((20, 8192), torch.float32, 93).to(dev()),
+                        rand((8192,), torch.float32, 94).to(dev()), 1e-5, torch.bfloat16)
+    with pytest.raises(o.KernelError, match="does not support"):
+        o.linear_rows64(wide, rand((64, 8192), torch.bfloat16, 95).to(dev()))
+    assert not o.rows64_swiglu_fusable(20, 8192) and not o.rows64_swiglu_fusable(16, 2048)
+    assert o.rows64_swiglu_fusable(17, 2048) and o.rows64_swiglu_fusable(32, 1024)
+    assert not o.rows64_swiglu_fusable(33, 2048)
+
+
+@pytest.mark.parametrize("M", [17, 24, 32])
+def test_steps_of_17_to_32_rows_through_linear(M):
+    """What the parts call: ``linear(..., accumulate=stream)`` of such a step adds to the
+    stream itself where the kernel pays (and says so), ``linear_swiglu`` takes rows that
+    await their norm; beyond 32 rows, or with a long K, the product comes back."""
+    o = ops()
+    N, K = 3072, 2048
+    w = rand((N, K), torch.bfloat16, 96)
+    x = rand((M, K), torch.bfloat16, 97)
+    base = rand((M, N), torch.float32, 98)
+    on_device = base.clone().to(dev())
+    o.form_log = []
+    try:
+        assert o.linear(x.to(dev()), w.to(dev()), partial_ok=True, accumulate=on_device) is None
+        log = o.form_log
+    finally:
+        o.form_log = None
+    assert log[-1]["added_to_stream"] and log[-1].get("kernel") == "rows64"
+    assert rel_err(on_device, base.double() + x.double() @ w.double().T) < F32_TOL
+    long_k = rand((256, 8192), torch.bfloat16, 99).to(dev())
+    kept = torch.zeros((M, 256), dtype=torch.float32, device=dev())
+    back = o.linear(rand((M, 8192), torch.bfloat16, 100).to(dev()), long_k, partial_ok=True, accumulate=kept)
+    assert back is not None and not kept.any()
+    stream = rand((M, K), torch.float32, 101) * 2.0
+    nw = 1.0 + rand((K,), torch.float32, 102)
+    normed = o.NormedRows(stream.to(dev()), nw.to(dev()), 1e-5, torch.bfloat16)
+    out = o.linear_swiglu(normed, w.to(dev()))
+    a, scale = _normed_operands(stream, nw, 1e-5)
+    gu = scale * (a @ w.double().T)
+    g, u = gu[:, :N // 2], gu[:, N // 2:]
+    assert rel_err(out, g / (1 + torch.exp(-g)) * u) < BF16_TOL
+    with pytest.raises(o.KernelError):                  # plain rows of such a step: not this call
+        o.linear_swiglu(x.to(dev()), w.to(dev()))
 
 
 def library_ranges(M, N, K):

@@ -244,6 +244,29 @@ def test_kernel_decode_forms_against_twins(M, N, K, bias):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K", [(20, 96, 1024), (32, 200, 2048), (64, 130, 1536), (17, 64, 4096)])
+def test_kernel_for_17_to_64_rows_against_the_twins(M, N, K):
+    """csrc/gemm_rows64.hip against the plain C++ functions: the norm twin followed by the
+    product's twin (the kernel rounds the operands once, as the norm kernel does, and scales
+    the sums), into the SwiGLU twin, and the product's twin plus the stream."""
+    o = ops()
+    res, nw = rand((M, K), 76, 2.0), 1.0 + rand((K,), 77, 0.3)
+    w = rand((N, K), 78, 0.05).to(torch.bfloat16)
+    _, normed = twin.add_rmsnorm(res, None, nw, 1e-5)
+    want = twin.linear(normed, w.float(), None)
+    x = o.NormedRows(res.to(dev()), nw.to(dev()), 1e-5, torch.bfloat16)
+    assert rel_err(o.linear_rows64(x, w.to(dev())), want) < BF16_TOL
+    assert rel_err(o.linear_rows64(x, w.to(dev()), mode=o.ROWS64_SWIGLU), twin.swiglu(want)) < BF16_TOL
+    a = rand((M, K), 79).to(torch.bfloat16)
+    stream = rand((M, N), 80)
+    on_device = stream.clone().to(dev())
+    o.linear_rows64(a.to(dev()), w.to(dev()), mode=o.ROWS64_ADD, accumulate=on_device,
+                    ksplit=2 if K >= 2048 else 1)
+    assert rel_err(on_device, stream + twin.linear(a.float(), w.float(), None)) < F32_TOL
+
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_kernel_embed_against_twin(dtype):
     table = rand((300, 72), 57).to(dtype)

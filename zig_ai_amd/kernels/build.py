@@ -27,8 +27,8 @@ from typing import Dict, Iterable, List, Optional
 PACKAGE_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC_DIR = os.path.join(PACKAGE_DIR, "csrc")
 ARCH = "gfx950"
-SOURCES = ("norm", "gemm", "rope_kv", "attention", "shortconv", "activation", "sampling", "blaslt",
-           "calibrate")
+SOURCES = ("norm", "gemm", "gemm_rows64", "rope_kv", "attention", "shortconv", "activation",
+           "sampling", "blaslt", "calibrate")
 HOST_SOURCES = ("host", "plain")    # plain C++, no device code: usable without a GPU or ROCm
 ALL_SOURCES = SOURCES + HOST_SOURCES
 CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden"]

@@ -73,6 +73,9 @@ _SIGNATURES = {
                                                  c_void_p, c_void_p, c_void_p, c_longlong,
                                                  c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                                  c_int, c_void_p],
+    ("gemm_rows64", "za_gemm_bf16_rows64"): [c_void_p, c_void_p, c_void_p, c_void_p, c_float,
+                                             c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                             c_void_p],
     ("sampling", "za_sample"): [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                 c_void_p, c_int, c_void_p],
     ("sampling", "za_repetition_penalty"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
@@ -521,6 +524,16 @@ def linear(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
         # workgroups would read rows of the stream while others add to them
         normed, x = None, x.materialise()
     splits = 1
+    if accumulate is not None and NORMED_ROWS_MAX_ROWS < M <= ROWS64_SWIGLU_ROWS and normed is None \
+            and bias is None and weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 \
+            and not force_tiled and rows64_add_splits(N, K):
+        # a step of 17 to 32 rows: the closing product of a mixer adds itself to the stream
+        # (so that the feed-forward's first product can run the norm, see above)
+        ks = rows64_add_splits(N, K)
+        linear_rows64(x, weight, ROWS64_ADD, accumulate, ks)
+        _note("linear", M=M, N=N, K=K, norm_in_product=False, added_to_stream=True,
+              partial_sums=1, out=accumulate.dtype, kernel="rows64")
+        return None
     if accumulate is not None:
         if weight.dtype == torch.bfloat16 and not force_tiled \
                 and (normed is not None or x.dtype == torch.bfloat16):
@@ -606,7 +619,8 @@ def linear(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
 def linear_swiglu(x, gate_up_weight: torch.Tensor) -> torch.Tensor:
     """``silu(x Wg^T) * (x Wu^T)`` for ``gate_up_weight = [Wg; Wu]`` of shape ``[2I, K]``
     and at most 16 rows of bfloat16 ``x`` (or a ``NormedRows``): the gate is applied to
-    the 32-bit accumulators, the ``[M, 2I]`` intermediate is never stored."""
+    the 32-bit accumulators, the ``[M, 2I]`` intermediate is never stored.  17 to
+    ``ROWS64_SWIGLU_ROWS`` rows are taken as ``NormedRows`` only (``rows64_swiglu_fusable``)."""
     if len(x.shape) != 2 or gate_up_weight.dim() != 2 or gate_up_weight.shape[0] % 2 \
             or gate_up_weight.shape[1] != x.shape[1]:
         raise KernelError(f"linear_swiglu takes x [M, K] and a weight [2I, K], got "
@@ -614,6 +628,14 @@ def linear_swiglu(x, gate_up_weight: torch.Tensor) -> torch.Tensor:
     M, K = x.shape
     I = gate_up_weight.shape[0] // 2
     _need(gate_up_weight, "gate_up_weight", torch.bfloat16)
+    if M > NORMED_ROWS_MAX_ROWS:
+        if not (isinstance(x, NormedRows) and x.dtype == torch.bfloat16
+                and rows64_swiglu_fusable(M, K)):
+            raise KernelError(f"linear_swiglu takes a step of {M} rows only as rows awaiting "
+                              f"their norm, up to {ROWS64_SWIGLU_ROWS} rows, got K={K}")
+        out = linear_rows64(x, gate_up_weight, ROWS64_SWIGLU)
+        _note("linear_swiglu", M=M, N=2 * I, K=K, norm_in_product=True, kernel="rows64")
+        return out
     normed = None
     if isinstance(x, NormedRows):
         if _takes_normed_rows(x, gate_up_weight, M, K):
@@ -636,6 +658,99 @@ def linear_swiglu(x, gate_up_weight: torch.Tensor) -> torch.Tensor:
     _check(rc, "linear_swiglu", f"M={M} I={I} K={K}")
     _note("linear_swiglu", M=M, N=2 * I, K=K, norm_in_product=normed is not None)
     return out
+
+
+# ------------------------------------------ products of 17 to 64 rows, fused forms
+ROWS64_MAX_ROWS = 64
+ROWS64_K_MULTIPLE = 512        # a workgroup's range of K: spans of 512, at least two
+ROWS64_STORE, ROWS64_SWIGLU, ROWS64_ADD = 0, 1, 2
+
+
+def rows64_takes(M: int, K: int, ksplit: int = 1) -> bool:
+    """Whether ``linear_rows64`` takes a product of ``M`` rows over ``K`` in ``ksplit`` ranges."""
+    return (1 <= M <= ROWS64_MAX_ROWS and ksplit >= 1 and K % ksplit == 0
+            and (K // ksplit) % ROWS64_K_MULTIPLE == 0 and K // ksplit >= 2 * ROWS64_K_MULTIPLE)
+
+
+# Where the kernel of csrc/gemm_rows64.hip is taken, by measurement (one MI355X, replayed
+# from graphs, weights from memory, against the norm kernel + the library's product + the
+# SwiGLU kernel): the fused norm + gate|up + SwiGLU of 2 x 8192 x 2048 takes 19.5-19.9 us at
+# 17 to 32 rows against 24.8-25.8, 22.8-23.9 at 40-48 rows against 25.6, 25.5 at 64 rows
+# against 25.9; the plain forms lose (norm + in_proj 15.3 against 13.2 at 24 rows, w2 added
+# to the stream 12.7-14.5 against the library's 10.3).  So it serves the feed-forward's
+# first product up to ROWS64_SWIGLU_ROWS rows, which needs the stream complete before it,
+# and therefore the mixer's closing product of such a step, added to the stream with
+# atomics (2048 x 2048: 8.6-9.4 us against the library's 6.6-8.8, without the stack of
+# partial sums that the norm kernel would have to add).
+ROWS64_SWIGLU_ROWS = 32
+ROWS64_ADD_MAX_K = 4096
+ROWS64_ADD_MIN_WORKGROUPS = 48
+
+
+def rows64_add_splits(N: int, K: int) -> int:
+    """Into how many ranges K is cut when a product of 17 to 64 rows is added to the stream
+    by the kernel of csrc/gemm_rows64.hip: as many as keep a range at 1,024 elements or
+    more (two spans).  0: the kernel is not taken (no cut fits, too few workgroups to pay,
+    or a K beyond what was measured to pay)."""
+    if K > ROWS64_ADD_MAX_K:
+        return 0
+    tiles = (N + 63) // 64
+    best = 0
+    for split in (1, 2, 3, 4):
+        if rows64_takes(1, K, split):
+            best = split
+    if best == 0 or tiles * best < ROWS64_ADD_MIN_WORKGROUPS:
+        return 0
+    return best
+
+
+def rows64_swiglu_fusable(rows: int, width: int) -> bool:
+    """Whether a step of ``rows`` rows takes the fused norm + gate|up + SwiGLU kernel for
+    17 to 64 rows (``linear_swiglu`` with a ``NormedRows``)."""
+    return (NORMED_ROWS_MAX_ROWS < rows <= ROWS64_SWIGLU_ROWS and width <= NORMED_ROWS_MAX_K
+            and rows64_takes(rows, width))
+
+
+def linear_rows64(x, weight: torch.Tensor, mode: int = ROWS64_STORE,
+                  accumulate: Optional[torch.Tensor] = None, ksplit: int = 1) -> Optional[torch.Tensor]:
+    """A product of at most 64 rows on the kernel of csrc/gemm_rows64.hip.  ``x``: bfloat16
+    ``[M, K]`` or a ``NormedRows`` (the kernel then runs the norm).  ``mode``:
+    ``ROWS64_STORE`` (``x W^T`` as bfloat16), ``ROWS64_SWIGLU`` (``weight = [Wg; Wu]``:
+    ``silu(x Wg^T) * (x Wu^T)`` as bfloat16) or ``ROWS64_ADD`` (``x W^T`` added to the 32-bit
+    ``accumulate [M, N]`` with atomics, K in ``ksplit`` ranges; returns ``None``)."""
+    if len(x.shape) != 2 or weight.dim() != 2 or weight.shape[1] != x.shape[1]:
+        raise KernelError(f"linear_rows64 takes x [M, K] and a weight [N, K], got {tuple(x.shape)} "
+                          f"and {tuple(weight.shape)}")
+    M, K = x.shape
+    _need(weight, "weight", torch.bfloat16)
+    N = weight.shape[0]
+    if mode == ROWS64_SWIGLU:
+        if N % 2:
+            raise KernelError("a fused gate|up weight has an even number of rows")
+        N //= 2
+    if not rows64_takes(M, K, ksplit) or (ksplit > 1 and mode != ROWS64_ADD):
+        raise KernelError(f"linear_rows64 takes at most {ROWS64_MAX_ROWS} rows and ranges of K that "
+                          f"are multiples of {ROWS64_K_MULTIPLE}, got M={M} K={K} in {ksplit} ranges")
+    normed = x if isinstance(x, NormedRows) else None
+    if normed is not None:
+        if mode == ROWS64_ADD or normed.dtype != torch.bfloat16:
+            raise KernelError("the kernel runs the norm only for bfloat16 products that it stores")
+    else:
+        _need(x, "x", torch.bfloat16)
+    if mode == ROWS64_ADD:
+        _need(accumulate, "accumulate", torch.float32, (M, N))
+        out = accumulate
+    else:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=weight.device)
+    rc = _fn("gemm_rows64", "za_gemm_bf16_rows64")(
+        None if normed is not None else _ptr(x),
+        _ptr(normed.residual) if normed is not None else None,
+        _ptr(normed.rows) if normed is not None else None,
+        _ptr(normed.weight) if normed is not None else None,
+        normed.eps if normed is not None else 0.0,
+        _ptr(weight), _ptr(out), int(mode), M, N, K, int(ksplit), _stream())
+    _check(rc, "gemm_bf16_rows64", f"M={M} N={N} K={K} mode={mode} ksplit={ksplit}")
+    return None if mode == ROWS64_ADD else out
 
 
 # ------------------------------------------------------------ rope + kv write

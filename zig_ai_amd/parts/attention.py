@@ -64,7 +64,7 @@ class GroupedQueryAttention(Mixer):
     kind = "gqa_attention"
     graph_safe = True
     takes_stream = True
-    kernel_sources = ("gemm", "rope_kv", "attention", "norm")
+    kernel_sources = ("gemm", "gemm_rows64", "rope_kv", "attention", "norm")
 
     @classmethod
     def tensor_rules(cls, params: Mapping[str, Any]) -> Dict[str, TensorRule]:

@@ -154,6 +154,7 @@ class Mixer(Part):
 
 class FeedForward(Part):
     takes_stream = False      # as for Mixer
+    opens_with_swiglu = False  # its first product is ``ops.linear_swiglu`` on what it is handed
 
     def forward(self, x: torch.Tensor, step) -> torch.Tensor:
         raise NotImplementedError
@@ -182,10 +183,13 @@ class Norm(Part):
         return self.forward(residual)
 
 
-    def deferred(self, residual: torch.Tensor, rows: Optional[torch.Tensor] = None):
+    def deferred(self, residual: torch.Tensor, rows: Optional[torch.Tensor] = None,
+                 swiglu: bool = False):
         """The norm of ``residual`` (of its ``rows``) as something a part with
         ``takes_stream`` accepts in place of activations, without running it now; or
-        ``None`` when this norm, or this step, has no such form."""
+        ``None`` when this norm, or this step, has no such form.  ``swiglu``: the part
+        says that its first product is a fused gate|up with its gate (``Part.opens_with_swiglu``),
+        for which more row counts have a fused form."""
         return None
 
 

@@ -48,7 +48,10 @@ def apply_normed(norm, part, residual: torch.Tensor, pending: Optional[torch.Ten
     afterwards, or ``None`` when the part has added it already."""
     if not getattr(part, "takes_stream", False):
         return part.forward(norm.add_forward(residual, pending), *args)
-    x = norm.deferred(residual) if pending is None else None
+    x = None
+    if pending is None:
+        x = norm.deferred(residual, swiglu=True) if getattr(part, "opens_with_swiglu", False) \
+            else norm.deferred(residual)
     if x is None:
         x = norm.add_forward(residual, pending)
     runtime = getattr(part, "runtime", None)

@@ -25,7 +25,8 @@ class SwiGLU(FeedForward):
     kind = "swiglu"
     graph_safe = True
     takes_stream = True
-    kernel_sources = ("gemm", "activation")
+    opens_with_swiglu = True
+    kernel_sources = ("gemm", "gemm_rows64", "activation")
 
     @classmethod
     def tensor_rules(cls, params: Mapping[str, Any]) -> Dict[str, TensorRule]:
@@ -41,9 +42,12 @@ class SwiGLU(FeedForward):
         ops.check_projection_weight(self.down, "feed_forward down")
 
     def forward(self, x, step=None, stream: Optional[torch.Tensor] = None):
-        if x.shape[0] <= 16 and x.dtype == torch.bfloat16 and self.gate_up.dtype == torch.bfloat16 \
-                and x.shape[1] <= 8192:
+        bf16 = x.dtype == torch.bfloat16 and self.gate_up.dtype == torch.bfloat16
+        if bf16 and x.shape[0] <= 16 and x.shape[1] <= 8192:
             # a decode batch: the gate is applied to the projection's accumulators
+            a = ops.linear_swiglu(x, self.gate_up)
+        elif bf16 and isinstance(x, ops.NormedRows) and ops.rows64_swiglu_fusable(*x.shape):
+            # 17 to 32 rows whose norm has not run: norm, product and gate in one kernel
             a = ops.linear_swiglu(x, self.gate_up)
         else:
             if isinstance(x, ops.NormedRows):

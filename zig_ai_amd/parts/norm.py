@@ -41,10 +41,16 @@ class RMSNorm(Norm):
                     rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         return ops.add_rmsnorm(residual, delta, self.weight, self.eps, self.runtime.dtype, rows=rows)
 
-    def deferred(self, residual: torch.Tensor, rows: Optional[torch.Tensor] = None):
+    def deferred(self, residual: torch.Tensor, rows: Optional[torch.Tensor] = None,
+                 swiglu: bool = False):
+        """``swiglu``: the part that takes the rows starts with a fused gate|up product
+        (which also has a form for 17 to 32 rows)."""
         # a decode batch in bfloat16: the projection that follows normalises the rows
         n = residual.shape[0] if rows is None else rows.numel()
-        if self.runtime.dtype != torch.bfloat16 or not ops.normed_rows_fusable(n, self.width):
+        if self.runtime.dtype != torch.bfloat16:
+            return None
+        if not (ops.normed_rows_fusable(n, self.width)
+                or (swiglu and ops.rows64_swiglu_fusable(n, self.width))):
             return None
         return ops.NormedRows(residual, self.weight, self.eps, self.runtime.dtype, rows)
 

@@ -25,7 +25,7 @@ class ShortConv(Mixer):
     kind = "short_conv"
     graph_safe = True
     takes_stream = True
-    kernel_sources = ("gemm", "shortconv")
+    kernel_sources = ("gemm", "gemm_rows64", "shortconv")
 
     @classmethod
     def tensor_rules(cls, params: Mapping[str, Any]) -> Dict[str, TensorRule]:
