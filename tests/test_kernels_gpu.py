@@ -973,6 +973,64 @@ def test_attention_over_long_contexts(window):
         assert rel_err(out, expect[-m:]) < BF16_TOL, (keys, nsplit)
 
 
+@pytest.mark.parametrize("nh,nkv,d,requests", [(16, 8, 64, 49), (4, 2, 128, 6), (8, 8, 128, 50)])
+def test_decode_attention_beyond_4096_keys_uncut(nh, nkv, d, requests):
+    """The decode kernel fetches the block-table entries of sixteen tiles a wave at once and
+    fetches again when they are used up: with four waves a workgroup (the form taken when
+    requests x key/value heads fill the chip, here 392 and 400 workgroups) that is after
+    4,096 keys of an uncut context, with eight after 8,192.  Contexts of 4,900 to 9,000 keys,
+    uncut; one key before and one behind the place of the second fetch are made to
+    dominate a query each, so that a tile read through a stale or misplaced entry shows."""
+    ps = 16
+    ctx = 9000 if requests < 10 else 4900
+    total = ctx + requests
+    k = rand((total, nkv, d), torch.bfloat16, 110)
+    v = rand((total, nkv, d), torch.bfloat16, 111)
+    q = rand((requests, nh, d), torch.bfloat16, 112)
+    near, far = 100, ctx - 300                 # (far lies behind every fetch but the last)
+    for key, row, elem in ((near, 0, 3), (far, 1, 5)):
+        k[key] = 0
+        k[key, :, elem] = 16.0
+        q[row] = 0
+        q[row, :, elem] = 16.0                 # score 32 / sqrt(d) x 8 against N(0, 4)
+    cache, table = paged_from_dense([k], [v], ps, torch.bfloat16, seed=12)
+    positions = torch.arange(ctx, ctx + requests, dtype=torch.int32)
+    expect = light_attention(q, k, v, positions.long(), 0)
+    group = nh // nkv
+    assert float((expect[0] - v[near].double().repeat_interleave(group, 0)).abs().max()) < 0.05
+    assert float((expect[1] - v[far].double().repeat_interleave(group, 0)).abs().max()) < 0.05
+    tables = table.repeat(requests, 1).to(dev())
+    out = ops().paged_attention_decode_mfma(q.to(dev()), cache.to(dev()), tables, positions.to(dev()),
+                                            None, None, None, requests, 1.0 / math.sqrt(d), 0, 0, 1)
+    assert rel_err(out, expect) < BF16_TOL
+
+
+@pytest.mark.parametrize("keys_per_split,nsplit", [(0, 1), (1024, 12), (512, 24)])
+def test_rope_attention_decode_beyond_8192_keys(keys_per_split, nsplit):
+    """The attention that prepares its own token, far into long contexts (the second fetch of
+    table entries, the token's own place in a late tile): the bits of the two kernels it
+    replaces, in the result and in the cache, uncut and in ranges."""
+    o = ops()
+    nh, nkv, d, page_size = 8, 2, 64, 16
+    positions = [8191, 8192, 8300, 9001, 12000]
+    qkv, cache, table, pos, slots = decode_step_case(nh, nkv, d, page_size, positions, 1200)
+    T = len(positions)
+    qw = (rand((d,), torch.float32, 1201) * 0.3 + 1.0).to(dev())
+    kw = (rand((d,), torch.float32, 1202) * 0.3 + 1.0).to(dev())
+    inv = (1.0 / torch.pow(torch.tensor(1e6, dtype=torch.float64),
+                           2.0 * torch.arange(0, d // 2, dtype=torch.float64) / d)).float().to(dev())
+    eps, scale = 1e-5, 1.0 / math.sqrt(d)
+    two = cache.clone()
+    q = o.qk_norm_rope_kv_write(qkv, pos, slots, qw, kw, inv, two, nh, nkv, d, d, False, eps)
+    want = o.paged_attention_decode_mfma(q, two, table, pos, None, None, None, T, scale, 0,
+                                         keys_per_split, nsplit)
+    one = cache.clone()
+    got = o.rope_attention_decode(qkv, pos, slots, qw, kw, inv, one, table, nh, eps, scale, 0,
+                                  keys_per_split, nsplit)
+    assert torch.equal(one, two) and not torch.equal(one, cache)
+    assert torch.equal(got, want)
+
+
 def test_single_token_attention_returns_value():
     """One key: the softmax is 1 and the output is V (derived, but only checked for
     finiteness, in /root/reference/src/transformer/hybrid_attn.zig:1207-1212)."""

@@ -42,8 +42,11 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--seed", type=int, default=42, help="seed of the sampling streams (default 42)")
     ap.add_argument("-b", "--batch-size", type=int, default=2048,
                     help="token budget of one step (default 2048)")
-    ap.add_argument("-ub", "--ubatch-size", type=int, default=512,
-                    help="largest portion of one prompt in a step (default 512)")
+    ap.add_argument("-ub", "--ubatch-size", type=int, default=2048,
+                    help="largest portion of one prompt in a step (default 2048, the step's "
+                         "whole budget; the reference's own default of 512 reads every weight "
+                         "four times per 2,048 prompt tokens: 8.5 ms instead of 5.0 on the "
+                         "LFM2-1.2B shape)")
     ap.add_argument("-np", type=int, default=1, dest="num_parallel",
                     help="run the prompt as this many parallel requests (default 1)")
     ap.add_argument("--backend", choices=["auto", "gpu", "cpu"], default="auto",

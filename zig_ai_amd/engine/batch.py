@@ -109,10 +109,10 @@ class PreparedEntries:
             self.counts[s] = len(e.tokens)
             self.want_counts[s] = len(e.want)
         try:
-            tokens = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64,
-                                 count=int(self.counts.sum()))
-            wants = np.fromiter((w for e in entries for w in e.want), dtype=np.int64,
-                                count=int(self.want_counts.sum()))
+            # (a list of integers becomes an array at some 20 ns an element; a generator
+            # over the tokens of a long portion costs five times that)
+            tokens = self._integers([e.tokens for e in entries], int(self.counts.sum()))
+            wants = self._integers([e.want for e in entries], int(self.want_counts.sum()))
         except (TypeError, ValueError, OverflowError) as err:
             raise StepError(f"token ids and wanted places must be integers: {err}") from err
         if tokens.size and (tokens.min() < 0 or tokens.max() >= vocab_size):
@@ -126,6 +126,23 @@ class PreparedEntries:
         self.ctx = np.empty((S,), dtype=np.int32)
         self.slots = np.empty((S,), dtype=np.int32)
         self.meta = np.zeros((6,), dtype=np.int64)
+
+    @staticmethod
+    def _integers(parts: Sequence[Sequence[int]], total: int) -> np.ndarray:
+        out = np.empty((total,), dtype=np.int64)
+        at = 0
+        for p in parts:
+            n = len(p)
+            if n:
+                a = np.asarray(p)
+                if a.dtype.kind not in "iu" or a.shape != (n,):
+                    if a.dtype.kind == "b" or a.shape != (n,) or \
+                            not all(isinstance(v, (int, np.integer)) and not isinstance(v, bool) for v in p):
+                        raise TypeError(f"not integers: {p!r:.60}")
+                    a = np.asarray([int(v) for v in p], dtype=np.int64)
+                out[at:at + n] = a
+                at += n
+        return out
 
     def build(self, cache: CacheManager, grans: np.ndarray, max_position: int, min_pages: int,
               sections: np.ndarray, out_ptr, cap: int) -> None:
@@ -145,11 +162,43 @@ class PreparedEntries:
         raise_for(rc)
 
 
+class StagingRing:
+    """A few pinned host buffers that take turns: a step is laid out in one of them and
+    goes to the device by a copy that does not block, so the host can lay out and issue the
+    next step while this one still runs (a copy from ordinary memory makes the host wait
+    for everything issued before it).  A buffer is used again only after its copy has
+    finished (an event per buffer)."""
+
+    def __init__(self, buffers: int = 4, words: int = 1 << 14):
+        self._buffers: List[Optional[torch.Tensor]] = [None] * buffers
+        self._events: List[Optional[torch.cuda.Event]] = [None] * buffers
+        self._words = words
+        self._at = -1
+
+    def take(self, words: int) -> torch.Tensor:
+        """A pinned int32 buffer of at least ``words`` entries, free to be written."""
+        self._at = (self._at + 1) % len(self._buffers)
+        ev = self._events[self._at]
+        if ev is not None:
+            ev.synchronize()
+        buf = self._buffers[self._at]
+        if buf is None or buf.numel() < words:
+            buf = torch.empty((max(self._words, 2 * words),), dtype=torch.int32, pin_memory=True)
+            self._buffers[self._at] = buf
+        return buf
+
+    def copied(self) -> None:
+        """The copy out of the buffer taken last has been issued on the current stream."""
+        if self._events[self._at] is None:
+            self._events[self._at] = torch.cuda.Event()
+        self._events[self._at].record()
+
+
 def build_step(entries: Sequence[StepEntry], cache: CacheManager, device: torch.device,
                vocab_size: int, item_granularities: Sequence[int] = (),
                max_position: int = 0, min_pages: int = 0, max_keys: int = 0,
                into: Optional[torch.Tensor] = None,
-               staging: Optional[torch.Tensor] = None,
+               staging=None,
                prepared: Optional[PreparedEntries] = None) -> StepContext:
     """Lay out the step.  Every request must be admitted and its pages for this
     step reserved beforehand; nothing is committed here.
@@ -161,7 +210,9 @@ def build_step(entries: Sequence[StepEntry], cache: CacheManager, device: torch.
     find every array at the address it was captured with.  ``staging`` is a pinned
     host buffer to lay the step out in, from which ``into`` is filled by a copy
     that does not block; the caller waits for that copy before it lays out the
-    next step there.  ``prepared``: the same entries, already turned into arrays."""
+    next step there; a ``StagingRing`` in its place hands out such buffers in turn and a new
+    device buffer is filled from them.  ``prepared``: the same entries, already turned
+    into arrays."""
     prep = prepared if prepared is not None else PreparedEntries(entries, cache, vocab_size)
     S = len(entries)
     counts, meta = prep.counts, prep.meta
@@ -175,6 +226,9 @@ def build_step(entries: Sequence[StepEntry], cache: CacheManager, device: torch.
         prep.build(cache, grans, max_position, min_pages, sections, out_ptr, cap)
 
     call(None, 0)                               # sizes first, then the buffer itself
+    ring = staging if isinstance(staging, StagingRing) else None
+    if ring is not None:
+        staging = ring.take(int(meta[5]))
     if staging is not None:
         if staging.numel() < int(meta[5]) or staging.dtype != torch.int32:
             raise StepError(f"the step needs {int(meta[5])} int32 entries, the staging buffer "
@@ -193,7 +247,11 @@ def build_step(entries: Sequence[StepEntry], cache: CacheManager, device: torch.
     seq_lens, ctx_lens, slots = counts.tolist(), ctx_arr.tolist(), slot_arr.tolist()
     item_lists = {gran: offsets[f"iseq{gran}"][1] for gran in grans.tolist()}
 
-    if into is None:
+    if into is None and ring is not None:
+        dev = torch.empty((host.size,), dtype=torch.int32, device=device)
+        dev.copy_(staging[:host.size], non_blocking=True)
+        ring.copied()
+    elif into is None:
         dev = torch.from_numpy(host).to(device)
     else:
         if into.numel() < host.size or into.dtype != torch.int32:

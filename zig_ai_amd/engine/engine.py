@@ -25,7 +25,7 @@ from .scheduler import RUNNING, Request, ScheduledEntry, Scheduler
 class Engine:
     def __init__(self, model_dir, dtype: str = "bfloat16", page_size: int = 16,
                  num_pages: Optional[int] = None, max_num_seqs: int = 64,
-                 max_num_batched_tokens: int = 2048, chunk_size: int = 512,
+                 max_num_batched_tokens: int = 2048, chunk_size: int = 2048,
                  max_model_len: Optional[int] = None, use_graphs: bool = True,
                  portion_graphs: bool = False,
                  on_step=None, memory_fraction: float = 0.85, multi_step: int = 8,

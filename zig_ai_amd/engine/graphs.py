@@ -33,6 +33,12 @@ PAGE_BUCKET = 64        # block-table width is rounded up to a multiple of this
 KEYS_BUCKET = 1024      # and the longest context to a multiple of this
 MAX_GRAPHS = 96         # recorded shapes kept; the one replayed longest ago goes first
 MAX_PORTION_GRAPHS = 24 # the same for steps with prompt portions (their tensors are larger)
+# Steps with prompt portions are recorded only where the host is the limit (beyond some
+# 1,000 tokens a step is bound by the GPU and a recording would only hold memory), and
+# the recorded steps together hold at most this many bytes of intermediate tensors: the
+# one replayed longest ago goes first.
+PORTION_GRAPH_MAX_TOKENS = 1024
+PORTION_GRAPH_BYTES = 2 << 30
 
 
 def _round_up(n: int, m: int) -> int:
@@ -230,6 +236,10 @@ class DecodeGraphs:
         back cost nothing), every later one is a replay."""
         cache, model = runner.cache, runner.model
         prepared = PreparedEntries(entries, cache, self._vocab)
+        if int(prepared.counts.sum()) > PORTION_GRAPH_MAX_TOKENS:
+            ctx = build_step(entries, cache, runner.device, self._vocab, self._granularities,
+                             self._max_position, prepared=prepared, staging=runner.staging)
+            return model.forward(ctx, runner.views)
         grans = np.asarray(sorted(set(int(g) for g in self._granularities)), dtype=np.int32)
         sections = np.zeros((2 * (7 + 2 * len(cache.groups) + 3 * len(grans)),), dtype=np.int64)
         prepared.build(cache, grans, self._max_position, 0, sections, None, 0)     # sizes only
@@ -241,9 +251,9 @@ class DecodeGraphs:
             if len(self.portion_entries) >= 4 * MAX_PORTION_GRAPHS:    # sightings are cheap, not free
                 for old in [k for k, v in self.portion_entries.items() if v["graph"] is None][:MAX_PORTION_GRAPHS]:
                     self.portion_entries.pop(old)
-            self.portion_entries[key] = {"graph": None, "seen": 1}
+            self.portion_entries[key] = {"graph": None, "seen": 1, "bytes": 0}
             ctx = build_step(entries, cache, runner.device, self._vocab, self._granularities,
-                             self._max_position, prepared=prepared)
+                             self._max_position, prepared=prepared, staging=runner.staging)
             return model.forward(ctx, runner.views)
         self.portion_entries[key] = self.portion_entries.pop(key)      # now the most recently used
         if slot["graph"] is None:
@@ -251,9 +261,10 @@ class DecodeGraphs:
                                self._max_position, min_pages=key[2], max_keys=key[3], prepared=prepared)
             words = probe.host.size
             recorded = [k for k, v in self.portion_entries.items() if v["graph"] is not None]
-            if len(recorded) >= MAX_PORTION_GRAPHS:
+            held = sum(self.portion_entries[k]["bytes"] for k in recorded)
+            while recorded and (len(recorded) >= MAX_PORTION_GRAPHS or held > PORTION_GRAPH_BYTES):
                 torch.cuda.current_stream().synchronize()    # its last replay may still run
-                self.portion_entries.pop(recorded[0])
+                held -= self.portion_entries.pop(recorded.pop(0))["bytes"]
             slot.update(buffer=torch.full((words,), -1, dtype=torch.int32, device=runner.device),
                         pinned=torch.empty((words,), dtype=torch.int32, pin_memory=True),
                         copied=None, words=words)
@@ -263,6 +274,7 @@ class DecodeGraphs:
             graph = torch.cuda.CUDAGraph()
             was_enabled = gc.isenabled()
             gc.disable()
+            before = torch.cuda.memory_reserved(runner.device)
             try:
                 with torch.cuda.graph(graph):                  # recorded, not executed
                     slot["logits"] = model.forward(ctx, runner.views)
@@ -270,6 +282,8 @@ class DecodeGraphs:
                 if was_enabled:
                     gc.enable()
             slot["graph"] = graph
+            # what the recording holds for good: its pool of intermediate tensors
+            slot["bytes"] = max(0, torch.cuda.memory_reserved(runner.device) - before) + 8 * words
             self.portion_captures += 1
         else:
             if slot["copied"] is not None:

@@ -19,7 +19,7 @@ from typing import Callable, Hashable, List, Optional, Sequence
 import torch
 
 from ..cache.pages import OutOfPages
-from .batch import StepContext, StepEntry, StepError, build_step
+from .batch import StagingRing, StepContext, StepEntry, StepError, build_step
 from .graphs import DecodeGraphs
 from .model import DecoderModel
 
@@ -35,6 +35,8 @@ class ModelRunner:
         self.cache = model.make_cache(page_size, num_pages, num_slots)
         self.views = model.cache_views(self.cache)
         self.steps_run = 0
+        # steps are laid out in pinned memory and copied without the host waiting
+        self.staging = StagingRing() if self.device.type == "cuda" else None
         self.portion_graphs = bool(portion_graphs)
         self.graphs = (DecodeGraphs(model.spec.vocab_size, model.item_granularities, model.spec.max_position)
                        if (use_graphs and model.graph_safe) else None)
@@ -61,7 +63,8 @@ class ModelRunner:
         """Reserve pages for the entries and lay out the step."""
         self.reserve(entries)
         return build_step(entries, self.cache, self.device, self.model.spec.vocab_size,
-                          self.model.item_granularities, self.model.spec.max_position)
+                          self.model.item_granularities, self.model.spec.max_position,
+                          staging=self.staging)
 
     def step(self, entries: Sequence[StepEntry],
              taps: Optional[list] = None) -> torch.Tensor:

@@ -90,7 +90,7 @@ class Scheduler:
     _REASONS = (None, "eos", "length", "max_model_len")
 
     def __init__(self, cache: CacheManager, max_num_seqs: int = 64,
-                 max_num_batched_tokens: int = 2048, chunk_size: int = 512,
+                 max_num_batched_tokens: int = 2048, chunk_size: int = 2048,
                  max_model_len: int = 0):
         if max_num_batched_tokens < 1 or chunk_size < 1 or max_num_seqs < 1:
             raise ValueError("max_num_seqs, max_num_batched_tokens and chunk_size must be >= 1")
