@@ -20,8 +20,9 @@ at contexts of 4,096 and 8,192 tokens and batch 64 at 4,096 stand too.  Further 
 of 8,192), and ``calibration``: what this GPU does at best, measured here (a kernel that
 only reads 1 GiB; matrix-core instructions issued back to back), with every fraction also
 given against those (``frac_measured``).  ``--phase prefill|decode`` runs that phase alone
-for a profiler: no calibration kernels, and the GEMM library's first answer for every
-shape (no timing of candidates, which allocates, frees and waits inside the first steps).
+for a profiler: no calibration kernels, the GEMM library's first answer for every
+shape (no timing of candidates, which allocates, frees and waits inside the first steps),
+and weights drawn with one kernel a tensor (other values than the default run's).
 The model is ``DecoderModel.from_random(cfg, seed=0)``: the tensors that
 ``write_random_model(cfg, folder, seed=0)`` stores, drawn on the device.
 """
@@ -208,9 +209,12 @@ def main() -> int:
 
         def __init__(self, cfg):
             self.cfg = cfg
-            # (a profiled phase takes the library's first answer for every shape)
+            # (a profiled phase takes the library's first answer for every shape, and its
+            # weights are drawn with one kernel a tensor: a profiler's counter mode runs
+            # every kernel alone, and the keyed generator is some 19,000 small ones)
             self.model = DecoderModel.from_random(cfg, seed=0, dtype="bfloat16",
-                                                  library_tuning=False if profiled else None)
+                                                  library_tuning=False if profiled else None,
+                                                  quick=profiled)
             self.vocab = cfg["vocab_size"]
             self.n_attn = sum(1 for k in cfg["layer_types"] if k != "conv")
             self.hd = cfg["hidden_size"] // cfg["num_attention_heads"]

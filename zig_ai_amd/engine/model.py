@@ -168,12 +168,13 @@ class DecoderModel:
                     device: Optional[torch.device] = None, std: float = 0.02,
                     norm_init: str = "ones", reproducible: bool = False,
                     role_std: Optional[Mapping[str, float]] = None,
-                    library_tuning: Optional[bool] = None):
+                    library_tuning: Optional[bool] = None, quick: bool = False):
         """The model that ``write_random_model(config, folder, seed, ...)`` followed by
         ``from_folder`` gives, without the trip through a file: every tensor is drawn on the
         device by the same keyed generator (a value depends on seed, tensor name and element
         index only) and kept as the loader would keep it.  ``config`` is a typed
-        configuration or a config.json dictionary."""
+        configuration or a config.json dictionary.  ``quick``: see ``random_tensor`` (other
+        values than the folder's, drawn with one kernel a tensor)."""
         from ..config import config_from_dict
         from ..weights.loader import expected_tensors, keep_dtype
         from ..weights.random_init import deviation_of, random_tensor
@@ -188,7 +189,7 @@ class DecoderModel:
             stored = random_tensor(seed, exp.names[0], exp.rule.stored_shape or exp.rule.shapes[0],
                                    exp.rule.role, rt.dtype,
                                    deviation_of(exp.names[0], exp.rule.role, std, role_std or {}),
-                                   norm_init, device)
+                                   norm_init, device, quick=quick)
             kept = keep_dtype(stored.dtype, exp.rule.role, rt.dtype)
             tensors.setdefault(exp.owner, {})[exp.local] = \
                 stored.reshape(exp.rule.shapes[0]).to(kept).contiguous()

@@ -88,15 +88,25 @@ def keyed_normal(seed: int, name: str, numel: int, device="cpu",
 
 
 def random_tensor(seed: int, name: str, shape, role: str, dtype: torch.dtype, std: float,
-                  norm_init: str, device="cpu") -> torch.Tensor:
+                  norm_init: str, device="cpu", quick: bool = False) -> torch.Tensor:
     """One tensor of a random model: N(0, std) from ``keyed_normal``; norm weights are 1,
-    N(0, std) or 1 + N(0, std) by ``norm_init``.  Drawn in 32-bit, rounded to ``dtype``."""
+    N(0, std) or 1 + N(0, std) by ``norm_init``.  Drawn in 32-bit, rounded to ``dtype``.
+    ``quick``: the deviates come from the tensor library's own generator instead, one
+    kernel a tensor (seeded by seed and name, but NOT the values a model folder of this
+    seed holds): for runs under a profiler's counters, which run every kernel alone, and
+    the keyed generator is some hundred small kernels per 16 million values."""
     n = 1
     for d in shape:
         n *= int(d)
     if role == "norm" and norm_init == "ones":
         return torch.ones(tuple(shape), dtype=dtype, device=device)
-    t = keyed_normal(seed, name, n, device).reshape(tuple(shape)) * float(std)
+    if quick:
+        g = torch.Generator(device=device)
+        g.manual_seed(tensor_key(seed, name)[0] & 0x7FFFFFFF)
+        t = torch.empty((n,), dtype=torch.float32, device=device).normal_(generator=g)
+        t = t.reshape(tuple(shape)) * float(std)
+    else:
+        t = keyed_normal(seed, name, n, device).reshape(tuple(shape)) * float(std)
     if role == "norm" and norm_init == "around_one":
         t = t + 1.0
     return t.to(dtype)
