@@ -450,6 +450,28 @@ def test_gemm_bf16_decode_rows_added_to_the_stream(M, N, K):
     assert back is not None and not kept.any()
 
 
+@pytest.mark.parametrize("src_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dst_dtype", [torch.float32, torch.bfloat16])
+def test_copy_columns(src_dtype, dst_dtype):
+    """Columns of a matrix's rows into a new tensor or into columns of another: exact when
+    the types agree or widen, one rounding when they narrow; everything else untouched."""
+    o = ops()
+    src = rand((37, 100), src_dtype, 120)
+    part = o.copy_columns(src.to(dev()), 13, 50, dtype=dst_dtype)
+    assert part.shape == (37, 50) and part.dtype == dst_dtype
+    assert torch.equal(part.cpu(), src[:, 13:63].to(dst_dtype))
+    out = rand((37, 77), dst_dtype, 121)
+    on_device = out.clone().to(dev())
+    assert o.copy_columns(src.to(dev()), 90, 10, on_device, 60) is on_device
+    want = out.clone()
+    want[:, 60:70] = src[:, 90:100].to(dst_dtype)
+    assert torch.equal(on_device.cpu(), want)
+    with pytest.raises(o.KernelError):
+        o.copy_columns(src.to(dev()), 95, 10)
+    with pytest.raises(o.KernelError):
+        o.copy_columns(src.to(dev()), 0, 10, on_device, 70)
+
+
 # ------------------------------------------------- products of 17 to 64 rows, fused forms
 @pytest.mark.parametrize("M", [1, 5, 17, 20, 32, 33, 47, 64])
 @pytest.mark.parametrize("N,K", [(50, 1024), (200, 1536), (6144, 2048), (130, 4096), (64, 2560)])

@@ -84,3 +84,39 @@ extern "C" int za_cast(const void* in, int in_dtype, void* out, int out_dtype, l
     return ZA_ERR_UNSUPPORTED;
   return za_launch_status();
 }
+
+// Columns [col0, col0 + ncols) of every row of `in` [rows, in_width] into columns
+// [out_col0, out_col0 + ncols) of `out` [rows, out_width], converted between the two
+// storage types: how a mixer takes q, k and v out of a fused projection's rows and puts
+// them back side by side, without the tensor library.
+template <typename TI, typename TO>
+__global__ void __launch_bounds__(256)
+copy_columns_kernel(const TI* __restrict__ in, TO* __restrict__ out, int in_width, int col0,
+                    int out_width, int out_col0, int ncols, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t row = idx / ncols;
+  const int c = (int)(idx % ncols);
+  out[row * out_width + out_col0 + c] = from_f32<TO>(to_f32<TI>(in[row * in_width + col0 + c]));
+}
+
+extern "C" int za_copy_columns(const void* in, int in_dtype, int in_width, int col0, void* out,
+                               int out_dtype, int out_width, int out_col0, int rows, int ncols,
+                               hipStream_t stream) {
+  if (rows == 0 || ncols == 0) return 0;
+  if (rows < 0 || ncols < 0 || !in || !out || col0 < 0 || out_col0 < 0 ||
+      col0 + ncols > in_width || out_col0 + ncols > out_width)
+    return ZA_ERR_ARG;
+  const size_t total = (size_t)rows * ncols;
+  dim3 grid((unsigned)((total + 255) / 256)), block(256);
+#define ZA_COPY_COLUMNS(TI, TO)                                                                   \
+  hipLaunchKernelGGL((copy_columns_kernel<TI, TO>), grid, block, 0, stream, (const TI*)in, (TO*)out, \
+                     in_width, col0, out_width, out_col0, ncols, total)
+  if (in_dtype == 0 && out_dtype == 0) ZA_COPY_COLUMNS(float, float);
+  else if (in_dtype == 0 && out_dtype == 1) ZA_COPY_COLUMNS(float, bf16_t);
+  else if (in_dtype == 1 && out_dtype == 0) ZA_COPY_COLUMNS(bf16_t, float);
+  else if (in_dtype == 1 && out_dtype == 1) ZA_COPY_COLUMNS(bf16_t, bf16_t);
+  else return ZA_ERR_UNSUPPORTED;
+#undef ZA_COPY_COLUMNS
+  return za_launch_status();
+}

@@ -60,6 +60,8 @@ _SIGNATURES = {
                                      c_longlong, c_void_p],
     ("activation", "za_swiglu"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     ("activation", "za_cast"): [c_void_p, c_int, c_void_p, c_int, c_longlong, c_void_p],
+    ("activation", "za_copy_columns"): [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int,
+                                        c_int, c_int, c_void_p],
     ("sampling", "za_argmax"): [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int,
                                 c_void_p],
     ("gemm", "za_gemm_bf16_rows16"): [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
@@ -1154,6 +1156,33 @@ def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     rc = _fn("activation", "za_cast")(_ptr(x), _code(x.dtype), _ptr(out), _code(dtype), x.numel(),
                                       _stream())
     _check(rc, "cast")
+    return out
+
+
+def copy_columns(src: torch.Tensor, col0: int, ncols: int, out: Optional[torch.Tensor] = None,
+                 out_col0: int = 0, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """Columns ``[col0, col0 + ncols)`` of every row of ``src [rows, width]``, as a new
+    ``[rows, ncols]`` tensor of ``dtype`` (the source's by default), or into columns
+    ``[out_col0, out_col0 + ncols)`` of ``out [rows, any width]``; converted between
+    float32 and bfloat16 on the way where the two differ."""
+    _need(src, "src", (torch.float32, torch.bfloat16))
+    if src.dim() != 2:
+        raise KernelError(f"copy_columns takes [rows, width], got {tuple(src.shape)}")
+    rows, width = src.shape
+    if out is None:
+        out = torch.empty((rows, ncols), dtype=dtype or src.dtype, device=src.device)
+        out_col0 = 0
+    _need(out, "out", (torch.float32, torch.bfloat16))
+    if out.dim() != 2 or out.shape[0] != rows:
+        raise KernelError(f"out has shape {tuple(out.shape)}, expected [{rows}, width]")
+    if not (0 <= col0 and col0 + ncols <= width and 0 <= out_col0
+            and out_col0 + ncols <= out.shape[1] and ncols >= 0):
+        raise KernelError(f"columns [{col0}, {col0 + ncols}) of {width} into [{out_col0}, "
+                          f"{out_col0 + ncols}) of {out.shape[1]}")
+    rc = _fn("activation", "za_copy_columns")(_ptr(src), _code(src.dtype), width, int(col0), _ptr(out),
+                                              _code(out.dtype), out.shape[1], int(out_col0), rows,
+                                              int(ncols), _stream())
+    _check(rc, "copy_columns")
     return out
 
 

@@ -64,7 +64,7 @@ class GroupedQueryAttention(Mixer):
     kind = "gqa_attention"
     graph_safe = True
     takes_stream = True
-    kernel_sources = ("gemm", "gemm_rows64", "rope_kv", "attention", "norm")
+    kernel_sources = ("gemm", "gemm_rows64", "rope_kv", "attention", "norm", "activation")
 
     @classmethod
     def tensor_rules(cls, params: Mapping[str, Any]) -> Dict[str, TensorRule]:
@@ -175,18 +175,23 @@ class GroupedQueryAttention(Mixer):
                 bool(rot) and self.position.pairing == "adjacent", self.eps,
                 write_kv=cache.writes)
         else:
-            # Any other encoding: norm with the norm kernel, encode through the
-            # part's own ``apply``, then let the fused kernel store what it is given.
-            heads = qkv.view(T, nh + 2 * nkv, d)
-            qh, kh, vh = heads[:, :nh], heads[:, nh:nh + nkv], heads[:, nh + nkv:]
+            # Any other encoding: norm with the norm kernel, encode through the part's own
+            # ``apply``, then let the fused kernel store what it is given.  q and k are
+            # taken out of the projection's rows and put back by a copy kernel.
+            qh = ops.copy_columns(qkv, 0, nh * d)
+            kh = ops.copy_columns(qkv, nh * d, nkv * d)
             if self.q_norm is not None:
-                qh = ops.add_rmsnorm(None, qh.reshape(-1, d).contiguous(), self.q_norm, self.eps,
-                                     qkv.dtype).view(T, nh, d)
-                kh = ops.add_rmsnorm(None, kh.reshape(-1, d).contiguous(), self.k_norm, self.eps,
-                                     qkv.dtype).view(T, nkv, d)
-            qh, kh = self.position.apply(qh, kh, step.positions)
-            packed = torch.cat([qh.to(qkv.dtype), kh.to(qkv.dtype), vh], dim=1).reshape(T, -1)
-            q = ops.qk_norm_rope_kv_write(packed.contiguous(), step.positions, slots, None, None,
+                qh = ops.add_rmsnorm(None, qh.view(T * nh, d), self.q_norm, self.eps, qkv.dtype)
+                kh = ops.add_rmsnorm(None, kh.view(T * nkv, d), self.k_norm, self.eps, qkv.dtype)
+            qh, kh = self.position.apply(qh.view(T, nh, d), kh.view(T, nkv, d), step.positions)
+            if tuple(qh.shape) != (T, nh, d) or tuple(kh.shape) != (T, nkv, d):
+                raise ValueError(f"position encoding {self.position.kind!r} returned "
+                                 f"{tuple(qh.shape)} and {tuple(kh.shape)}")
+            packed = torch.empty_like(qkv)
+            ops.copy_columns(qh.reshape(T, nh * d).contiguous(), 0, nh * d, packed, 0)
+            ops.copy_columns(kh.reshape(T, nkv * d).contiguous(), 0, nkv * d, packed, nh * d)
+            ops.copy_columns(qkv, (nh + nkv) * d, nkv * d, packed, (nh + nkv) * d)
+            q = ops.qk_norm_rope_kv_write(packed, step.positions, slots, None, None,
                                           None, cache.kv, nh, nkv, d, 0, False, self.eps,
                                           write_kv=cache.writes)
         mfma = self.mfma and cache.kv.shape[3] % 4 == 0
