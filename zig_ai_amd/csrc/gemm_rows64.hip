@@ -9,18 +9,21 @@
 //
 //   y [M, N] = x [M, K] . W [N, K]^T,   17 <= M <= 64 (any M from 1 runs)
 //
-// One workgroup of twelve waves takes 64 weight rows (one tile) and one range of K.
-// Waves 0-3 multiply: each owns 16 of the tile's weight rows over the whole range, reads
-// them from memory straight into matrix-core operand registers (16 bytes a lane and
-// step of 32 elements of K, sixteen steps requested ahead) and keeps the sums of all of
-// the step's rows, MB = ceil(M / 16) accumulators, so no sums meet across waves.  Waves
-// 4-11 only bring the step's rows: the range is cut into chunks of 256 elements of K,
-// they read a chunk's rows from memory (whole lines), turn them into bfloat16 operands
-// (with the norm: multiply by the norm's weight, add up the squares) and put them into
-// a ring of four chunks in LDS, two chunks ahead of the multiplying waves; one barrier
-// a chunk.  The rows' loads wait behind no weight (a wave's loads return in the order
-// of their requests: staged by the multiplying waves themselves, a chunk of rows would
-// queue behind every weight requested before it) and the weights' behind no row.
+// One workgroup of sixteen waves takes 64 weight rows (one tile) and one range of K,
+// which it walks in spans of 512 elements.  Waves 0-7 multiply: wave 4 h + g owns the
+// tile's g-th group of 16 weight rows and the h-th half of every span, reads its weights
+// from memory straight into matrix-core operand registers (16 bytes a lane and step of 32
+// elements of K, the fragments of two spans requested ahead) and keeps the sums of all of
+// the step's rows, MB = ceil(M / 16) accumulators; the two halves' sums meet in LDS at the
+// end.  Waves 8-15 only bring the step's rows: they read a span's rows from memory (whole
+// lines, a wave 2 MB rows), turn them into bfloat16 operands (with the norm: multiply by
+// the norm's weight, which lies in LDS, and add up the squares) and put them into one of
+// two places in LDS, a span ahead of the multiplying waves; one barrier a span.  The
+// rows' loads wait behind no weight (a wave's loads return in the order of their
+// requests: staged by the multiplying waves themselves, a span of rows would queue behind
+// every weight requested before it) and the weights' behind no row.  Up to 32 rows the
+// staging waves hold two spans in flight in registers, beyond that one.  The workgroups
+// of a die start their walk over K at different spans (see `rot` below).
 //
 // Forms (MODE):
 //   STORE    y as bfloat16
