@@ -737,6 +737,8 @@ def linear_rows64(x, weight: torch.Tensor, mode: int = ROWS64_STORE,
     if normed is not None:
         if mode == ROWS64_ADD or normed.dtype != torch.bfloat16:
             raise KernelError("the kernel runs the norm only for bfloat16 products that it stores")
+        if normed.residual.numel() >= 1 << 31:
+            raise KernelError("the kernel addresses the stream's rows with 32-bit offsets")
     else:
         _need(x, "x", torch.bfloat16)
     if mode == ROWS64_ADD:
