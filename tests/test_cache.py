@@ -124,6 +124,35 @@ def test_planes_and_typed_state_in_memory():
         CacheManager({0: PagedNeed(())}, 4, 4, 1, allocate=False)
 
 
+def test_state_that_starts_elsewhere_than_zero():
+    """A state need may name its starting value: a running maximum at -inf, a product at 1,
+    a counter at -1; every new request finds it, also in a slot another request used, and
+    the entries beside it still start at zero."""
+    import math
+
+    import torch
+    needs = {"top": StateNeed((4,), init=-math.inf), "conv": StateNeed((2, 3)),
+             "scale": StateNeed((2,), dtype=torch.float32, init=1.0),
+             "last": StateNeed((1,), dtype=torch.int32, init=-1)}
+    m = CacheManager(needs, 4, 4, 2, device=torch.device("cpu"), dtype=torch.float32)
+    top, conv, scale, last = (m.view(k).state for k in ("top", "conv", "scale", "last"))
+    for name in ("a", "b"):
+        slot = m.admit(name)
+        assert bool(torch.isinf(top[slot]).all()) and float(top[slot].max()) < 0
+        assert float(conv[slot].abs().sum()) == 0.0
+        assert scale[slot].tolist() == [1.0, 1.0] and int(last[slot, 0]) == -1
+        top[slot] = 3.0
+        conv[slot] = 7.0
+        scale[slot] = 0.5
+        last[slot, 0] = 12
+    m.release("a")
+    slot = m.admit("c")                              # a's slot again
+    assert bool(torch.isinf(top[slot]).all()) and float(conv[slot].abs().sum()) == 0.0
+    assert scale[slot].tolist() == [1.0, 1.0] and int(last[slot, 0]) == -1
+    other = m.slot_of("b")
+    assert float(top[other, 0]) == 3.0 and int(last[other, 0]) == 12     # b's state is untouched
+
+
 def test_reserve_is_all_or_nothing():
     m = manager(num_pages=4, window=6)
     m.admit("a")

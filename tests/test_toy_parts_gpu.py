@@ -55,7 +55,38 @@ def toy_classes():
                 row += n
             return ops.linear(out.to(x.dtype), self.weight)
 
+    class RunningMaxMixer(Mixer):
+        """y[t] = W * max(x[0..t]), element by element: the state is the largest input
+        so far, which for a new request is minus infinity, not zero."""
+        kind = "toy_running_max"
+        kernel_sources = ("gemm",)
+
+        @classmethod
+        def tensor_rules(cls, params):
+            w = int(params["width"])
+            return {"mix.weight": TensorRule(((w, w),))}
+
+        @classmethod
+        def cache_need(cls, params):
+            return StateNeed((int(params["width"]),), init=float("-inf"))
+
+        def __init__(self, params, tensors, runtime):
+            super().__init__(params, tensors, runtime)
+            self.weight = tensors["mix.weight"]
+
+        def forward(self, x, step, cache):
+            out = torch.empty_like(x, dtype=torch.float32)
+            row = 0
+            for n, slot in zip(step.seq_lens_host, step.slots_host):
+                state = cache.state[slot]
+                top = torch.cummax(torch.cat([state[None], x[row:row + n].float()]), dim=0).values[1:]
+                out[row:row + n] = top
+                state.copy_(top[-1])
+                row += n
+            return ops.linear(out.to(x.dtype), self.weight)
+
     register_mixer(RunningMeanMixer.kind, RunningMeanMixer)
+    register_mixer(RunningMaxMixer.kind, RunningMaxMixer)
     return RunningMeanMixer
 
 
@@ -79,8 +110,9 @@ class ToyConfig:
         layers = []
         for i, kind in enumerate(d["kinds"]):
             p = f"layers.{i}."
-            if kind == "toy":
-                mixer = PartSpec("toy_running_mean", {"width": H}, {"mix.weight": (p + "mix.weight",)})
+            if kind in ("toy", "max"):
+                mixer = PartSpec("toy_running_mean" if kind == "toy" else "toy_running_max",
+                                 {"width": H}, {"mix.weight": (p + "mix.weight",)})
             else:
                 rope = PartSpec("rope", {"head_dim": d["head_dim"], "rotary_dim": d["head_dim"] // 2,
                                          "theta": 100.0, "pairing": "adjacent"})
@@ -113,11 +145,11 @@ TOY = {"architectures": ["ToyForCausalLM"], "width": 48, "vocab_size": 97, "ffn"
        "schedule": [(0, 0), (1, 1), (2, 2), (0, 3), (1, 1, False)]}
 
 
-def toy_oracle(folder, tokens):
+def toy_oracle(folder, tokens, d=None):
     """The toy model, whole sequence, float64, written out directly."""
     from safetensors.torch import load_file
     w = {k: v.double() for k, v in load_file(folder + "/model.safetensors").items()}
-    d = TOY
+    d = d or TOY
     H, nh, hd = d["width"], d["heads"], d["head_dim"]
     x = w["embed.weight"][torch.tensor(tokens)]
     pos = torch.arange(len(tokens))
@@ -129,6 +161,8 @@ def toy_oracle(folder, tokens):
         if d["kinds"][layer] == "toy":
             mean = torch.cumsum(n1, 0) / torch.arange(1, len(tokens) + 1)[:, None]
             m = mean @ w[p + "mix.weight"].T
+        elif d["kinds"][layer] == "max":
+            m = torch.cummax(n1, 0).values @ w[p + "mix.weight"].T
         else:
             T = len(tokens)
             q = (n1 @ w[p + "q_proj.weight"].T).view(T, nh, hd)
@@ -176,6 +210,33 @@ def test_toy_architecture_steps_through_the_engine(dtype):
         # the window of 9 lets pages behind it go back while the request still runs
         assert runner.cache.stats()["groups"][0]["pages_high_water"] < sum(
             (n + 3) // 4 for n in lengths)
+
+
+TOY_MAX = dict(TOY, kinds=["max", "attn"], schedule=[(0, 0), (1, 1)])
+
+
+def test_a_state_that_does_not_start_at_zero():
+    """A mixer whose state starts at minus infinity: every request, also one that takes
+    a slot another request has left, begins from that value and from nothing else."""
+    from zig_ai_amd.config import register_architecture
+    from zig_ai_amd.engine import DecoderModel, ModelRunner
+    toy_classes()
+    register_architecture("ToyForCausalLM", ToyConfig)
+    folder = eu.model_folder(TOY_MAX, 12, torch.float32, std=0.2, norm_init="around_one",
+                             role_std={"norm": 0.2, "q_proj.weight": 0.08, "k_proj.weight": 0.08})
+    model = DecoderModel.from_folder(folder, "float32")
+    lengths = [21, 9, 30, 14, 11]
+    prompts = [eu.random_tokens(n, 97, 700 + n) for n in lengths]
+    # every input of the first request is below zero at some channel with near
+    # certainty, so a state that started at zero would show in its first tokens
+    expect = [toy_oracle(folder, p, TOY_MAX) for p in prompts]
+    for schedule in (eu.whole(lengths), eu.mixed(lengths, seed=5, max_live=2, decode_tail=4)):
+        # two slots for five requests: each slot is used again, after a request that
+        # left its running maximum there
+        runner = ModelRunner(model, page_size=4, num_pages=24, num_slots=2)
+        got = eu.run_schedule(runner, prompts, schedule)
+        for g, e in zip(got, expect):
+            assert eu.rel_err(g, e) < 1e-4
 
 
 # ------------------------------ a feed-forward with routing, another position encoding

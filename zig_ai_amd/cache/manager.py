@@ -173,6 +173,9 @@ class CacheManager:
             offset += (nbytes + 15) // 16 * 16
         self.bytes_per_slot = offset
         self.slot_memory: Optional[torch.Tensor] = None
+        # what a new request's slot holds: zero bytes, or a row with every state entry's own
+        # starting value (``StateNeed.init``)
+        self._slot_start: Optional[torch.Tensor] = None
         if allocate:
             if device is None:
                 raise ValueError("a device is needed to allocate the cache")
@@ -182,6 +185,13 @@ class CacheManager:
             if self.bytes_per_slot:
                 self.slot_memory = torch.zeros((num_slots, self.bytes_per_slot),
                                                dtype=torch.uint8, device=device)
+                if any(need.init != 0 for _, need in state_entries):
+                    start = torch.zeros((self.bytes_per_slot,), dtype=torch.uint8, device=device)
+                    for cid, need in state_entries:
+                        if need.init != 0:
+                            off, nbytes, _, dt = self._state_layout[cid]
+                            start[off:off + nbytes].view(dt).fill_(need.init)
+                    self._slot_start = start
         self._n_groups = G
         self._scratch = (ctypes.c_int * max(G, 1))()
 
@@ -257,14 +267,21 @@ class CacheManager:
     def admit(self, req: Hashable) -> int:
         slot = ctypes.c_int()
         raise_for(self._lib.za_cache_admit(self._ptr, self.handles.of(req), ctypes.byref(slot)))
-        if self.slot_memory is not None:
-            self.slot_memory[slot.value].zero_()
+        self._start_slot(slot.value)
         return slot.value
 
+    def _start_slot(self, slot: int) -> None:
+        """A new request's state: every entry at its starting value."""
+        if self.slot_memory is None:
+            return
+        if self._slot_start is None:
+            self.slot_memory[slot].zero_()
+        else:
+            self.slot_memory[slot].copy_(self._slot_start)
+
     def admitted_by_scheduler(self, req: Hashable) -> None:
-        """The host library's scheduler admitted ``req`` itself: clear its state."""
-        if self.slot_memory is not None:
-            self.slot_memory[self.slot_of(req)].zero_()
+        """The host library's scheduler admitted ``req`` itself: start its state."""
+        self._start_slot(self.slot_of(req))
 
     def pages_needed(self, req: Hashable, n_new: int) -> Dict[int, int]:
         if req not in self:

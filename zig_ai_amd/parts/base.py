@@ -79,15 +79,15 @@ class PagedNeed:
 @dataclass(frozen=True)
 class StateNeed:
     """Per-request state of fixed size; 32-bit floats unless ``dtype`` says otherwise.
-    A new request's state is ZERO BYTES (the cache manager clears the slot at admission
-    and knows no other start).  A mixer whose state starts elsewhere (a running maximum
-    at -inf, a product at 1) stores it relative to that start, so that zero bytes mean
-    it (the maximum as ``exp(-m)`` or with a "seen anything" flag beside it, the product
-    minus one), or treats a request's first portion, ``step.ctx_lens_host[i] == 0``, as
-    the start itself."""
+    A new request's state is ``init`` in every element (zero by default: the cache manager
+    fills the slot at admission); a state that starts at a running maximum's ``-inf`` or a
+    product's ``1`` says so here.  A state whose elements start at different values stores
+    them relative to their start, or treats a request's first portion,
+    ``step.ctx_lens_host[i] == 0``, as the start itself."""
 
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
+    init: float = 0.0
 
 
 # ------------------------------------------------------------------- runtime
