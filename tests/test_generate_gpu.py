@@ -237,6 +237,46 @@ def test_steps_issued_ahead_change_nothing():
         assert stats["requests"] == 0 and all(g["pages_free"] == g["pages"] for g in stats["groups"])
 
 
+def test_runs_of_steps_issued_before_the_last_run_is_read():
+    """Runs of 3 decode steps, the next run issued before the tokens of the last one are
+    read: a request that meets its stop token in one run while the next is already on the
+    GPU, requests that reach their lengths at different steps, and so few pages that a
+    run ends early and a request is preempted; always the tokens of one step at a time."""
+    from zig_ai_amd.engine import Engine
+    from zig_ai_amd.sampling.sampler import SamplingParams
+    folder = folder_for(TINY_B, 1)
+    prompts = [eu.random_tokens(n, 512, 640 + n) for n in (12, 30, 7)]
+    for kw in (dict(temperature=0.0), dict(temperature=0.8, top_p=0.95, seed=5)):
+        def engine(multi_step, num_pages=64):         # a new engine: requests numbered from 0
+            return Engine(folder, dtype="float32", page_size=8, num_pages=num_pages, max_num_seqs=3,
+                          multi_step=multi_step)
+        free_run = engine(1).generate(prompts, max_new_tokens=30, eos_token_id=-1, **kw)
+        stop = free_run[2][7]                         # request 2 stops in the third run of 3
+        want = engine(1).generate(prompts, max_new_tokens=30, eos_token_id=stop, **kw)
+        assert len(want[2]) <= 8
+        ahead = engine(3)
+        assert ahead.generate(prompts, max_new_tokens=30, eos_token_id=stop, **kw) == want
+        assert ahead.runner.graphs.replays > 20
+        stats = ahead.stats()
+        assert stats["requests"] == 0 and all(g["pages_free"] == g["pages"] for g in stats["groups"])
+        # requests with different lengths left: the run is as long as the shortest allows
+        sampling = SamplingParams(temperature=kw["temperature"], top_p=kw.get("top_p", 1.0),
+                                  seed=kw.get("seed", 42))
+
+        def uneven(e):
+            reqs = [e.add_request(p, n, sampling, eos_token_id=-1) for p, n in zip(prompts, (30, 11, 23))]
+            e.run()
+            return [list(r.output) for r in reqs]
+        got = uneven(engine(3))
+        assert got == uneven(engine(1)) and [len(g) for g in got] == [30, 11, 23]
+        # 14 pages of 8 tokens: the three requests need 6 + 6 + 4 at their ends
+        tight = engine(3, num_pages=14)
+        assert tight.generate(prompts, max_new_tokens=30, eos_token_id=-1, **kw) == free_run
+        assert tight.stats()["preemptions"] >= 1
+        stats = tight.stats()
+        assert stats["requests"] == 0 and all(g["pages_free"] == g["pages"] for g in stats["groups"])
+
+
 def test_command_line_greedy():
     folder = folder_for(TINY_A, 0)
     oracle = plain.PlainLfm2(folder)

@@ -11,6 +11,7 @@ from __future__ import annotations
 import time
 from typing import Hashable, List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..sampling.sampler import SamplingParams, sample_rows, uniforms
@@ -93,6 +94,8 @@ class Engine:
         self.timings = {"steps": 0, "step_seconds": 0.0, "tokens_run": 0, "tokens_generated": 0}
         self.max_num_batched_tokens = int(max_num_batched_tokens)
         self.max_num_seqs = int(max_num_seqs)
+        self._token_staging = None       # pinned buffers for the tokens of runs of decode steps
+        self._token_turn = 0
         self.warm_up_steps = self.warm_up() if warm_up else 0
 
     # ----------------------------------------------------------------- warm-up
@@ -193,12 +196,13 @@ class Engine:
         return done
 
     def _steps_ahead(self, plan: Sequence[ScheduledEntry]) -> int:
-        """How many decode steps may be issued in one go after this plan: more than
-        one only if every entry is a decoding request, nobody waits to be admitted,
-        and no request needs its history on the host between steps."""
+        """How many decode steps may follow this plan before the first of its requests
+        reaches its length: more than one only if every entry is a decoding request,
+        nobody waits to be admitted, and no request needs its history on the host
+        between steps.  (``multi_step`` of them are issued in one go.)"""
         if self.multi_step <= 1 or self.scheduler.has_waiting():
             return 1
-        k = self.multi_step
+        k = 1 << 30
         for e in plan:
             req = e.request
             if e.count != 1 or not e.samples or e.start == 0 \
@@ -208,37 +212,93 @@ class Engine:
                     self.max_model_len - len(req.prompt) - len(req.output))
         return max(1, k)
 
-    def _decode_many(self, plan: Sequence[ScheduledEntry], k: int, start: float) -> List[Request]:
-        reqs = [e.request for e in plan]
-        params = [r.sampling for r in reqs]
-        device = self.model.runtime.device
-        if all(p.greedy for p in params):
-            def sample(logits: torch.Tensor, i: int) -> torch.Tensor:
-                return ops.argmax(logits)
-        else:
-            S = len(reqs)
-            packed = torch.tensor([[p.temperature for p in params], [p.top_p for p in params]],
-                                  dtype=torch.float32).to(device)
-            top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32).to(device)
-            u = torch.tensor(uniforms([p.seed for p in params] * k,
-                                      [r.number for r in reqs] * k,
-                                      [len(r.output) + i for i in range(k) for r in reqs]),
-                             dtype=torch.float32).view(k, S).to(device)
+    def _to_device(self, host: np.ndarray) -> torch.Tensor:
+        """A small array to the device through pinned memory, without the host waiting
+        (a copy from ordinary memory waits for everything issued before it)."""
+        words = host.size
+        ring = self.runner.staging
+        pinned = ring.take(words)
+        pinned.numpy()[:words] = host.view(np.int32)
+        dev = torch.empty((words,), dtype=torch.int32, device=self.model.runtime.device)
+        dev.copy_(pinned[:words], non_blocking=True)
+        ring.copied()
+        return dev
 
-            def sample(logits: torch.Tensor, i: int) -> torch.Tensor:
-                return ops.sample(logits, packed[0], top_k, packed[1], u[i])
-        drawn = self.runner.decode_steps([r.id for r in reqs],
-                                         [r.span(e.start, 1)[0] for r, e in zip(reqs, plan)],
-                                         k, sample).tolist()        # the one wait of the run
+    def _decode_many(self, plan: Sequence[ScheduledEntry], horizon: int, start: float) -> List[Request]:
+        """Decode steps of the plan's requests, ``multi_step`` at a time, until the first
+        of them reaches its length (``horizon`` steps) or one meets its stop token.  The
+        next run of steps is issued before the tokens of the last one are read, so the GPU
+        does not wait while the host records them; a request that stops inside a run
+        wastes the steps that were issued after its last token, nothing else."""
+        reqs = [e.request for e in plan]
+        ids = [r.id for r in reqs]
+        params = [r.sampling for r in reqs]
+        S = len(reqs)
+        base = [len(r.output) for r in reqs]        # (the outputs grow only when tokens are read)
+        greedy = all(p.greedy for p in params)
+        if not greedy:
+            fixed = self._to_device(np.concatenate([
+                np.asarray([p.temperature for p in params], dtype=np.float32).view(np.int32),
+                np.asarray([p.top_p for p in params], dtype=np.float32).view(np.int32),
+                np.asarray([p.top_k for p in params], dtype=np.int32)]))
+            temperature, top_p = fixed[:S].view(torch.float32), fixed[S:2 * S].view(torch.float32)
+            top_k = fixed[2 * S:]
+        if self._token_staging is None or self._token_staging[0].numel() < self.multi_step * S:
+            self._token_staging = [torch.empty((self.multi_step * max(S, self.max_num_seqs),),
+                                               dtype=torch.int32, pin_memory=True) for _ in range(3)]
+        issued = 0
+        in_flight: List[tuple] = []      # (first step, steps, pinned tokens, event), oldest first
+        current: Optional[torch.Tensor] = None
+        alive = list(range(S))
         done: List[Request] = []
-        alive = list(range(len(reqs)))
-        for j, row in enumerate(drawn):
-            step_plan = [ScheduledEntry(reqs[a], plan[a].start + j, 1, True) for a in alive]
-            done += self.scheduler.update(step_plan, {reqs[a].id: row[a] for a in alive})
-            self.timings["tokens_generated"] += len(alive)
-            self.timings["tokens_run"] += len(alive)
-            alive = [a for a in alive if reqs[a].phase == RUNNING]
-        self.timings["steps"] += len(drawn)
+        while True:
+            n = min(self.multi_step, horizon - issued)
+            more = n >= 1 and len(alive) == S and len(in_flight) < 2
+            if more:
+                if greedy:
+                    def sample(logits: torch.Tensor, i: int) -> torch.Tensor:
+                        return ops.argmax(logits)
+                else:
+                    u = self._to_device(np.asarray(
+                        uniforms([p.seed for p in params] * n, [r.number for r in reqs] * n,
+                                 [b + issued + i for i in range(n) for b in base]),
+                        dtype=np.float32)).view(torch.float32).view(n, S)
+
+                    def sample(logits: torch.Tensor, i: int, u=u) -> torch.Tensor:
+                        return ops.sample(logits, temperature, top_k, top_p, u[i])
+                tokens = [r.span(e.start, 1)[0] for r, e in zip(reqs, plan)] if current is None else None
+                drawn = self.runner.decode_steps(ids, tokens, n, sample, device_tokens=current,
+                                                 optional=current is not None)
+                if drawn is None:                 # no pages for a further run
+                    horizon = issued
+                    continue
+                steps = drawn.shape[0]
+                pinned = self._token_staging[self._token_turn % 3]
+                self._token_turn += 1
+                pinned[:steps * S].copy_(drawn.view(-1), non_blocking=True)
+                event = torch.cuda.Event()
+                event.record()
+                in_flight.append((issued, steps, pinned, event))
+                issued += steps
+                current = drawn[steps - 1]
+                if steps < n:                     # pages ran out inside the run
+                    horizon = issued
+                if len(in_flight) < 2 and issued < horizon:
+                    continue                      # the next run first, then this one's tokens
+            if not in_flight:
+                break
+            first, steps, pinned, event = in_flight.pop(0)
+            event.synchronize()                   # the one wait of the run
+            rows = pinned[:steps * S].view(steps, S).tolist()
+            for j, row in enumerate(rows):
+                if not alive:
+                    break
+                step_plan = [ScheduledEntry(reqs[a], plan[a].start + first + j, 1, True) for a in alive]
+                done += self.scheduler.update(step_plan, {reqs[a].id: row[a] for a in alive})
+                self.timings["tokens_generated"] += len(alive)
+                self.timings["tokens_run"] += len(alive)
+                alive = [a for a in alive if reqs[a].phase == RUNNING]
+            self.timings["steps"] += steps
         self.timings["step_seconds"] += time.perf_counter() - start
         return done
 

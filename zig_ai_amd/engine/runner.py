@@ -84,21 +84,32 @@ class ModelRunner:
         self.steps_run += 1
         return logits
 
-    def decode_steps(self, requests: Sequence[Hashable], tokens: Sequence[int], n_steps: int,
-                     sample: Callable[[torch.Tensor, int], torch.Tensor]) -> torch.Tensor:
+    def decode_steps(self, requests: Sequence[Hashable], tokens: Optional[Sequence[int]], n_steps: int,
+                     sample: Callable[[torch.Tensor, int], torch.Tensor],
+                     device_tokens: Optional[torch.Tensor] = None,
+                     optional: bool = False) -> Optional[torch.Tensor]:
         """Up to ``n_steps`` decode steps of the same requests without the host waiting
-        in between: ``tokens`` are the requests' next tokens, ``sample(logits, i)``
-        draws the tokens of step ``i`` (int32 ``[len(requests)]`` on the device, without
-        looking at them on the host), and those are the next step's tokens, handed over
-        on the device.  Returns what was drawn, ``[steps done, len(requests)]`` on the
-        device; fewer steps than asked for are done when pages run out after the first
-        (``OutOfPages`` from the first step is raised)."""
-        if len(requests) != len(tokens) or not requests:
+        in between: ``tokens`` are the requests' next tokens (or ``device_tokens``, int32
+        ``[len(requests)]`` on the device, for instance the last tokens of an earlier
+        call whose result the host has not read yet), ``sample(logits, i)`` draws the
+        tokens of step ``i`` (int32 ``[len(requests)]`` on the device, without looking at
+        them on the host), and those are the next step's tokens, handed over on the
+        device.  Returns what was drawn, ``[steps done, len(requests)]`` on the device;
+        fewer steps than asked for are done when pages run out after the first
+        (``OutOfPages`` from the first step is raised, or with ``optional`` answered
+        with ``None``: nothing was done)."""
+        if device_tokens is None and (tokens is None or len(requests) != len(tokens)) or not requests:
             raise StepError("one next token per request is needed")
-        entries = [StepEntry(r, [t], [0]) for r, t in zip(requests, tokens)]
+        if device_tokens is not None and (device_tokens.dtype != torch.int32
+                                          or device_tokens.numel() != len(requests)):
+            raise StepError(f"device_tokens must be int32 [{len(requests)}]")
+        if device_tokens is not None and self.graphs is None:
+            tokens = device_tokens.view(-1).tolist()
+        entries = [StepEntry(r, [0 if tokens is None else t], [0])
+                   for r, t in zip(requests, tokens if tokens is not None else requests)]
         ones = [1] * len(requests)
         drawn: List[torch.Tensor] = []
-        current = None
+        current = device_tokens if self.graphs is not None else None
         for i in range(n_steps):
             try:
                 if self.graphs is not None:
@@ -111,6 +122,8 @@ class ModelRunner:
                     logits = self.model.forward(self.prepare(entries), self.views)
             except OutOfPages:
                 if i == 0:
+                    if optional:
+                        return None
                     raise
                 break
             current = sample(logits, i)
