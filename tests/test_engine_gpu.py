@@ -791,6 +791,51 @@ def test_decode_steps_hand_tokens_over_on_the_device(dtype):
         assert drawn.tolist() == want[:drawn.shape[0]]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_batches_with_padding_rows(dtype):
+    """A decode batch of 19 requests filled up to 24 with rows of the runner's own: every
+    request's logits are those of the plain implementation at each step (run as it is,
+    recorded, replayed), the batch of 17 that is left when two requests end meets the same
+    recording, and a runner without slots to spare records the batch as it is."""
+    from zig_ai_amd.engine import ModelRunner, StepEntry
+    model, _, _ = setup("D", dtype)
+    cfg, seed = CONFIGS["D"]
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    oracle = plain.PlainLfm2(eu.model_folder(cfg, seed, store, **eu.sharp_kwargs()))
+    ids = list(range(19))
+    lens = [3 + (7 * i) % 23 for i in ids]
+    new = 5
+    seqs = [eu.random_tokens(n + new, cfg["vocab_size"], 7000 + i) for i, n in zip(ids, lens)]
+    expect = [oracle.logits(q) for q in seqs]
+    for slots, shape in ((19 + 7, 24), (19, 19)):
+        runner = ModelRunner(model, page_size=8, num_pages=160, num_slots=slots, pad_decode=True)
+        for r, n, q in zip(ids, lens, seqs):
+            runner.admit(r)
+            runner.step([StepEntry(r, q[:n], [])])
+        live = list(ids)
+        for j in range(new):
+            if j == 3:                               # two requests end: 17 are left
+                for r in (4, 11):
+                    runner.release(r)
+                    live.remove(r)
+            logits = runner.step([StepEntry(r, [seqs[r][lens[r] + j]], [0]) for r in live])
+            assert logits.shape[0] == len(live)
+            for row, r in enumerate(live):
+                err = eu.rel_err(logits[row], expect[r][lens[r] + j])
+                assert err < TOL[dtype], f"{slots} slots, step {j}, request {r}: off by {err:.3e}"
+        sizes = {key[0] for key in runner.graphs.entries}
+        assert sizes == ({shape} if shape == 24 else {19, 17}), sizes
+        if shape == 24:
+            assert runner.graphs.captures == 1 and runner.graphs.replays == new - 1
+        for r in live:
+            runner.release(r)
+        runner.release_padding()
+        runner.cache.check()
+        stats = runner.cache.stats()
+        assert stats["requests"] == 0 and stats["slots_free"] == stats["slots"]
+        assert all(g["pages_free"] == g["pages"] for g in stats["groups"])
+
+
 def test_recorded_shapes_are_dropped_when_there_are_too_many(monkeypatch):
     """Only so many recorded steps are kept; the one used longest ago goes, and comes
     back (recorded anew) when its shape does.  Three batch sizes in turn, three steps

@@ -185,6 +185,35 @@ def test_tokens_do_not_depend_on_scheduling():
     assert all(g["pages_free"] == g["pages"] for g in stats["groups"])
 
 
+def test_decode_batches_filled_up_to_recorded_sizes():
+    """28 requests that stop one after the other: above 16 requests the decode batch is
+    filled up to a multiple of 8 with rows of the engine's own, so the batches of 28 down
+    to 17 requests meet two recorded shapes instead of twelve.  The tokens are those of an
+    engine that records nothing; the rows' slots and pages are back when no request is left."""
+    from zig_ai_amd.engine import Engine
+    from zig_ai_amd.sampling.sampler import SamplingParams
+    folder = folder_for(TINY_B, 1)
+    prompts = [eu.random_tokens(3 + (5 * i) % 17, 512, 900 + i) for i in range(28)]
+    lengths = [6 + i for i in range(28)]
+    for sampling in (SamplingParams(temperature=0.0), SamplingParams(temperature=0.9, top_k=50, seed=8)):
+        def run(engine):
+            reqs = [engine.add_request(p, n, sampling, eos_token_id=-1) for p, n in zip(prompts, lengths)]
+            engine.run()
+            return [list(r.output) for r in reqs]
+        kw = dict(dtype="float32", page_size=8, num_pages=256, max_num_seqs=28)
+        want = run(Engine(folder, use_graphs=False, **kw))
+        engine = Engine(folder, **kw)
+        assert run(engine) == want
+        graphs = engine.runner.graphs
+        sizes = sorted({key[0] for key in graphs.entries})
+        assert [n for n in sizes if n > 16] == [24, 32], sizes
+        assert graphs.replays >= 12          # of the 16 steps with more than 16 requests
+        stats = engine.stats()
+        assert stats["requests"] == 0 and stats["slots_free"] == stats["slots"]
+        assert all(g["pages_free"] == g["pages"] for g in stats["groups"])
+        engine.runner.cache.check()
+
+
 def test_a_length_limit_beyond_the_models_own_is_refused():
     """``max_model_len`` above the model's ``max_position_embeddings`` would stop a step in
     the middle of a call and every request of the call with it: refused when the engine is

@@ -84,8 +84,12 @@ class Engine:
                         f"cache of one request of {limit} tokens ({per_request * per_page / 2**30:.1f}"
                         " GiB); lower max_model_len")
                 num_pages = min(num_pages, fit)
-        self.runner = ModelRunner(self.model, page_size, num_pages, max_num_seqs,
-                                  use_graphs=use_graphs, portion_graphs=portion_graphs)
+        # (the slots beyond max_num_seqs are for the rows that fill decode batches up to
+        # recorded sizes, see ModelRunner.PAD_ROWS; they are given back when no request is left)
+        self.runner = ModelRunner(self.model, page_size, num_pages,
+                                  max_num_seqs + ModelRunner.PAD_ROWS - 1,
+                                  use_graphs=use_graphs, portion_graphs=portion_graphs,
+                                  pad_decode=use_graphs)
         self.on_step = on_step
         self.multi_step = 1 if on_step is not None else max(1, int(multi_step))
         self.scheduler = Scheduler(self.runner.cache, max_num_seqs, max_num_batched_tokens,
@@ -167,11 +171,15 @@ class Engine:
         """One scheduled step; returns the requests that finished in it."""
         plan = self.scheduler.schedule()
         if not plan:
+            self.runner.release_padding()
             return []
         start = time.perf_counter()
         k = self._steps_ahead(plan)
         if k > 1:
-            return self._decode_many(plan, k, start)
+            done = self._decode_many(plan, k, start)
+            if done and not self.scheduler.has_work():
+                self.runner.release_padding()
+            return done
         entries = []
         for e in plan:
             entries.append(StepEntry(e.request.id, e.request.span(e.start, e.count),
@@ -193,6 +201,8 @@ class Engine:
                           "tokens": drawn, "seconds": elapsed})
         self.timings["tokens_run"] += sum(e.count for e in plan)
         self.timings["tokens_generated"] += len(sampling)
+        if done and not self.scheduler.has_work():
+            self.runner.release_padding()
         return done
 
     def _steps_ahead(self, plan: Sequence[ScheduledEntry]) -> int:
@@ -331,6 +341,8 @@ class Engine:
     def abort(self, request: Request) -> None:
         """Take a request out of the engine; what it holds is given back."""
         self.scheduler.abort(request)
+        if not self.scheduler.has_work():
+            self.runner.release_padding()
 
     def stats(self) -> dict:
         out = self.runner.cache.stats()

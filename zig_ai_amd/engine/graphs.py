@@ -87,7 +87,8 @@ class DecodeGraphs:
         raise_for(rc)
 
     def run(self, runner, entries: Sequence[StepEntry],
-            device_tokens: Optional[torch.Tensor] = None, more_to_come: bool = False) -> torch.Tensor:
+            device_tokens: Optional[torch.Tensor] = None, more_to_come: bool = False,
+            padded: bool = True) -> torch.Tensor:
         """Logits ``[len(entries), vocab]`` of a step of single tokens (one row per
         entry, whatever the entries want).  Takes the pages the new tokens need (all
         or none: ``OutOfPages`` leaves everything as it was).
@@ -103,12 +104,20 @@ class DecodeGraphs:
         what the sampler drew from the last step's logits) the entries' own tokens are
         ignored and the step reads its token ids from that tensor, copied on the
         device: the host never waits for them, so it can lay out this step while the
-        last one is still running."""
+        last one is still running.
+
+        A runner that pads its decode batches (``ModelRunner.padding``) adds rows of its
+        own behind the entries (unless ``padded`` is false); the step runs them like any
+        request's, and their logits are not returned."""
         cache = runner.cache
-        S = len(entries)
+        asked_for = len(entries)
         if device_tokens is not None and (device_tokens.dtype != torch.int32
-                                          or device_tokens.numel() != S):
-            raise StepError(f"device_tokens must be int32 [{S}]")
+                                          or device_tokens.numel() != asked_for):
+            raise StepError(f"device_tokens must be int32 [{asked_for}]")
+        pads = runner.padding(asked_for) if padded and hasattr(runner, "padding") else []
+        if pads:
+            entries = list(entries) + [StepEntry(name, [0], [0]) for name in pads]
+        S = len(entries)
         sc = self._scratch(S)
         ptr = sc["ptr"]
         known = cache.handles.known
@@ -129,6 +138,10 @@ class DecodeGraphs:
         lib = self._lib
         rc = lib.za_decode_prepare(cache.native, S, ptr["reqs"], ptr["toks"], self._vocab,
                                    self._max_position, ptr["extent"])
+        if rc == hostlib.OUT_OF_PAGES and pads:
+            # the requests' own rows may still fit once the padding rows' pages are back
+            runner.release_padding()
+            return self.run(runner, entries[:asked_for], device_tokens, more_to_come, padded=False)
         if rc:
             self._raise(rc, entries)
         widest, longest = int(sc["extent"][0]), int(sc["extent"][1])
@@ -160,14 +173,14 @@ class DecodeGraphs:
             slot["copied"].record()
             if device_tokens is not None:
                 first = int(slot["sections"][0])          # where the token ids sit
-                slot["buffer"][first:first + S].copy_(device_tokens.view(-1))
+                slot["buffer"][first:first + asked_for].copy_(device_tokens.view(-1))
             slot["graph"].replay()
             self.replays += 1
-            return slot["logits"]
+            return slot["logits"][:asked_for] if pads else slot["logits"]
         model = runner.model
         if device_tokens is not None:                     # a first step of this shape: on the host
             entries = [StepEntry(e.request, [t], [0])
-                       for e, t in zip(entries, device_tokens.view(-1).tolist())]
+                       for e, t in zip(entries, device_tokens.view(-1).tolist())] + entries[asked_for:]
         asked = [StepEntry(e.request, e.tokens, [0]) for e in entries]
         prepared = PreparedEntries(asked, cache, self._vocab)
         if slot is None:
@@ -200,6 +213,8 @@ class DecodeGraphs:
         slot["seen"] += 1
         if first:
             logits = model.forward(ctx, runner.views)      # this step, eagerly
+            if pads:
+                logits = logits[:asked_for]
             if not more_to_come:
                 return logits
         graph = torch.cuda.CUDAGraph()
@@ -219,7 +234,7 @@ class DecodeGraphs:
             return logits
         graph.replay()                                     # the shape's second step
         self.replays += 1
-        return slot["logits"]
+        return slot["logits"][:asked_for] if pads else slot["logits"]
 
     # ------------------------------------------------- steps with prompt portions
     def run_portions(self, runner, entries: Sequence[StepEntry]) -> torch.Tensor:

@@ -18,18 +18,28 @@ from typing import Callable, Hashable, List, Optional, Sequence
 
 import torch
 
-from ..cache.pages import OutOfPages
+from ..cache.pages import OutOfPages, OutOfSlots
 from .batch import StagingRing, StepContext, StepEntry, StepError, build_step
 from .graphs import DecodeGraphs
 from .model import DecoderModel
 
 
 class ModelRunner:
+    # A recorded decode step serves one number of requests.  With ``pad_decode`` a batch of
+    # more than PAD_FROM requests is filled up to a multiple of PAD_ROWS with rows of the
+    # runner's own (each a request that stays at its first token), so that batches which
+    # shrink or grow by a request at a time keep meeting recorded shapes.
+    PAD_ROWS = 8
+    PAD_FROM = 16
+
     def __init__(self, model: DecoderModel, page_size: int = 16, num_pages: int = 1024,
-                 num_slots: int = 64, use_graphs: bool = True, portion_graphs: bool = False):
+                 num_slots: int = 64, use_graphs: bool = True, portion_graphs: bool = False,
+                 pad_decode: bool = False):
         """``use_graphs``: replay steps of single tokens as HIP graphs when every part
         of the model declares itself safe to record (``graph_safe``).  ``portion_graphs``:
-        also steps with prompt portions, from the second time a shape is seen."""
+        also steps with prompt portions, from the second time a shape is seen.
+        ``pad_decode``: see ``PAD_ROWS``; the rows take up to ``PAD_ROWS - 1`` of the
+        ``num_slots`` and a page each per cache group until ``release_padding``."""
         self.model = model
         self.device = model.runtime.device
         self.cache = model.make_cache(page_size, num_pages, num_slots)
@@ -40,6 +50,36 @@ class ModelRunner:
         self.portion_graphs = bool(portion_graphs)
         self.graphs = (DecodeGraphs(model.spec.vocab_size, model.item_granularities, model.spec.max_position)
                        if (use_graphs and model.graph_safe) else None)
+
+        self.pad_decode = bool(pad_decode) and self.graphs is not None
+        self._pads: List[Hashable] = []
+
+    # ------------------------------------------------------------- padding rows
+    def padding(self, n_requests: int) -> List[Hashable]:
+        """The requests that fill a decode batch of ``n_requests`` up to a recorded size:
+        admitted, each with the pages of one token, which it never gets beyond.  Empty if
+        the batch needs none, or if slots or pages for them cannot be had (then the rows
+        that were there are given back too)."""
+        if not self.pad_decode or n_requests <= self.PAD_FROM:
+            return []
+        rows = -n_requests % self.PAD_ROWS
+        try:
+            while len(self._pads) < rows:
+                name = ("padding row", id(self), len(self._pads))
+                self.cache.admit(name)
+                self._pads.append(name)
+                self.cache.reserve(name, 1)
+        except (OutOfPages, OutOfSlots):
+            self.release_padding()
+            return []
+        return self._pads[:rows]
+
+    def release_padding(self) -> None:
+        """Give back what the padding rows hold."""
+        pads, self._pads = self._pads, []
+        for name in pads:
+            if name in self.cache.requests:
+                self.cache.release(name)
 
     # ----------------------------------------------------------------- requests
     def admit(self, request: Hashable) -> None:
