@@ -238,16 +238,31 @@ def main() -> int:
                 last.append(int(ops.argmax(logits)[0]))
             requests = list(range(batch))
 
+            greedy = lambda logits, i: ops.argmax(logits)
+            pinned = [torch.empty((8 * batch,), dtype=torch.int32, pin_memory=True) for _ in range(2)]
+
             def run(cur, n):
-                """``n`` decode steps the way generation issues them: greedy tokens handed
-                from step to step on the device, the host reading them every 8 steps."""
-                done = 0
+                """``n`` decode steps the way generation issues them (``Engine``): greedy
+                tokens handed from step to step on the device, in runs of 8; the host reads
+                a run's tokens, from pinned memory behind an event, once the next run is
+                issued."""
+                done, device, waiting, turn = 0, None, None, 0
                 while done < n:
                     k = min(8, n - done)
-                    drawn = runner.decode_steps(requests, cur, k, lambda logits, i: ops.argmax(logits))
-                    cur = drawn[-1].tolist()
-                    done += drawn.shape[0]
-                return cur
+                    drawn = runner.decode_steps(requests, cur, k, greedy, device_tokens=device)
+                    k = drawn.shape[0]
+                    pinned[turn][:k * batch].copy_(drawn.view(-1), non_blocking=True)
+                    event = torch.cuda.Event()
+                    event.record()
+                    if waiting is not None:
+                        waiting[0].synchronize()
+                        waiting[1].tolist()
+                    waiting = (event, pinned[turn][:k * batch])
+                    turn ^= 1
+                    device, cur = drawn[k - 1], None
+                    done += k
+                waiting[0].synchronize()
+                return waiting[1].view(-1, batch)[-1].tolist()
 
             last = run(last, warmup)
             torch.cuda.synchronize()

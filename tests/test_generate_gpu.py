@@ -298,6 +298,18 @@ def test_runs_of_steps_issued_before_the_last_run_is_read():
             return [list(r.output) for r in reqs]
         got = uneven(engine(3))
         assert got == uneven(engine(1)) and [len(g) for g in got] == [30, 11, 23]
+        # a call of step() returns after a bounded number of runs: a request added between
+        # two calls joins then
+        calls = engine(2)
+        calls.RUNS_PER_CALL = 2
+        first = calls.add_request(prompts[0], 30, sampling, eos_token_id=-1)
+        calls.step()                                  # the prompt
+        before = calls.stats()["steps"]
+        calls.step()
+        assert calls.stats()["steps"] - before == 4
+        second = calls.add_request(prompts[1], 11, sampling, eos_token_id=-1)
+        calls.run()
+        assert [first.output, second.output] == got[:2]
         # 14 pages of 8 tokens: the three requests need 6 + 6 + 4 at their ends
         tight = engine(3, num_pages=14)
         assert tight.generate(prompts, max_new_tokens=30, eos_token_id=-1, **kw) == free_run

@@ -44,8 +44,9 @@ class Engine:
         time a shape is seen (see ``DecodeGraphs.run_portions``).
         ``multi_step``: while every running request decodes and none waits, up to this
         many decode steps are issued without the host waiting for the tokens in
-        between (each step's tokens reach the next on the device); a request that
-        meets its stop token inside such a run wastes the steps after it, nothing
+        between (each step's tokens reach the next on the device), and the next such
+        run is issued before the tokens of the last one are read; a request that
+        meets its stop token inside a run wastes the steps issued after it, nothing
         else changes.  1 switches it off, and so does ``on_step``.
         ``on_step(info)``, if given, is called after every step with a dict:
         ``step``, ``plan`` (the scheduled entries), ``logits`` (32-bit, one row per
@@ -101,6 +102,8 @@ class Engine:
         self._token_staging = None       # pinned buffers for the tokens of runs of decode steps
         self._token_turn = 0
         self.warm_up_steps = self.warm_up() if warm_up else 0
+
+    RUNS_PER_CALL = 8                 # runs of ``multi_step`` decode steps in one call of step()
 
     # ----------------------------------------------------------------- warm-up
     WARM_UP_MIN_WEIGHT = 1 << 19      # elements; smaller products are never timed
@@ -176,7 +179,9 @@ class Engine:
         start = time.perf_counter()
         k = self._steps_ahead(plan)
         if k > 1:
-            done = self._decode_many(plan, k, start)
+            # (a call returns after at most RUNS_PER_CALL runs, so that a request added
+            # between two calls waits no longer than that many steps)
+            done = self._decode_many(plan, min(k, self.multi_step * self.RUNS_PER_CALL), start)
             if done and not self.scheduler.has_work():
                 self.runner.release_padding()
             return done
