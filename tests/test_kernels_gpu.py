@@ -588,6 +588,33 @@ def test_steps_of_17_to_32_rows_through_linear(M):
         o.linear_swiglu(x.to(dev()), w.to(dev()))
 
 
+@pytest.mark.parametrize("M,N,K", [(1100, 520, 4096), (2048, 2048, 8192), (1025, 136, 4104)])
+def test_library_product_added_to_the_stream(M, N, K):
+    """Beyond 1,024 rows a product with K >= 4096 that is asked to add itself to the stream
+    does so in the GEMM library (twice in a row: the second is added to the first; timing
+    the library's candidates at the first call leaves the stream alone); a shorter K, or
+    fewer rows, comes back or goes the ways tested above."""
+    o = ops()
+    assert o.library_adds(M, N, K) and not o.library_adds(M, N, 2048) and not o.library_adds(1024, N, K)
+    w = rand((N, K), torch.bfloat16, 140)
+    x = rand((M, K), torch.bfloat16, 141)
+    base = rand((M, N), torch.float32, 142) * 3.0
+    stream = base.clone().to(dev())
+    o.form_log = []
+    try:
+        for _ in range(2):
+            assert o.linear(x.to(dev()), w.to(dev()), partial_ok=True, accumulate=stream) is None
+        log = o.form_log
+    finally:
+        o.form_log = None
+    assert all(r["added_to_stream"] and r.get("kernel") == "library" for r in log[-2:])
+    assert rel_err(stream, base.double() + 2.0 * (x.double() @ w.double().T)) < F32_TOL
+    short = torch.zeros((M, N), dtype=torch.float32, device=dev())
+    back = o.linear(x[:, :2048].contiguous().to(dev()), w[:, :2048].contiguous().to(dev()),
+                    partial_ok=True, accumulate=short)
+    assert back is not None and not short.any()
+
+
 def library_ranges(M, N, K):
     """The documented choice: with few outputs, K >= 4096 goes in 8 ranges up to 256 rows
     and in 4 up to 1,024, K >= 2048 in 4 ranges up to 128 rows; a range is a multiple of

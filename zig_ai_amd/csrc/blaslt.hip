@@ -6,6 +6,8 @@
 //                                              32-bit out
 //   y [P, M, N] (32-bit) with K cut into P ranges, as one batched product: partial
 //                                              sums that the consumer adds up
+//   y [M, N] (32-bit) += x . w^T               the product added to what y holds (the
+//                                              residual stream), the library's beta = 1
 //
 // No device code here.  What a call costs on the host matters for steps of a few
 // hundred tokens, which issue some sixty of these products: the descriptors and the
@@ -58,6 +60,8 @@ struct Plan {
   bool settled = true;   // false: the candidates are still to be timed
   std::vector<hipblasLtMatmulHeuristicResult_t> candidates;
 };
+
+constexpr int OUT_BF16 = 0, OUT_F32 = 1, OUT_ADDED = 2;   // what y is: see the head of this file
 
 constexpr int TUNE_MIN_ROWS = 17;      // (up to 16 rows this package's own kernels run)
 constexpr size_t TUNE_MIN_WEIGHT = (size_t)1 << 19;   // elements: a megabyte of bfloat16; below, nothing to gain
@@ -125,10 +129,10 @@ bool ok(hipblasStatus_t s, const char* what, std::string* why) {
 // Column-major terms: y^T (N x M, leading dimension N) = w (stored K x N, transposed)
 // times x^T (stored K x M).  A range p of K starts p * K/P elements into a row of
 // either operand; its result is the p-th [M, N] block of y.
-bool make_plan(hipblasLtHandle_t handle, int M, int N, int K, int out_f32, int P,
+bool make_plan(hipblasLtHandle_t handle, int M, int N, int K, int out_kind, int P,
                size_t workspace_bytes, bool tune, Plan* plan, std::string* why) {
   const int kp = K / P;
-  const hipDataType out_type = out_f32 ? HIP_R_32F : HIP_R_16BF;
+  const hipDataType out_type = out_kind != OUT_BF16 ? HIP_R_32F : HIP_R_16BF;
   if (!ok(hipblasLtMatmulDescCreate(&plan->op, HIPBLAS_COMPUTE_32F, HIP_R_32F), "MatmulDescCreate", why))
     return false;
   const int32_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
@@ -195,8 +199,26 @@ bool make_plan(hipblasLtHandle_t handle, int M, int N, int K, int out_f32, int P
 constexpr int TUNE_RUNS = 3;
 constexpr int TUNE_COPIES = 7;
 int fastest_candidate(hipblasLtHandle_t handle, const Plan& plan, const void* x, const void* w,
-                      size_t weight_bytes, void* y, void* workspace, size_t workspace_bytes,
-                      hipStream_t stream) {
+                      size_t weight_bytes, void* y, size_t added_bytes, void* workspace,
+                      size_t workspace_bytes, hipStream_t stream) {
+  // a product that is added to y is timed on a y of its own (`added_bytes` of it, zero at
+  // first): the caller's holds what the product proper is to be added to
+  const float* beta = added_bytes ? &kOne : &kZero;
+  struct Release {
+    void* p;
+    ~Release() { if (p) (void)hipFree(p); }
+  };
+  void* own_y = nullptr;
+  if (added_bytes) {
+    if (hipMalloc(&own_y, added_bytes) != hipSuccess ||
+        hipMemsetAsync(own_y, 0, added_bytes, stream) != hipSuccess) {
+      (void)hipGetLastError();
+      if (own_y) (void)hipFree(own_y);
+      return 0;                   // no room: the first answer
+    }
+    y = own_y;
+  }
+  Release release_y{own_y};
   int copies = (int)(TUNE_COPY_BYTES / weight_bytes);
   if (copies > TUNE_COPIES) copies = TUNE_COPIES;
   char* room = nullptr;
@@ -204,10 +226,7 @@ int fastest_candidate(hipblasLtHandle_t handle, const Plan& plan, const void* x,
     (void)hipGetLastError();
     copies = 0;                   // no room: every run on the weight itself
   }
-  struct Release {
-    void* p;
-    ~Release() { if (p) (void)hipFree(p); }
-  } release{room};
+  Release release{room};
   for (int c = 0; c < copies; ++c)
     if (hipMemcpyAsync(room + (size_t)c * weight_bytes, w, weight_bytes, hipMemcpyDeviceToDevice,
                        stream) != hipSuccess) {
@@ -233,13 +252,13 @@ int fastest_candidate(hipblasLtHandle_t handle, const Plan& plan, const void* x,
     // (the clocks come up under the first runs: the first candidate is not to pay for that)
     hipblasLtMatmulAlgo_t algo = plan.candidates[0].algo;
     for (int r = 0; r < 4; ++r)
-      (void)hipblasLtMatmul(handle, plan.op, &kOne, next_weight(), plan.a, x, plan.b, &kZero, y, plan.c,
+      (void)hipblasLtMatmul(handle, plan.op, &kOne, next_weight(), plan.a, x, plan.b, beta, y, plan.c,
                             y, plan.c, &algo, workspace, workspace_bytes, stream);
   }
   for (size_t i = 0; i < plan.candidates.size(); ++i) {
     hipblasLtMatmulAlgo_t algo = plan.candidates[i].algo;
     auto run = [&]() {
-      return hipblasLtMatmul(handle, plan.op, &kOne, next_weight(), plan.a, x, plan.b, &kZero, y,
+      return hipblasLtMatmul(handle, plan.op, &kOne, next_weight(), plan.a, x, plan.b, beta, y,
                              plan.c, y, plan.c, &algo, workspace, workspace_bytes,
                              stream) == HIPBLAS_STATUS_SUCCESS;
     };
@@ -273,11 +292,14 @@ ZA_API const char* za_lt_last_error() { return g_error.c_str(); }
 // Returns 0, ZA_ERR_ARG, ZA_ERR_UNSUPPORTED (the library has no algorithm for the
 // shape: nothing was launched) or a positive hipBLAS status.
 // `tune`: see the head of this file.
-ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int K, int out_f32,
+// `out_kind`: 0 bfloat16, 1 32-bit, 2 32-bit added to what y holds (P = 1).
+ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int K, int out_kind,
                         int P, int tune, void* workspace, size_t workspace_bytes,
                         hipStream_t stream) {
-  if (!x || !w || !y || M < 1 || N < 1 || K < 1 || P < 1 || K % P || (P > 1 && !out_f32))
+  if (!x || !w || !y || M < 1 || N < 1 || K < 1 || P < 1 || K % P || out_kind < OUT_BF16 ||
+      out_kind > OUT_ADDED || (P > 1 && out_kind != OUT_F32))
     return fail(ZA_ERR_ARG, "za_lt_matmul: bad argument");
+  const float* beta = out_kind == OUT_ADDED ? &kOne : &kZero;
   int device = 0;
   if (hipGetDevice(&device) != hipSuccess) return fail(ZA_ERR_ARG, "za_lt_matmul: no current device");
   Plan plan;
@@ -293,18 +315,18 @@ ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int
     }
     handle = h->second;
     const bool tuning = tune && M >= TUNE_MIN_ROWS && (size_t)N * K >= TUNE_MIN_WEIGHT;
-    const Key key(device, M, N, K, out_f32, P, tuning ? 1 : 0);
+    const Key key(device, M, N, K, out_kind, P, tuning ? 1 : 0);
     auto it = g_plans.find(key);
     if (it == g_plans.end()) {
       Plan made;
       std::string why;
-      if (!make_plan(handle, M, N, K, out_f32, P, workspace_bytes, tuning, &made, &why))
+      if (!make_plan(handle, M, N, K, out_kind, P, workspace_bytes, tuning, &made, &why))
         return fail(ZA_ERR_ARG, "za_lt_matmul: " + why);
       it = g_plans.emplace(key, made).first;
     }
     Plan& kept = it->second;
     if (kept.usable && !kept.settled) {
-      const TunedKey block(device, tune_block(M), N, K, out_f32, P);
+      const TunedKey block(device, tune_block(M), N, K, out_kind, P);
       auto choose = [&](size_t i) {
         kept.algo = kept.candidates[i].algo;
         kept.workspace = kept.candidates[i].workspaceSize;
@@ -324,11 +346,13 @@ ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int
       } else if (!recording) {
         const auto began = std::chrono::steady_clock::now();
         const int best = fastest_candidate(handle, kept, x, w, (size_t)N * K * sizeof(uint16_t), y,
+                                           out_kind == OUT_ADDED ? (size_t)M * N * sizeof(float) : 0,
                                            workspace, workspace_bytes, stream);
         choose((size_t)best);
         if (tune_log())
           fprintf(stderr, "[zig_ai_amd] timed %zu candidates for M=%d N=%d K=%d P=%d %s: answer %d in %.1f ms\n",
-                  kept.candidates.size(), M, N, K, P, out_f32 ? "f32" : "bf16", best,
+                  kept.candidates.size(), M, N, K, P,
+                  out_kind == OUT_ADDED ? "added to f32" : out_kind == OUT_F32 ? "f32" : "bf16", best,
                   std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - began).count());
         g_tuned.emplace(block, hipblaslt_ext::getIndexFromAlgo(kept.algo));
       }
@@ -345,7 +369,7 @@ ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int
   hipblaslt_ext::Gemm* instance = nullptr;
   {
     std::lock_guard<std::mutex> guard(g_lock);
-    const InstanceKey ikey(Key(device, M, N, K, out_f32, P,
+    const InstanceKey ikey(Key(device, M, N, K, out_kind, P,
                                tune && M >= TUNE_MIN_ROWS && (size_t)N * K >= TUNE_MIN_WEIGHT ? 1 : 0),
                            x, w, y, workspace);
     auto it = g_instances.find(ikey);
@@ -363,7 +387,7 @@ ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int
     } else {
       if (!it->second) {
         std::unique_ptr<hipblaslt_ext::Gemm> made(new hipblaslt_ext::Gemm(
-            handle, plan.op, &kOne, w, plan.a, x, plan.b, &kZero, y, plan.c, y, plan.c));
+            handle, plan.op, &kOne, w, plan.a, x, plan.b, beta, y, plan.c, y, plan.c));
         hipblasLtMatmulAlgo_t algo = plan.algo;
         if (made->initialize(algo, workspace) == HIPBLAS_STATUS_SUCCESS) it->second = std::move(made);
       }
@@ -372,7 +396,7 @@ ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int
   }
   const hipblasStatus_t s =
       instance ? instance->run(stream)
-               : hipblasLtMatmul(handle, plan.op, &kOne, w, plan.a, x, plan.b, &kZero, y, plan.c, y,
+               : hipblasLtMatmul(handle, plan.op, &kOne, w, plan.a, x, plan.b, beta, y, plan.c, y,
                                  plan.c, &plan.algo, workspace, workspace_bytes, stream);
   if (s != HIPBLAS_STATUS_SUCCESS)
     return fail((int)s > 0 ? (int)s : ZA_ERR_ARG,

@@ -396,9 +396,11 @@ library_tuning = os.environ.get("ZIG_AI_GEMM_TUNE", "1") != "0"
 
 
 def _library_matmul(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype,
-                    splits: int, tune: Optional[bool] = None) -> Optional[torch.Tensor]:
+                    splits: int, tune: Optional[bool] = None,
+                    added_to: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """``x @ weight^T`` through the GEMM library (csrc/blaslt.hip): ``[M, N]``, or the
-    stack ``[splits, M, N]`` of 32-bit partial sums over ranges of K.  ``None`` when
+    stack ``[splits, M, N]`` of 32-bit partial sums over ranges of K, or, with ``added_to``
+    (32-bit ``[M, N]``), that tensor with the product added to it.  ``None`` when
     the library names no algorithm for the shape (nothing was launched)."""
     M, K = x.shape
     N = weight.shape[0]
@@ -408,9 +410,13 @@ def _library_matmul(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtyp
         work = torch.empty((LIBRARY_WORKSPACE_BYTES,), dtype=torch.uint8, device=x.device)
         _library_workspace[device] = work
     f32 = splits > 1 or out_dtype == torch.float32
-    shape = (splits, M, N) if splits > 1 else (M, N)
-    out = torch.empty(shape, dtype=torch.float32 if f32 else torch.bfloat16, device=x.device)
-    rc = _fn("blaslt", "za_lt_matmul")(_ptr(x), _ptr(weight), _ptr(out), M, N, K, 1 if f32 else 0,
+    if added_to is not None:
+        out, kind = added_to, 2
+    else:
+        shape = (splits, M, N) if splits > 1 else (M, N)
+        out = torch.empty(shape, dtype=torch.float32 if f32 else torch.bfloat16, device=x.device)
+        kind = 1 if f32 else 0
+    rc = _fn("blaslt", "za_lt_matmul")(_ptr(x), _ptr(weight), _ptr(out), M, N, K, kind,
                                        splits, 1 if (library_tuning if tune is None else tune) else 0,
                                        _ptr(work),
                                        LIBRARY_WORKSPACE_BYTES, _stream())
@@ -454,6 +460,19 @@ def _merged_splits(N: int, K: int) -> int:
         if K % (split * 512) == 0 and K // split <= 4096 and (groups * split <= 640 or split == 1):
             return split
     return 0
+
+
+LIBRARY_ADDS_MIN_K = 4096
+
+
+def library_adds(M: int, N: int, K: int) -> bool:
+    """Whether a product of this shape, asked to add itself to the 32-bit stream, does so
+    through the GEMM library (its beta = 1): beyond the rows whose K the library gets in
+    ranges, and with K long enough that reading and writing the stream in the product's
+    epilogue costs less than the next norm saves by not adding (measured at 2,048 rows:
+    [2048, 8192] 75 us against 79 into bfloat16, the norm after it 4.8 us against 7.7;
+    [2048, 2048] 25.5 against 22.2, which the norm does not win back)."""
+    return M > LIBRARY_SPLIT_ROWS and K >= LIBRARY_ADDS_MIN_K and K % 8 == 0
 
 
 def accumulate_plan(M: int, N: int, K: int, normed: bool) -> int:
@@ -536,6 +555,15 @@ def linear(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
         _note("linear", M=M, N=N, K=K, norm_in_product=False, added_to_stream=True,
               partial_sums=1, out=accumulate.dtype, kernel="rows64")
         return None
+    if accumulate is not None and library_adds(M, N, K) and normed is None and bias is None \
+            and weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and not force_tiled:
+        # many rows and a long K: the library adds its product to the stream itself
+        _need(weight, "weight", torch.bfloat16, (N, K))
+        _need(accumulate, "accumulate", torch.float32, (M, N))
+        if _library_matmul(x, weight, torch.float32, 1, tune, added_to=accumulate) is not None:
+            _note("linear", M=M, N=N, K=K, norm_in_product=False, added_to_stream=True,
+                  partial_sums=1, out=accumulate.dtype, kernel="library")
+            return None
     if accumulate is not None:
         if weight.dtype == torch.bfloat16 and not force_tiled \
                 and (normed is not None or x.dtype == torch.bfloat16):
