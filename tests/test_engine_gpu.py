@@ -836,6 +836,38 @@ def test_decode_batches_with_padding_rows(dtype):
         assert all(g["pages_free"] == g["pages"] for g in stats["groups"])
 
 
+def test_padding_rows_give_their_pages_back_when_requests_need_them():
+    """17 requests and 7 padding rows in a pool with ten pages to spare: when every request
+    needs its second page the padding rows' pages are what is missing; they are given back,
+    the step runs without them, and so do the later ones (no page is left for such rows)."""
+    from zig_ai_amd.engine import ModelRunner, StepEntry
+    model, _, _ = setup("A", "float32")
+    cfg, seed = CONFIGS["A"]
+    oracle = plain.PlainLfm2(eu.model_folder(cfg, seed, torch.float32, **eu.sharp_kwargs()))
+    ids = list(range(17))
+    seqs = [eu.random_tokens(3 + 4, cfg["vocab_size"], 7100 + i) for i in ids]
+    expect = [oracle.logits(q) for q in seqs]
+    runner = ModelRunner(model, page_size=4, num_pages=17 + 7 + 10, num_slots=24, pad_decode=True)
+    for r, q in zip(ids, seqs):
+        runner.admit(r)
+        runner.step([StepEntry(r, q[:3], [])])
+    shapes = []
+    for j in range(4):
+        logits = runner.step([StepEntry(r, [seqs[r][3 + j]], [0]) for r in ids])
+        shapes.append(len(runner._pads))
+        for r in ids:
+            assert eu.rel_err(logits[r], expect[r][3 + j]) < TOL["float32"], (j, r)
+        runner.cache.check()
+    # position 3 fills the first page (7 rows beside the requests), position 4 needs the second
+    assert shapes == [7, 0, 0, 0]
+    assert {key[0] for key in runner.graphs.entries} == {24, 17}
+    for r in ids:
+        runner.release(r)
+    runner.release_padding()
+    stats = runner.cache.stats()
+    assert stats["requests"] == 0 and all(g["pages_free"] == g["pages"] for g in stats["groups"])
+
+
 def test_recorded_shapes_are_dropped_when_there_are_too_many(monkeypatch):
     """Only so many recorded steps are kept; the one used longest ago goes, and comes
     back (recorded anew) when its shape does.  Three batch sizes in turn, three steps
