@@ -72,9 +72,9 @@ SHAPES = {
 }
 
 
-def serve(cfg, name, n_requests, new_tokens, portion_graphs=False, chunk_size=None) -> int:
+def serve(cfg, name, n_requests, new_tokens, portion_graphs=False, chunk_size=None) -> dict:
     """Requests with prompts of 128 to 2,048 tokens through the scheduler, the step
-    function and the sampler (temperature 0.7), all admitted at once."""
+    function and the sampler (temperature 0.7), all admitted at once.  Returns the record."""
     import random
     import tempfile
 
@@ -100,21 +100,28 @@ def serve(cfg, name, n_requests, new_tokens, portion_graphs=False, chunk_size=No
         # the shape's first call (some 10 ms each; a server does that once in its life)
         engine.generate(prompts, max_new_tokens=new_tokens, temperature=0.7, seed=3, eos_token_id=-1)
         torch.cuda.synchronize()
+        before = dict(engine.stats())
         t0 = time.perf_counter()
         out = engine.generate(prompts, max_new_tokens=new_tokens, temperature=0.7, seed=3,
                               eos_token_id=-1)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         stats = engine.stats()
+        chunk = engine.scheduler.chunk_size
+        del engine
+        torch.cuda.empty_cache()
     prompt_tokens, generated = sum(len(p) for p in prompts), sum(len(o) for o in out)
-    print(json.dumps({
+    with_prompts = stats["seconds_with_prompts"] - before["seconds_with_prompts"]
+    return {
         "workload": "serve", "model": f"LFM2-{name} shape", "requests": n_requests,
         "prompt_tokens": prompt_tokens, "generated_tokens": generated, "seconds": dt,
         "generated_per_s": generated / dt, "tokens_per_s": (prompt_tokens + generated) / dt,
-        "steps": stats["steps"], "preemptions": stats["preemptions"], "dtype": "bf16",
-        "chunk_size": engine.scheduler.chunk_size,
-        "data": "synthetic token ids; random weights N(0, 0.02)"}), flush=True)
-    return 0
+        # steps that held prompt portions (beside decoding requests), and the rest
+        "seconds_in_steps_with_prompts": with_prompts,
+        "seconds_in_decode_steps": stats["step_seconds"] - before["step_seconds"] - with_prompts,
+        "steps": stats["steps"] - before["steps"], "preemptions": stats["preemptions"],
+        "dtype": "bf16", "chunk_size": chunk,
+        "data": "synthetic token ids; random weights N(0, 0.02)"}
 
 
 def count_bytes(model):
@@ -191,8 +198,9 @@ def main() -> int:
     torch.cuda.set_device(0)
     cfg = dict(SHAPES[args.shape])
     if args.workload == "serve":
-        return serve(cfg, args.shape.upper(), args.requests, args.new_tokens, args.portion_graphs,
-                     args.chunk_size)
+        print(json.dumps(serve(cfg, args.shape.upper(), args.requests, args.new_tokens,
+                               args.portion_graphs, args.chunk_size)), flush=True)
+        return 0
     full_layers = cfg["num_hidden_layers"]
     if args.layers is not None and args.layers < full_layers:
         cfg["num_hidden_layers"] = args.layers
@@ -379,6 +387,11 @@ def main() -> int:
                 shapes[name] = detail
                 del other
                 torch.cuda.empty_cache()
+            # and the mixed workload of the 350M shape: 64 requests through the scheduler
+            record = serve(dict(SHAPES["350m"]), "350M", 64, 256)
+            shapes["350m"]["serve"] = {k: record[k] for k in (
+                "requests", "prompt_tokens", "generated_tokens", "seconds", "generated_per_s",
+                "tokens_per_s", "seconds_in_steps_with_prompts", "seconds_in_decode_steps", "steps")}
 
     vocab, hd, n_attn = cfg["vocab_size"], main_shape.hd, main_shape.n_attn
     line = {

@@ -96,7 +96,10 @@ class Engine:
         self.scheduler = Scheduler(self.runner.cache, max_num_seqs, max_num_batched_tokens,
                                    chunk_size, limit)
         self._next_id = 0
-        self.timings = {"steps": 0, "step_seconds": 0.0, "tokens_run": 0, "tokens_generated": 0}
+        # (seconds_with_prompts: the part of step_seconds spent in steps that held prompt
+        # portions; the rest went to steps of decoding requests only)
+        self.timings = {"steps": 0, "step_seconds": 0.0, "seconds_with_prompts": 0.0,
+                        "tokens_run": 0, "tokens_generated": 0}
         self.max_num_batched_tokens = int(max_num_batched_tokens)
         self.max_num_seqs = int(max_num_seqs)
         self._token_staging = None       # pinned buffers for the tokens of runs of decode steps
@@ -201,6 +204,8 @@ class Engine:
         self.timings["steps"] += 1
         elapsed = time.perf_counter() - start
         self.timings["step_seconds"] += elapsed
+        if any(e.count > 1 or not e.samples or e.start == 0 for e in plan):
+            self.timings["seconds_with_prompts"] += elapsed
         if self.on_step is not None:
             self.on_step({"step": self.timings["steps"] - 1, "plan": plan, "logits": logits,
                           "tokens": drawn, "seconds": elapsed})
