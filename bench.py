@@ -368,6 +368,11 @@ def main() -> int:
             d, ctx = main_shape.decode_run(b, args.prompt_len, steps, 4)
             points[f"decode_b{b}"] = b * steps / d
             points_detail[f"decode_b{b}"] = main_shape.against_memory(b, d / steps, ctx, calibration)
+        # the batch sizes between: the last that this package's kernels for up to 16 rows
+        # take, and the steps of 17 to 32 rows
+        for b in (16, 24, 32):
+            d, ctx = main_shape.decode_run(b, args.prompt_len, 32, 4)
+            points_detail[f"decode_b{b}"] = main_shape.against_memory(b, d / 32, ctx, calibration)
         # further contexts (prefilled to there, 16 steps each)
         for b, ctx0 in ((8, 4096), (8, 8192), (64, 4096)):
             d, ctx = main_shape.decode_run(b, ctx0, 16, 4)
