@@ -183,6 +183,8 @@ def main() -> int:
     ap.add_argument("--phase", choices=["all", "prefill", "decode"], default="all",
                     help="measure only one phase (for profiling); the JSON line then holds "
                          "only that phase")
+    ap.add_argument("--prefill-tokens", type=int, default=2048,
+                    help="--phase prefill: the prompt's length (in steps of 2,048 tokens)")
     ap.add_argument("--tuned", action="store_true",
                     help="with --phase: let the GEMM library time its candidates as a plain run "
                          "does (not under a profiler's counters)")
@@ -342,7 +344,8 @@ def main() -> int:
                           "value": args.batch * args.steps / dt, "unit": "tokens/s"}), flush=True)
         return 0
     if args.phase == "prefill":
-        print(json.dumps({"phase": "prefill", **main_shape.prefill_run(T, T, None)}), flush=True)
+        print(json.dumps({"phase": "prefill",
+                          **main_shape.prefill_run(args.prefill_tokens, T, None)}), flush=True)
         return 0
 
     # ---- what this GPU does at best
