@@ -184,7 +184,8 @@ def main() -> int:
                     help="measure only one phase (for profiling); the JSON line then holds "
                          "only that phase")
     ap.add_argument("--prefill-tokens", type=int, default=2048,
-                    help="--phase prefill: the prompt's length (in steps of 2,048 tokens)")
+                    help="--phase prefill: the prompt's length (in steps of 2,048 tokens, or of "
+                    "--chunk-size)")
     ap.add_argument("--tuned", action="store_true",
                     help="with --phase: let the GEMM library time its candidates as a plain run "
                          "does (not under a profiler's counters)")
@@ -345,7 +346,8 @@ def main() -> int:
         return 0
     if args.phase == "prefill":
         print(json.dumps({"phase": "prefill",
-                          **main_shape.prefill_run(args.prefill_tokens, T, None)}), flush=True)
+                          **main_shape.prefill_run(args.prefill_tokens, args.chunk_size or T, None)}),
+              flush=True)
         return 0
 
     # ---- what this GPU does at best
