@@ -72,3 +72,16 @@ def test_where_the_kernel_for_17_to_64_rows_is_taken():
         for N in (1024, 2048, 4096):
             ks = ops.rows64_add_splits(N, K)
             assert ks == 0 or ops.rows64_takes(32, K, ks)
+
+
+def test_where_the_library_adds_a_product_to_the_stream_itself():
+    """Beyond the rows whose K the library gets in ranges, and only with a long K (the
+    feed-forward's closing product): elsewhere the product comes back and the next norm
+    adds it."""
+    assert ops.library_adds(2048, 2048, 8192) and ops.library_adds(1025, 1024, 4608)
+    assert ops.library_adds(4096, 2560, 10752)
+    assert not ops.library_adds(2048, 2048, 2048)          # the mixers' closing products
+    assert not ops.library_adds(1024, 2048, 8192)          # K in ranges instead
+    assert not ops.library_adds(2048, 2048, 4100)          # rows that do not start on 16 bytes
+    for M in (17, 64, 512, 1024):
+        assert not ops.library_adds(M, 2048, 8192)
