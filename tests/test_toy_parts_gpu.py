@@ -4,7 +4,8 @@ model folder, and stepped through the engine's step function, cache manager and
 run order without a change to the framework's files.  Also: a run order that
 names a layer twice, and a layer that reads another layer's cache; and a second
 toy architecture with a feed-forward that routes tokens to experts and a position
-encoding of another kind, beside the framework's own ShortConv mixer.
+encoding of another kind, beside the framework's own ShortConv mixer; and a norm, an
+embedding and a head of another kind around the framework's own layers.
 """
 
 import pytest
@@ -521,6 +522,189 @@ def test_a_nested_position_part_decides_whether_steps_are_recorded():
                                    21, torch.float32, **eu.sharp_kwargs())
     rotary = plain.PlainLfm2(plain_folder).logits(tokens)[19:]
     assert eu.rel_err(outs["toy_added_waves"], rotary) > 1e-2
+
+
+# ------------------------- another norm, another embedding and another head around LFM2's layers
+def capped_classes():
+    from zig_ai_amd.kernels import ops
+    from zig_ai_amd.parts import (Norm, Part, TensorRule, register_embedding, register_head,
+                                  register_norm)
+
+    class CenteredNorm(Norm):
+        """``(x - mean) / sqrt(var + eps) * weight + bias`` over the last axis, in 32-bit.  It
+        has no fused forms: the base class adds what is pending to the stream and calls
+        ``forward``; the parts behind it receive plain activations."""
+        kind = "toy_centered_norm"
+        graph_safe = True
+
+        @classmethod
+        def tensor_rules(cls, params):
+            w = int(params["width"])
+            return {"weight": TensorRule(((w,),), role="norm"), "bias": TensorRule(((w,),), role="bias")}
+
+        def __init__(self, params, tensors, runtime):
+            super().__init__(params, tensors, runtime)
+            self.eps = float(params["eps"])
+            self.weight, self.bias = tensors["weight"], tensors["bias"]
+
+        def forward(self, x):
+            x = x.float()
+            x = x - x.mean(dim=-1, keepdim=True)
+            y = x * torch.rsqrt((x * x).mean(dim=-1, keepdim=True) + self.eps)
+            return (y * self.weight + self.bias).to(self.runtime.dtype)
+
+    class ScaledEmbedding(Part):
+        """The table's row times ``sqrt(width)``."""
+        kind = "toy_scaled_embedding"
+        graph_safe = True
+        kernel_sources = ("norm",)
+
+        @classmethod
+        def tensor_rules(cls, params):
+            return {"weight": TensorRule(((int(params["vocab_size"]), int(params["hidden_size"])),),
+                                         role="table")}
+
+        def __init__(self, params, tensors, runtime):
+            super().__init__(params, tensors, runtime)
+            self.weight = tensors["weight"]
+            self.scale = float(params["hidden_size"]) ** 0.5
+
+        def forward(self, token_ids):
+            return ops.embed_gather(token_ids, self.weight) * self.scale
+
+    class CappedHead(Part):
+        """``cap * tanh(logits / cap)``: logits that cannot leave (-cap, cap)."""
+        kind = "toy_capped_head"
+        graph_safe = True
+        kernel_sources = ("gemm",)
+
+        @classmethod
+        def tensor_rules(cls, params):
+            return {"weight": TensorRule(((int(params["vocab_size"]), int(params["hidden_size"])),),
+                                         role="table")}
+
+        def __init__(self, params, tensors, runtime):
+            super().__init__(params, tensors, runtime)
+            self.weight = tensors["weight"]
+            self.cap = float(params["cap"])
+
+        def forward(self, x):
+            logits = ops.linear(x, self.weight, out_dtype=torch.float32)
+            return torch.tanh(logits / self.cap) * self.cap
+
+    register_norm(CenteredNorm.kind, CenteredNorm)
+    register_embedding(ScaledEmbedding.kind, ScaledEmbedding)
+    register_head(CappedHead.kind, CappedHead)
+
+
+class CappedLfm2Config:
+    """LFM2's mixers and feed-forwards between a scaled embedding, centered norms with a
+    bias everywhere, and a head with capped logits."""
+
+    def __init__(self, data):
+        self.data = dict(data)
+
+    @classmethod
+    def from_dict(cls, data):
+        return cls(data)
+
+    def to_dict(self):
+        return dict(self.data)
+
+    def to_spec(self):
+        import dataclasses
+
+        from zig_ai_amd.config.lfm2 import Lfm2Config
+        from zig_ai_amd.config.spec import LayerSpec, PartSpec
+        inner = dict(self.data, architectures=["Lfm2ForCausalLM"], tie_embedding=False)
+        cap = inner.pop("logit_cap")
+        spec = Lfm2Config.from_dict(inner).to_spec()
+
+        def centered(norm):
+            name = norm.tensors["weight"][0]
+            return PartSpec("toy_centered_norm", dict(norm.params),
+                            {"weight": (name,), "bias": (name[:-len("weight")] + "bias",)})
+        layers = []
+        for layer in spec.layers:
+            parts = dict(layer.parts)
+            for name in ("mixer_norm", "feed_forward_norm"):
+                parts[name] = centered(parts[name])
+            layers.append(LayerSpec(parts, layer.arrangement))
+        head = PartSpec("toy_capped_head", dict(spec.lm_head.params, cap=cap), dict(spec.lm_head.tensors))
+        return dataclasses.replace(
+            spec, architecture=self.data["architectures"][0], layers=tuple(layers),
+            embedding=PartSpec("toy_scaled_embedding", dict(spec.embedding.params),
+                               dict(spec.embedding.tensors)),
+            final_norm=centered(spec.final_norm), lm_head=head)
+
+
+CAPPED = {"architectures": ["ToyCappedForCausalLM"], "model_type": "lfm2", "hidden_size": 72,
+          "num_hidden_layers": 3, "num_attention_heads": 3, "num_key_value_heads": 1, "head_dim": 32,
+          "vocab_size": 131, "layer_types": ["conv", "full_attention", "conv"],
+          "intermediate_size": 104, "rope_theta": 10000.0, "norm_eps": 1e-5, "conv_L_cache": 4,
+          "conv_bias": True, "max_position_embeddings": 512, "logit_cap": 3.0}
+
+
+def capped_oracle(folder, tokens):
+    """The model in float64, written out with the plain implementation's mixers."""
+    from safetensors.torch import load_file
+    w = {k: v.double() for k, v in load_file(folder + "/model.safetensors").items()}
+    spec = CappedLfm2Config(CAPPED).to_spec()
+    lfm2 = plain.PlainLfm2.__new__(plain.PlainLfm2)              # its naming of a layer's tensors
+    lfm2.w, lfm2.H = w, CAPPED["hidden_size"]
+    lfm2.kinds = ["attention" if t == "full_attention" else "conv" for t in CAPPED["layer_types"]]
+
+    def centered(x, part):
+        x = x - x.mean(dim=-1, keepdim=True)
+        y = x / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + CAPPED["norm_eps"])
+        return y * w[part.tensors["weight"][0]] + w[part.tensors["bias"][0]]
+
+    x = w[spec.embedding.tensors["weight"][0]][torch.tensor(tokens)] * CAPPED["hidden_size"] ** 0.5
+    pos = torch.arange(len(tokens))
+    for i, layer in enumerate(spec.layers):
+        lw = lfm2.layer_weights(i)
+        n1 = centered(x, layer.mixer_norm)
+        if lfm2.kinds[i] == "attention":
+            m = plain.attention_mixer(n1, lw, pos, CAPPED["num_attention_heads"], CAPPED["num_key_value_heads"],
+                                      CAPPED["head_dim"], CAPPED["norm_eps"], CAPPED["rope_theta"])
+        else:
+            m = plain.short_conv_mixer(n1, lw)
+        x = x + m
+        ff = layer.feed_forward.tensors
+        x = x + plain.swiglu_ffn(centered(x, layer.feed_forward_norm), w[ff["gate.weight"][0]],
+                                 w[ff["up.weight"][0]], w[ff["down.weight"][0]])
+    logits = centered(x, spec.final_norm) @ w[spec.lm_head.tensors["weight"][0]].T
+    return torch.tanh(logits / CAPPED["logit_cap"]) * CAPPED["logit_cap"]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_another_norm_embedding_and_head(dtype):
+    """A norm, an embedding and a head defined here, registered from outside, around the
+    framework's own mixers and feed-forwards: built from a folder that the random model
+    writer made from the same spec (it asks the parts for their tensors, the norm's bias
+    among them), stepped whole, in portions and mixed, recorded and replayed."""
+    from zig_ai_amd.config import register_architecture
+    from zig_ai_amd.engine import DecoderModel, ModelRunner
+    capped_classes()
+    register_architecture("ToyCappedForCausalLM", CappedLfm2Config)
+    store = torch.float32 if dtype == "float32" else torch.bfloat16
+    folder = eu.model_folder(CAPPED, 31, store, std=0.2, norm_init="around_one",
+                             role_std={"norm": 0.2, "bias": 0.3, "table": 0.1,
+                                       "q_proj.weight": 0.08, "k_proj.weight": 0.08})
+    model = DecoderModel.from_folder(folder, dtype)
+    assert model.graph_safe
+    lengths = [33, 7, 20]
+    prompts = [eu.random_tokens(n, CAPPED["vocab_size"], 800 + n) for n in lengths]
+    expect = [capped_oracle(folder, p) for p in prompts]
+    assert max(float(e.abs().max()) for e in expect) > 0.7 * CAPPED["logit_cap"]   # the cap is at work
+    tol = 1e-4 if dtype == "float32" else 2.5e-2
+    for schedule in (eu.whole(lengths), eu.changing_portions(lengths, 1),
+                     eu.mixed(lengths, seed=9, max_live=3, decode_tail=6)):
+        runner = ModelRunner(model, page_size=4, num_pages=24, num_slots=3)
+        got = eu.run_schedule(runner, prompts, schedule)
+        for g, e in zip(got, expect):
+            assert eu.rel_err(g, e) < tol
+    assert runner.graphs is not None and runner.graphs.replays > 0
 
 
 # ---------- another arrangement (four norms, two mixers), a mixer that pages ONE vector
