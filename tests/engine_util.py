@@ -168,6 +168,8 @@ class Forms:
                 self.seen.add("decode attention of many rows, contexts uncut")
             if r["op"] == "linear" and r["M"] > 16 and r["partial_sums"] > 1:
                 self.seen.add("library product with ranges of K")
+            if r["op"] == "linear" and r.get("kernel") == "library" and r["added_to_stream"]:
+                self.seen.add("library product added to the stream")
         if products:
             L = self.n_layers
             assert len(products) == 4 * L + (1 if wanted_rows else 0), \

@@ -543,6 +543,9 @@ def test_decoding_at_a_context_beyond_2048_at_real_layer_sizes(dtype):
         assert "ranges merged by the combine kernel" in forms.seen
         assert "decode attention of many rows, contexts uncut" in forms.seen
         assert "library product with ranges of K" in forms.seen
+        # (the long request's first step, more than 1,024 rows: w2 added to the stream by
+        # the library itself)
+        assert "library product added to the stream" in forms.seen
     replaying = ModelRunner(model, page_size=16, num_pages=pages, num_slots=SHORT_REQUESTS + 1)
     again = eu.run_schedule(replaying, prompts, schedule, wants=wants)
     assert replaying.graphs.captures >= 2 and replaying.graphs.replays >= 24
