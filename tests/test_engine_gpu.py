@@ -839,6 +839,35 @@ def test_decode_batches_with_padding_rows(dtype):
         assert all(g["pages_free"] == g["pages"] for g in stats["groups"])
 
 
+def test_a_batch_that_stays_gets_a_recording_of_its_own(monkeypatch):
+    """A batch that is filled up with padding rows runs them at every step; once it has come
+    as it is more often than ``PROMOTE_AFTER`` it is recorded without them."""
+    from zig_ai_amd.engine import ModelRunner, StepEntry, graphs
+    monkeypatch.setattr(graphs, "PROMOTE_AFTER", 2)
+    model, _, _ = setup("D", "float32")
+    cfg, seed = CONFIGS["D"]
+    oracle = plain.PlainLfm2(eu.model_folder(cfg, seed, torch.float32, **eu.sharp_kwargs()))
+    ids = list(range(19))
+    new = 7
+    seqs = [eu.random_tokens(4 + r % 5 + new, cfg["vocab_size"], 7300 + r) for r in ids]
+    expect = [oracle.logits(q) for q in seqs]
+    runner = ModelRunner(model, page_size=8, num_pages=160, num_slots=19 + 7, pad_decode=True)
+    for r, q in zip(ids, seqs):
+        runner.admit(r)
+        runner.step([StepEntry(r, q[:len(q) - new], [])])
+    sizes = []
+    for j in range(new):
+        logits = runner.step([StepEntry(r, [seqs[r][len(seqs[r]) - new + j]], [0]) for r in ids])
+        for r in ids:
+            assert eu.rel_err(logits[r], expect[r][len(seqs[r]) - new + j]) < TOL["float32"], (j, r)
+        sizes.append(sorted(key[0] for key, slot in runner.graphs.entries.items()
+                            if slot["graph"] is not None))
+    # two steps filled up to 24 (the second records that shape), then the batch of 19 as it
+    # is: run, recorded, replayed
+    assert sizes == [[], [24], [24], [19, 24], [19, 24], [19, 24], [19, 24]], sizes
+    assert runner.graphs.captures == 2 and runner.graphs.replays == 1 + 4
+
+
 def test_padding_rows_give_their_pages_back_when_requests_need_them():
     """17 requests and 7 padding rows in a pool with ten pages to spare: when every request
     needs its second page the padding rows' pages are what is missing; they are given back,
@@ -851,6 +880,7 @@ def test_padding_rows_give_their_pages_back_when_requests_need_them():
     seqs = [eu.random_tokens(3 + 4, cfg["vocab_size"], 7100 + i) for i in ids]
     expect = [oracle.logits(q) for q in seqs]
     runner = ModelRunner(model, page_size=4, num_pages=17 + 7 + 10, num_slots=24, pad_decode=True)
+    runner.PAD_SPARE_PAGES = 0               # (by itself a runner takes no such rows in so small a pool)
     for r, q in zip(ids, seqs):
         runner.admit(r)
         runner.step([StepEntry(r, q[:3], [])])

@@ -33,6 +33,10 @@ PAGE_BUCKET = 64        # block-table width is rounded up to a multiple of this
 KEYS_BUCKET = 1024      # and the longest context to a multiple of this
 MAX_GRAPHS = 96         # recorded shapes kept; the one replayed longest ago goes first
 MAX_PORTION_GRAPHS = 24 # the same for steps with prompt portions (their tensors are larger)
+# A batch that a runner fills up with rows of its own (``ModelRunner.padding``) gets a
+# recording without those rows once it has come this often as it is: recording costs about
+# 2 ms, the rows some 0.01 ms each a step.
+PROMOTE_AFTER = 64
 # Steps with prompt portions are recorded only where the host is the limit (beyond some
 # 1,000 tokens a step is bound by the GPU and a recording would only hold memory), and
 # the recorded steps together hold at most this many bytes of intermediate tensors: the
@@ -60,6 +64,7 @@ class DecodeGraphs:
         self._lib = hostlib.lib()
         self.captures = 0
         self.replays = 0
+        self._unpadded_sightings: Dict[Tuple[int, int, int], int] = {}
         # steps of any other shape (prompt portions, alone or beside single tokens)
         self.portion_entries: Dict[tuple, dict] = {}          # in order of last use
         self.portion_captures = 0
@@ -107,45 +112,75 @@ class DecodeGraphs:
         last one is still running.
 
         A runner that pads its decode batches (``ModelRunner.padding``) adds rows of its
-        own behind the entries (unless ``padded`` is false); the step runs them like any
-        request's, and their logits are not returned."""
+        own behind the entries of a batch that has no recording as it is (unless ``padded``
+        is false); the step runs them like any request's, and their logits are not
+        returned."""
         cache = runner.cache
         asked_for = len(entries)
         if device_tokens is not None and (device_tokens.dtype != torch.int32
                                           or device_tokens.numel() != asked_for):
             raise StepError(f"device_tokens must be int32 [{asked_for}]")
-        pads = runner.padding(asked_for) if padded and hasattr(runner, "padding") else []
-        if pads:
-            entries = list(entries) + [StepEntry(name, [0], [0]) for name in pads]
-        S = len(entries)
-        sc = self._scratch(S)
-        ptr = sc["ptr"]
-        known = cache.handles.known
-        reqs, toks = sc["reqs"], sc["toks"]
-        for i, e in enumerate(entries):
-            h = known(e.request)
-            if h is None:
-                raise StepError(f"request {e.request!r} was not admitted")
-            reqs[i] = h
-            if device_tokens is not None:
-                toks[i] = 0                      # a stand-in; the ids are copied on the device
-                continue
-            try:
-                toks[i] = e.tokens[0]
-            except (OverflowError, TypeError, ValueError):
-                raise StepError(f"token id {e.tokens[0]!r} of request {e.request!r} is outside "
-                                f"the vocabulary of {self._vocab}") from None
         lib = self._lib
-        rc = lib.za_decode_prepare(cache.native, S, ptr["reqs"], ptr["toks"], self._vocab,
-                                   self._max_position, ptr["extent"])
-        if rc == hostlib.OUT_OF_PAGES and pads:
-            # the requests' own rows may still fit once the padding rows' pages are back
-            runner.release_padding()
-            return self.run(runner, entries[:asked_for], device_tokens, more_to_come, padded=False)
+
+        def prepare(entries):
+            """The entries into the host library's arrays, their pages taken: the failure
+            code (0: none), the arrays and the shape's key."""
+            n = len(entries)
+            sc = self._scratch(n)
+            known = cache.handles.known
+            reqs, toks = sc["reqs"], sc["toks"]
+            for i, e in enumerate(entries):
+                h = known(e.request)
+                if h is None:
+                    raise StepError(f"request {e.request!r} was not admitted")
+                reqs[i] = h
+                if device_tokens is not None:
+                    toks[i] = 0                  # a stand-in; the ids are copied on the device
+                    continue
+                try:
+                    toks[i] = e.tokens[0]
+                except (OverflowError, TypeError, ValueError):
+                    raise StepError(f"token id {e.tokens[0]!r} of request {e.request!r} is outside "
+                                    f"the vocabulary of {self._vocab}") from None
+            rc = lib.za_decode_prepare(cache.native, n, sc["ptr"]["reqs"], sc["ptr"]["toks"],
+                                       self._vocab, self._max_position, sc["ptr"]["extent"])
+            widest, longest = int(sc["extent"][0]), int(sc["extent"][1])
+            return rc, sc, (n, _round_up(widest, PAGE_BUCKET), _round_up(longest, KEYS_BUCKET))
+
+        rc, sc, key = prepare(entries)
+        if rc == hostlib.OUT_OF_PAGES and padded and hasattr(runner, "release_padding") \
+                and runner.release_padding():
+            rc, sc, key = prepare(entries)       # with the pages that the runner's own rows held
         if rc:
             self._raise(rc, entries)
-        widest, longest = int(sc["extent"][0]), int(sc["extent"][1])
-        key = (S, _round_up(widest, PAGE_BUCKET), _round_up(longest, KEYS_BUCKET))
+        pads = []
+        recorded = self.entries.get(key)
+        if padded and hasattr(runner, "padding") \
+                and (recorded is None or recorded["graph"] is None):
+            # The batch as it is has no recording.  Filled up to the next size that
+            # recordings are kept for, it probably has; so that is what runs, until the batch
+            # has come as it is PROMOTE_AFTER times: then it is worth a recording of its own,
+            # which does not run the rows that fill it up.
+            sightings = self._unpadded_sightings.get(key, 0) + 1
+            if len(self._unpadded_sightings) > 4096:
+                self._unpadded_sightings.clear()
+            self._unpadded_sightings[key] = sightings
+            if sightings <= PROMOTE_AFTER:
+                pads = runner.padding(asked_for)
+            if pads:
+                filled = list(entries) + [StepEntry(name, [0], [0]) for name in pads]
+                rc, sc_filled, key_filled = prepare(filled)
+                if rc == hostlib.OUT_OF_PAGES:
+                    # (cannot be: the rows hold their pages; but then the requests' own rows,
+                    # whose pages are taken, run without them)
+                    runner.release_padding()
+                    pads = []
+                elif rc:
+                    self._raise(rc, filled)
+                else:
+                    entries, sc, key = filled, sc_filled, key_filled
+        S = len(entries)
+        ptr = sc["ptr"]
         slot = self.entries.get(key)
         if slot is not None:
             self.entries[key] = self.entries.pop(key)     # now the most recently used
