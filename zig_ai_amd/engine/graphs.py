@@ -155,7 +155,7 @@ class DecodeGraphs:
             self._raise(rc, entries)
         pads = []
         recorded = self.entries.get(key)
-        if padded and hasattr(runner, "padding") \
+        if padded and getattr(runner, "pad_decode", False) \
                 and (recorded is None or recorded["graph"] is None):
             # The batch as it is has no recording.  Filled up to the next size that
             # recordings are kept for, it probably has; so that is what runs, until the batch
