@@ -85,3 +85,13 @@ def test_where_the_library_adds_a_product_to_the_stream_itself():
     assert not ops.library_adds(2048, 2048, 4100)          # rows that do not start on 16 bytes
     for M in (17, 64, 512, 1024):
         assert not ops.library_adds(M, 2048, 8192)
+
+
+def test_the_batch_sizes_that_recordings_are_kept_for():
+    """A decode batch without a recording of its own is filled up to 1, 2, 4, 8, 16 requests
+    or, beyond, to a multiple of 8: never by more than 7 rows."""
+    from zig_ai_amd.engine.runner import ModelRunner
+    sizes = [ModelRunner.padded_size(n) for n in range(1, 70)]
+    assert sizes[:17] == [1, 2, 4, 4, 8, 8, 8, 8, 16, 16, 16, 16, 16, 16, 16, 16, 24]
+    assert all(0 <= s - n <= 7 for n, s in zip(range(1, 70), sizes))
+    assert all(s % 8 == 0 for s in sizes[16:]) and sizes[63] == 64 and sizes[64] == 72
