@@ -215,7 +215,7 @@ class DecodeGraphs:
         model = runner.model
         if device_tokens is not None:                     # a first step of this shape: on the host
             entries = [StepEntry(e.request, [t], [0])
-                       for e, t in zip(entries, device_tokens.view(-1).tolist())] + entries[asked_for:]
+                       for e, t in zip(entries, device_tokens.view(-1).tolist())] + list(entries[asked_for:])
         asked = [StepEntry(e.request, e.tokens, [0]) for e in entries]
         prepared = PreparedEntries(asked, cache, self._vocab)
         if slot is None:
