@@ -23,10 +23,13 @@
 // call of a shape times the first TUNE_CANDIDATES answers on the call's own operands and
 // keeps the fastest.  In a model every weight comes from memory: the timed runs take turns
 // over copies of the weight, so that a run's weights do not lie in a cache (timed warm, the
-// ranking is another one: a decode step of 64 rows got slower).  Shapes whose row counts fall into the same block (of
+// ranking is another one: a decode step of 64 rows got slower), and they are issued behind a
+// copy that keeps the GPU busy meanwhile, so that they run back to back and the kernels are
+// timed, not the host's calls.  Shapes whose row counts fall into the same block (of
 // TUNE_BUCKET rows from TUNE_BUCKET rows on, between two powers of two below) share the
-// choice, so a server that sees every batch size and portion length times a few dozen
-// shapes, some 10 ms each, not thousands.  (Naming the winner to the library by its index
+// choice where the heuristic names a block's winner for them too, and at most TUNE_PER_BLOCK
+// row counts of a block are timed themselves, so a server that sees every batch size and
+// portion length times some dozens of shapes, 10 to 60 ms each, not thousands.  (Naming the winner to the library by its index
 // for a new row count of a block, instead of looking for it among the heuristic's answers
 // for that row count, cost 300 ms at its first use.)  Which answer wins can differ from run
 // to run when two are close: callers that want the same bits run after run pass tune = 0
@@ -67,6 +70,7 @@ constexpr int TUNE_MIN_ROWS = 17;      // (up to 16 rows this package's own kern
 constexpr size_t TUNE_MIN_WEIGHT = (size_t)1 << 19;   // elements: a megabyte of bfloat16; below, nothing to gain
 constexpr int TUNE_BUCKET = 256;
 constexpr int TUNE_CANDIDATES = 24;
+constexpr size_t TUNE_PER_BLOCK = 4;     // row counts of one block that are timed themselves
 constexpr size_t TUNE_COPY_BYTES = (size_t)512 << 20;    // room for copies of a weight
 
 bool tune_log() {
@@ -85,7 +89,7 @@ int tune_block(int M) {
 }
 
 using Key = std::tuple<int, int, int, int, int, int, int>;   // device, M, N, K, output type, P, tune
-// device, block of rows, N, K, output type, P -> the library's index of the algorithm that won
+// device, block of rows, N, K, output type, P -> the library's indices of the algorithms that won
 using TunedKey = std::tuple<int, int, int, int, int, int>;
 
 // A product on given operands, with its kernel arguments made: issuing it again is one
@@ -110,7 +114,7 @@ size_t max_instances() {
 std::mutex g_lock;
 std::map<int, hipblasLtHandle_t> g_handles;
 std::map<Key, Plan> g_plans;
-std::map<TunedKey, int> g_tuned;
+std::map<TunedKey, std::vector<int>> g_tuned;   // a block's winners, the first timed first
 std::map<InstanceKey, std::unique_ptr<hipblaslt_ext::Gemm>> g_instances;
 const float kOne = 1.0f, kZero = 0.0f;
 thread_local std::string g_error;
@@ -196,8 +200,14 @@ bool make_plan(hipblasLtHandle_t handle, int M, int N, int K, int out_kind, int 
 // run's way and ranked the candidates differently from a loop over many weights.)  The
 // stream is waited for; this happens once per block of row counts.  A candidate that
 // fails is out.
-constexpr int TUNE_RUNS = 3;
+// The timed runs of a candidate are issued behind a copy that keeps the GPU busy for as
+// long as the host needs to issue them (some 8 us a call): they then run back to back, and
+// what is timed is the kernels, not the host (a product of a few microseconds, timed as
+// fast as the host could issue it, looked the same with every candidate: [1024, 1024] at
+// 24 to 64 rows 8.1 to 8.9 us for twenty of twenty-four, where the kernels take 5.6 to 11).
+constexpr int TUNE_RUNS = 8;
 constexpr int TUNE_COPIES = 7;
+constexpr size_t TUNE_BACKLOG_BYTES = (size_t)128 << 20;   // copied twice: some 100 us
 int fastest_candidate(hipblasLtHandle_t handle, const Plan& plan, const void* x, const void* w,
                       size_t weight_bytes, void* y, size_t added_bytes, void* workspace,
                       size_t workspace_bytes, hipStream_t stream) {
@@ -241,6 +251,19 @@ int fastest_candidate(hipblasLtHandle_t handle, const Plan& plan, const void* x,
     (void)hipStreamSynchronize(stream);
     return 0;
   }
+  char* backlog = nullptr;
+  if (hipMalloc((void**)&backlog, 2 * TUNE_BACKLOG_BYTES) != hipSuccess) {
+    (void)hipGetLastError();
+    backlog = nullptr;            // no room: the runs are timed as the host issues them
+  }
+  Release release_backlog{backlog};
+  auto keep_busy = [&]() {
+    if (!backlog) return;
+    (void)hipMemcpyAsync(backlog + TUNE_BACKLOG_BYTES, backlog, TUNE_BACKLOG_BYTES,
+                         hipMemcpyDeviceToDevice, stream);
+    (void)hipMemcpyAsync(backlog, backlog + TUNE_BACKLOG_BYTES, TUNE_BACKLOG_BYTES,
+                         hipMemcpyDeviceToDevice, stream);
+  };
   int turn = 0;
   auto next_weight = [&]() -> const void* {
     const int c = turn++ % (copies + 1);
@@ -263,7 +286,9 @@ int fastest_candidate(hipblasLtHandle_t handle, const Plan& plan, const void* x,
                              stream) == HIPBLAS_STATUS_SUCCESS;
     };
     float ms = 0.f;
-    bool fine = run() && hipEventRecord(t0, stream) == hipSuccess;
+    bool fine = run();
+    keep_busy();
+    fine = fine && hipEventRecord(t0, stream) == hipSuccess;
     for (int r = 0; r < TUNE_RUNS && fine; ++r) fine = run();
     fine = fine && hipEventRecord(t1, stream) == hipSuccess && hipEventSynchronize(t1) == hipSuccess &&
            hipEventElapsedTime(&ms, t0, t1) == hipSuccess;
@@ -334,16 +359,21 @@ ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int
       hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
       const bool recording = hipStreamIsCapturing(stream, &capturing) != hipSuccess ||
                              capturing != hipStreamCaptureStatusNone;
-      auto won = g_tuned.find(block);
-      if (won != g_tuned.end()) {
-        // a neighbouring row count has been timed: its winner, if it is among this
-        // shape's answers (else the first answer stays)
-        for (size_t i = 0; i < kept.candidates.size(); ++i)
-          if (hipblaslt_ext::getIndexFromAlgo(kept.candidates[i].algo) == won->second) {
+      // Neighbouring row counts that have been timed: the winner of one of them, the one
+      // timed last first, if it is among this shape's answers.  The heuristic does not
+      // give every row count of a block the same answers (64 rows on [1024, 1024] lack
+      // what wins at 48 rows, and the first answer takes twice as long): a row count
+      // without any of the block's winners is timed itself, up to TUNE_PER_BLOCK a block;
+      // beyond that the first answer stays.
+      std::vector<int>& winners = g_tuned[block];
+      bool found = false;
+      for (size_t wi = winners.size(); wi-- > 0 && !found;)
+        for (size_t i = 0; i < kept.candidates.size() && !found; ++i)
+          if (hipblaslt_ext::getIndexFromAlgo(kept.candidates[i].algo) == winners[wi]) {
             choose(i);
-            break;
+            found = true;
           }
-      } else if (!recording) {
+      if (!found && !recording && winners.size() < TUNE_PER_BLOCK) {
         const auto began = std::chrono::steady_clock::now();
         const int best = fastest_candidate(handle, kept, x, w, (size_t)N * K * sizeof(uint16_t), y,
                                            out_kind == OUT_ADDED ? (size_t)M * N * sizeof(float) : 0,
@@ -354,7 +384,7 @@ ZA_API int za_lt_matmul(const void* x, const void* w, void* y, int M, int N, int
                   kept.candidates.size(), M, N, K, P,
                   out_kind == OUT_ADDED ? "added to f32" : out_kind == OUT_F32 ? "f32" : "bf16", best,
                   std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - began).count());
-        g_tuned.emplace(block, hipblaslt_ext::getIndexFromAlgo(kept.algo));
+        winners.push_back(hipblaslt_ext::getIndexFromAlgo(kept.algo));
       }
       // (a shape first met while a stream is recorded keeps the first answer for good:
       // the same shape always runs the same kernel)
