@@ -53,10 +53,14 @@ def test_when_the_output_projection_merges_the_context_ranges():
 
 
 def test_where_the_kernel_for_17_to_64_rows_is_taken():
-    """The feed-forward's fused first product up to 32 rows, for widths whose K is spans of
-    512 (at least two) up to 4096; the mixer's closing product of such a step adds itself to
-    the stream when K is short and enough workgroups come of it."""
+    """The feed-forward's fused first product up to 32 rows, up to 64 on a stream no wider
+    than 1,024, for widths whose K is spans of 512 (at least two) up to 4096; the mixer's
+    closing product of such a step adds itself to the stream (through the library, see the
+    next test; this package's kernel, where the library has nothing, when K is short and
+    enough workgroups come of it)."""
     assert ops.rows64_swiglu_fusable(17, 2048) and ops.rows64_swiglu_fusable(32, 1024)
+    assert ops.rows64_swiglu_fusable(33, 1024) and ops.rows64_swiglu_fusable(64, 1024)
+    assert not ops.rows64_swiglu_fusable(65, 1024) and not ops.rows64_swiglu_fusable(48, 1536)
     assert ops.rows64_swiglu_fusable(20, 1536) and ops.rows64_swiglu_fusable(24, 4096)
     assert not ops.rows64_swiglu_fusable(16, 2048)      # the decode kernel's
     assert not ops.rows64_swiglu_fusable(33, 2048)      # measured no faster than the library's path
@@ -75,9 +79,10 @@ def test_where_the_kernel_for_17_to_64_rows_is_taken():
 
 
 def test_where_the_library_adds_a_product_to_the_stream_itself():
-    """Beyond the rows whose K the library gets in ranges, and only with a long K (the
-    feed-forward's closing product): elsewhere the product comes back and the next norm
-    adds it."""
+    """Many rows (beyond those whose K the library gets in ranges): only with a long K, the
+    feed-forward's closing product.  Few rows (17 to 64): only with a short K, a mixer's
+    closing product, and only where a feed-forward that runs its norm itself can follow on a
+    stream of that width.  Elsewhere the product comes back and the next norm adds it."""
     assert ops.library_adds(2048, 2048, 8192) and ops.library_adds(1025, 1024, 4608)
     assert ops.library_adds(4096, 2560, 10752)
     assert not ops.library_adds(2048, 2048, 2048)          # the mixers' closing products
@@ -85,6 +90,16 @@ def test_where_the_library_adds_a_product_to_the_stream_itself():
     assert not ops.library_adds(2048, 2048, 4100)          # rows that do not start on 16 bytes
     for M in (17, 64, 512, 1024):
         assert not ops.library_adds(M, 2048, 8192)
+    # few rows
+    for M in (17, 24, 32):
+        assert ops.library_adds(M, 2048, 2048) and ops.library_adds(M, 1024, 1024)
+        assert ops.library_adds(M, 2048, 1024)
+    for M in (33, 48, 64):
+        assert ops.library_adds(M, 1024, 1024) and not ops.library_adds(M, 2048, 2048)
+    for M in (16, 65, 128, 512):
+        assert not ops.library_adds(M, 1024, 1024)
+    assert not ops.library_adds(24, 1280, 1024)            # no fused feed-forward at that width
+    assert not ops.library_adds(24, 2048, 4096)            # a long K stays in ranges
 
 
 def test_the_batch_sizes_that_recordings_are_kept_for():

@@ -252,7 +252,12 @@ int fastest_candidate(hipblasLtHandle_t handle, const Plan& plan, const void* x,
     return 0;
   }
   char* backlog = nullptr;
-  if (hipMalloc((void**)&backlog, 2 * TUNE_BACKLOG_BYTES) != hipSuccess) {
+  static const bool host_paced = [] {       // (ZIG_AI_GEMM_TUNE_HOST_PACED=1: for comparisons)
+    const char* v = std::getenv("ZIG_AI_GEMM_TUNE_HOST_PACED");
+    return v && v[0] == '1';
+  }();
+  if (host_paced) {
+  } else if (hipMalloc((void**)&backlog, 2 * TUNE_BACKLOG_BYTES) != hipSuccess) {
     (void)hipGetLastError();
     backlog = nullptr;            // no room: the runs are timed as the host issues them
   }

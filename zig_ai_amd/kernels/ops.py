@@ -467,12 +467,27 @@ LIBRARY_ADDS_MIN_K = 4096
 
 def library_adds(M: int, N: int, K: int) -> bool:
     """Whether a product of this shape, asked to add itself to the 32-bit stream, does so
-    through the GEMM library (its beta = 1): beyond the rows whose K the library gets in
-    ranges, and with K long enough that reading and writing the stream in the product's
-    epilogue costs less than the next norm saves by not adding (measured at 2,048 rows:
-    [2048, 8192] 75 us against 79 into bfloat16, the norm after it 4.8 us against 7.7;
-    [2048, 2048] 25.5 against 22.2, which the norm does not win back)."""
-    return M > LIBRARY_SPLIT_ROWS and K >= LIBRARY_ADDS_MIN_K and K % 8 == 0
+    through the GEMM library (its beta = 1).
+
+    Many rows (beyond those whose K the library gets in ranges): with K long enough that
+    reading and writing the stream in the product's epilogue costs less than the next norm
+    saves by not adding (measured at 2,048 rows: [2048, 8192] 75 us against 79 into bfloat16,
+    the norm after it 4.8 us against 7.7; [2048, 2048] 25.5 against 22.2, which the norm does
+    not win back).
+
+    Few rows (a decode batch beyond this package's kernels for 16 rows): a mixer's closing
+    product, K short, where the stream of width N is then complete for a feed-forward whose
+    first product runs the norm itself (``rows64_swiglu_fusable``).  Added by the library,
+    [2048, 2048] takes 6.5 us at 24 rows and 7.8 at 32 (its partial sums 6.0 to 6.2, which the
+    norm kernel would have to add; this package's kernel adding with atomics 9.0 and 9.5),
+    [1024, 1024] 5.6 to 7.4 us at 24 to 64 rows, as its partial sums do.  A long K (the
+    feed-forward's own closing product) stays in ranges: [2048, 8192] at 24 rows 13.2 us
+    added against 10.4 in ranges."""
+    if K % 8:
+        return False
+    if M > LIBRARY_SPLIT_ROWS:
+        return K >= LIBRARY_ADDS_MIN_K
+    return M > LIBRARY_GEMM_ROWS and K < LIBRARY_ADDS_MIN_K and rows64_swiglu_fusable(M, N)
 
 
 def accumulate_plan(M: int, N: int, K: int, normed: bool) -> int:
@@ -545,25 +560,27 @@ def linear(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
         # workgroups would read rows of the stream while others add to them
         normed, x = None, x.materialise()
     splits = 1
-    if accumulate is not None and NORMED_ROWS_MAX_ROWS < M <= ROWS64_SWIGLU_ROWS and normed is None \
-            and bias is None and weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 \
-            and not force_tiled and rows64_add_splits(N, K):
-        # a step of 17 to 32 rows: the closing product of a mixer adds itself to the stream
-        # (so that the feed-forward's first product can run the norm, see above)
-        ks = rows64_add_splits(N, K)
-        linear_rows64(x, weight, ROWS64_ADD, accumulate, ks)
-        _note("linear", M=M, N=N, K=K, norm_in_product=False, added_to_stream=True,
-              partial_sums=1, out=accumulate.dtype, kernel="rows64")
-        return None
     if accumulate is not None and library_adds(M, N, K) and normed is None and bias is None \
             and weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and not force_tiled:
-        # many rows and a long K: the library adds its product to the stream itself
+        # the library adds its product to the stream itself (many rows and a long K, or
+        # the closing product of a mixer in a step of 17 to 64 rows)
         _need(weight, "weight", torch.bfloat16, (N, K))
         _need(accumulate, "accumulate", torch.float32, (M, N))
         if _library_matmul(x, weight, torch.float32, 1, tune, added_to=accumulate) is not None:
             _note("linear", M=M, N=N, K=K, norm_in_product=False, added_to_stream=True,
                   partial_sums=1, out=accumulate.dtype, kernel="library")
             return None
+    if accumulate is not None and NORMED_ROWS_MAX_ROWS < M <= ROWS64_SWIGLU_ROWS and normed is None \
+            and bias is None and weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 \
+            and not force_tiled and rows64_add_splits(N, K):
+        # a step of 17 to 32 rows for which the library has no algorithm: the closing product
+        # of a mixer adds itself to the stream with this package's kernel
+        # (so that the feed-forward's first product can run the norm, see above)
+        ks = rows64_add_splits(N, K)
+        linear_rows64(x, weight, ROWS64_ADD, accumulate, ks)
+        _note("linear", M=M, N=N, K=K, norm_in_product=False, added_to_stream=True,
+              partial_sums=1, out=accumulate.dtype, kernel="rows64")
+        return None
     if accumulate is not None:
         if weight.dtype == torch.bfloat16 and not force_tiled \
                 and (normed is not None or x.dtype == torch.bfloat16):
@@ -713,6 +730,7 @@ def rows64_takes(M: int, K: int, ksplit: int = 1) -> bool:
 # atomics (2048 x 2048: 8.6-9.4 us against the library's 6.6-8.8, without the stack of
 # partial sums that the norm kernel would have to add).
 ROWS64_SWIGLU_ROWS = 32
+ROWS64_NARROW_WIDTH = 1024
 ROWS64_ADD_MAX_K = 4096
 ROWS64_ADD_MIN_WORKGROUPS = 48
 
@@ -736,8 +754,13 @@ def rows64_add_splits(N: int, K: int) -> int:
 
 def rows64_swiglu_fusable(rows: int, width: int) -> bool:
     """Whether a step of ``rows`` rows takes the fused norm + gate|up + SwiGLU kernel for
-    17 to 64 rows (``linear_swiglu`` with a ``NormedRows``)."""
-    return (NORMED_ROWS_MAX_ROWS < rows <= ROWS64_SWIGLU_ROWS and width <= NORMED_ROWS_MAX_K
+    17 to 64 rows (``linear_swiglu`` with a ``NormedRows``): up to 32 rows, and up to 64
+    where the stream is narrow (every workgroup reads all of the step's rows: at width 1024
+    the fused form takes 13.7 us at 40 and 48 rows and 15.3 at 64, [9216, 1024], against
+    18.4 to 18.6 for norm, library product and SwiGLU kernel; at width 2048 it only equals
+    them at 64 rows)."""
+    most = ROWS64_MAX_ROWS if width <= ROWS64_NARROW_WIDTH else ROWS64_SWIGLU_ROWS
+    return (NORMED_ROWS_MAX_ROWS < rows <= most and width <= NORMED_ROWS_MAX_K
             and rows64_takes(rows, width))
 
 
