@@ -214,6 +214,28 @@ def test_decode_batches_filled_up_to_recorded_sizes():
         engine.runner.cache.check()
 
 
+def test_the_engine_warms_up_before_its_first_request():
+    """A bfloat16 engine whose projections are large enough to be timed runs one step of
+    every block of row counts up to its token budget when it is made, with a request of
+    its own that leaves nothing behind; a 32-bit engine, and one whose model takes the
+    library's first answer, have nothing to warm up."""
+    from zig_ai_amd.engine import DecoderModel, Engine
+    from tiny_configs import REAL_350M_2L
+    model = DecoderModel.from_random(REAL_350M_2L, seed=0, dtype="bfloat16", quick=True)
+    engine = Engine(model, page_size=16, num_pages=512, max_num_seqs=8, max_num_batched_tokens=600)
+    # 24 ... 64 (the sizes decode batches are filled up to), 128, 255, 256, 512
+    assert engine.warm_up_steps == 10
+    stats = engine.stats()
+    assert stats["requests"] == 0 and stats["slots_free"] == stats["slots"]
+    assert all(g["pages_free"] == g["pages"] for g in stats["groups"])
+    out = engine.generate([eu.random_tokens(40, REAL_350M_2L["vocab_size"], 3)], max_new_tokens=4,
+                          temperature=0.0, eos_token_id=-1)
+    assert len(out[0]) == 4
+    fixed = DecoderModel.from_random(REAL_350M_2L, seed=0, dtype="bfloat16", quick=True, reproducible=True)
+    assert Engine(fixed, page_size=16, num_pages=512, max_num_seqs=8).warm_up_steps == 0
+    assert Engine(folder_for(TINY_A, 0), dtype="float32", page_size=4, num_pages=64).warm_up_steps == 0
+
+
 def test_a_length_limit_beyond_the_models_own_is_refused():
     """``max_model_len`` above the model's ``max_position_embeddings`` would stop a step in
     the middle of a call and every request of the call with it: refused when the engine is

@@ -113,8 +113,8 @@ class Engine:
 
     def warm_up(self) -> int:
         """The GEMM library times its candidates for a shape at the shape's first call
-        (some 10 ms a shape, shared by the row counts of a block: 17-32, 33-64, 65-128,
-        129-255, then blocks of 256).  Run one step of every block up to
+        (10 to 60 ms a shape, shared by the row counts of a block, 17-32, 33-64, 65-128,
+        129-255, then blocks of 256, where the library names a block's winner for them too).  Run one step of every block up to
         ``max_num_batched_tokens`` now, with a request of its own that is released again,
         so that no request pays for it.  Nothing to do, and nothing done, for 32-bit
         models, models that take the library's first answer (``reproducible``,
@@ -132,7 +132,9 @@ class Engine:
                     for part in top for q in walk_parts(part) for v in vars(q).values())
         if not large:
             return 0
-        sizes = [m for m in (32, 64, 128, 255) if m <= self.max_num_batched_tokens]
+        # (up to 64 rows: the sizes that decode batches are filled up to; the heuristic does
+        # not name the same algorithms for every row count of a block)
+        sizes = [m for m in (24, 32, 40, 48, 56, 64, 128, 255) if m <= self.max_num_batched_tokens]
         sizes += list(range(256, self.max_num_batched_tokens + 1, 256))
         name = ("warm-up", id(self))
         steps = 0
