@@ -668,7 +668,7 @@ def test_a_decode_step_at_real_layer_sizes_runs_no_norm_kernel(monkeypatch):
         runner = ModelRunner(model, page_size=16, num_pages=8, num_slots=2, use_graphs=False)
         runner.admit("a")
         runner.admit("b")
-        for tokens, few in (([list(range(20)), list(range(30, 47))], False), ([[5], [6]], True),
+        for tokens, few in (([list(range(30)), list(range(30, 52))], False), ([[5], [6]], True),
                             ([list(range(50, 62)), list(range(70, 80))], "some")):
             calls.update(norm=0, stacks=0)
             runner.step([StepEntry("a", tokens[0], [len(tokens[0]) - 1]),

@@ -441,8 +441,8 @@ def test_gemm_bf16_decode_rows_added_to_the_stream(M, N, K):
     assert o.linear(x.to(dev()), w.to(dev()), b.to(dev()), accumulate=stream) is None
     assert rel_err(stream, stream0.double() + 2 * product) < F32_TOL
     # more rows than any kernel that adds takes, or 32-bit weights: the product comes back instead
-    many = rand((40, K), torch.bfloat16, 64).to(dev())
-    kept = torch.zeros((40, N), dtype=torch.float32, device=dev())
+    many = rand((70, K), torch.bfloat16, 64).to(dev())
+    kept = torch.zeros((70, N), dtype=torch.float32, device=dev())
     back = o.linear(many, w.to(dev()), accumulate=kept)
     assert back is not None and not kept.any()
     kept = torch.zeros((M, N), dtype=torch.float32, device=dev())
@@ -550,7 +550,7 @@ def test_rows64_refuses_what_it_does_not_take():
         o.linear_rows64(wide, rand((64, 8192), torch.bfloat16, 95).to(dev()))
     assert not o.rows64_swiglu_fusable(20, 8192) and not o.rows64_swiglu_fusable(16, 2048)
     assert o.rows64_swiglu_fusable(17, 2048) and o.rows64_swiglu_fusable(32, 1024)
-    assert not o.rows64_swiglu_fusable(33, 2048)
+    assert o.rows64_swiglu_fusable(48, 2048) and not o.rows64_swiglu_fusable(49, 2048)
     assert o.rows64_swiglu_fusable(64, 1024) and not o.rows64_swiglu_fusable(65, 1024)
 
 

@@ -573,7 +573,7 @@ def linear(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
     if accumulate is not None and NORMED_ROWS_MAX_ROWS < M <= ROWS64_SWIGLU_ROWS and normed is None \
             and bias is None and weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 \
             and not force_tiled and rows64_add_splits(N, K):
-        # a step of 17 to 32 rows for which the library has no algorithm: the closing product
+        # such a step for which the library has no algorithm: the closing product
         # of a mixer adds itself to the stream with this package's kernel
         # (so that the feed-forward's first product can run the norm, see above)
         ks = rows64_add_splits(N, K)
@@ -725,11 +725,11 @@ def rows64_takes(M: int, K: int, ksplit: int = 1) -> bool:
 # 17 to 32 rows against 24.8-25.8, 22.8-23.9 at 40-48 rows against 25.6, 25.5 at 64 rows
 # against 25.9; the plain forms lose (norm + in_proj 15.3 against 13.2 at 24 rows, w2 added
 # to the stream 12.7-14.5 against the library's 10.3).  So it serves the feed-forward's
-# first product up to ROWS64_SWIGLU_ROWS rows, which needs the stream complete before it,
+# first product up to ROWS64_SWIGLU_ROWS rows (64 on a narrow stream), which needs the stream complete before it,
 # and therefore the mixer's closing product of such a step, added to the stream with
 # atomics (2048 x 2048: 8.6-9.4 us against the library's 6.6-8.8, without the stack of
 # partial sums that the norm kernel would have to add).
-ROWS64_SWIGLU_ROWS = 32
+ROWS64_SWIGLU_ROWS = 48
 ROWS64_NARROW_WIDTH = 1024
 ROWS64_ADD_MAX_K = 4096
 ROWS64_ADD_MIN_WORKGROUPS = 48
@@ -754,11 +754,13 @@ def rows64_add_splits(N: int, K: int) -> int:
 
 def rows64_swiglu_fusable(rows: int, width: int) -> bool:
     """Whether a step of ``rows`` rows takes the fused norm + gate|up + SwiGLU kernel for
-    17 to 64 rows (``linear_swiglu`` with a ``NormedRows``): up to 32 rows, and up to 64
+    17 to 64 rows (``linear_swiglu`` with a ``NormedRows``): up to 48 rows, and up to 64
     where the stream is narrow (every workgroup reads all of the step's rows: at width 1024
     the fused form takes 13.7 us at 40 and 48 rows and 15.3 at 64, [9216, 1024], against
-    18.4 to 18.6 for norm, library product and SwiGLU kernel; at width 2048 it only equals
-    them at 64 rows)."""
+    18.4 to 18.6 for norm, library product and SwiGLU kernel; at width 2048, [16384, 2048],
+    22.8 to 23.9 at 40 to 48 rows against 25.6, and at 64 rows it only equals them: a decode
+    step of the 1.2B shape at batch 40 1.50 -> 1.47 ms, at batch 48 1.53 -> 1.49, at batch 64
+    1.562 -> 1.557)."""
     most = ROWS64_MAX_ROWS if width <= ROWS64_NARROW_WIDTH else ROWS64_SWIGLU_ROWS
     return (NORMED_ROWS_MAX_ROWS < rows <= most and width <= NORMED_ROWS_MAX_K
             and rows64_takes(rows, width))

@@ -47,7 +47,7 @@ class SwiGLU(FeedForward):
             # a decode batch: the gate is applied to the projection's accumulators
             a = ops.linear_swiglu(x, self.gate_up)
         elif bf16 and isinstance(x, ops.NormedRows) and ops.rows64_swiglu_fusable(*x.shape):
-            # 17 to 32 rows whose norm has not run: norm, product and gate in one kernel
+            # a step beyond 16 rows whose norm has not run: norm, product and gate in one kernel
             a = ops.linear_swiglu(x, self.gate_up)
         else:
             if isinstance(x, ops.NormedRows):

@@ -44,7 +44,7 @@ class RMSNorm(Norm):
     def deferred(self, residual: torch.Tensor, rows: Optional[torch.Tensor] = None,
                  swiglu: bool = False):
         """``swiglu``: the part that takes the rows starts with a fused gate|up product
-        (which also has a form for 17 to 32 rows)."""
+        (which also has a form for steps of 17 rows and more, see ``ops.rows64_swiglu_fusable``)."""
         # a decode batch in bfloat16: the projection that follows normalises the rows
         n = residual.shape[0] if rows is None else rows.numel()
         if self.runtime.dtype != torch.bfloat16:
