@@ -165,7 +165,12 @@ bool make_plan(hipblasLtHandle_t handle, int M, int N, int K, int out_kind, int 
   hipblasLtMatmulPreference_t pref = nullptr;
   if (!ok(hipblasLtMatmulPreferenceCreate(&pref), "PreferenceCreate", why)) return false;
   const uint64_t limit = workspace_bytes;
-  const int wanted = tune ? TUNE_CANDIDATES : 1;
+  static const int tune_candidates = [] {    // (ZIG_AI_GEMM_TUNE_CANDIDATES: for comparisons)
+    const char* v = std::getenv("ZIG_AI_GEMM_TUNE_CANDIDATES");
+    const int n = v ? std::atoi(v) : 0;
+    return n > 0 && n <= 512 ? n : TUNE_CANDIDATES;
+  }();
+  const int wanted = tune ? tune_candidates : 1;
   std::vector<hipblasLtMatmulHeuristicResult_t> found(wanted);
   int n_found = 0;
   bool good = ok(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES,
